@@ -1,0 +1,203 @@
+/*
+ * pshbm — C ABI of the HBM-resident sparse table that serves one pico-ps server shard.
+ *
+ * One `pshbm_table` holds what one shard of the reference's KVShardStorage holds
+ * (pico-ps/storage/KVShardStorage.h:844-952): uint64 key -> fp32 row of `dim` weights plus
+ * optimizer state, resident in device memory as an open-addressing hash table, and served by
+ * HIP kernels written for gfx950. Every entry point below stands where one of the reference's
+ * server-side operator loops stands; the citation on each says which.
+ *
+ * Conventions
+ *  - Every function returns an int32_t whose values are the reference's StatusCode values
+ *    (pico-ps/common/Status.h:15-29). No exception crosses this boundary.
+ *  - Pointers named `d_*` are device pointers on the table's GPU; all others are host pointers
+ *    (pageable or pinned) owned by the caller and valid for the duration of the call.
+ *  - `*_dev` entry points enqueue work on `stream` (a hipStream_t passed as void*; NULL = the
+ *    null stream) and return without waiting, except where noted. The caller orders calls
+ *    that touch one table: use one stream, or events between streams. Host-pointer entry
+ *    points are synchronous and may be called from several host threads: pulls without
+ *    insertion share the table, everything else takes it exclusively — the locking discipline
+ *    of pico-ps/operator/SparsePullOperator.h:188-192 and SparsePushOperator.h:220.
+ *  - A row is `dim` fp32 weights followed by its optimizer state: SUM and SGD none, ADAGRAD
+ *    `dim` accumulators, FTRL `dim` z then `dim` n. `pshbm_value_floats()` gives the total.
+ *  - Keys 0xFFFFFFFFFFFFFFFF and 0xFFFFFFFFFFFFFFFE are reserved (the reference's key types
+ *    reserve empty_key()/deleted_key() the same way: KVShardStorage.h:386-402,
+ *    SparsePullOperator.h:324); a batch that holds one is rejected with PSHBM_ERROR.
+ */
+#ifndef PSHBM_H
+#define PSHBM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* StatusCode values, pico-ps/common/Status.h:15-29 */
+#define PSHBM_OK 0
+#define PSHBM_INVALID_CONFIG 1
+#define PSHBM_INVALID_ID 2
+#define PSHBM_OUT_OF_MEMORY 3
+#define PSHBM_ERROR 10
+#define PSHBM_FATAL 11
+
+/* What store_push_value (SparsePushOperator.h:448) does with the aggregated gradient g of a key.
+ * The reference ships no optimizer (the hook is user code); SUM is its test operator
+ * (pico-ps/test/TestOps.h:112-117), the other three are defined by this library:
+ *   SUM      w += g
+ *   SGD      w -= lr*g
+ *   ADAGRAD  n += g*g;  w -= lr*g / sqrtf(n)            (n starts at init_acc, no epsilon)
+ *   FTRL     s = (sqrtf(n+g*g) - sqrtf(n))/alpha;  z += g - s*w;  n += g*g;
+ *            w = |z| <= l1 ? 0 : -(z - sign(z)*l1) / ((beta + sqrtf(n))/alpha + l2)
+ * all per element in fp32 with no fused multiply-add. A key inserted by a push starts from
+ * zero weights (and n = init_acc for ADAGRAD, z = n = 0 for FTRL) and then takes the same
+ * step with that batch's g, the way the test operator folds the first push into
+ * init_store_value (TestOps.h:91-96). */
+#define PSHBM_OPT_SUM 0
+#define PSHBM_OPT_SGD 1
+#define PSHBM_OPT_ADAGRAD 2
+#define PSHBM_OPT_FTRL 3
+
+typedef struct pshbm_config {
+    uint32_t struct_size;        /* sizeof(pshbm_config), for forward compatibility */
+    int32_t device;              /* HIP device ordinal */
+    uint32_t dim;                /* fp32 weights per key, >= 1 */
+    int32_t optimizer;           /* PSHBM_OPT_* */
+    float lr;                    /* SGD, ADAGRAD */
+    float init_acc;              /* ADAGRAD accumulator of a fresh key */
+    float alpha, beta, l1, l2;   /* FTRL */
+    uint64_t expected_max_items; /* capacity in keys; the table never rehashes. Mirrors
+                                    pool_hash_map.expected_max_items, KVShardStorage.h:879-897 */
+    float max_load_factor;       /* of the slot array; 0 selects 0.5 */
+    int32_t read_only;           /* pulls never insert: PullOperator.h:45-47 */
+    uint64_t max_batch;          /* workspace is pre-sized for batches of this many keys;
+                                    larger batches grow it (which allocates and synchronizes) */
+} pshbm_config;
+
+typedef struct pshbm_stats {
+    uint64_t size;               /* keys stored */
+    uint64_t capacity;           /* expected_max_items */
+    uint64_t slots;              /* slots in the hash array */
+    uint64_t memory_usage;       /* device bytes held by the table */
+    double load_factor;          /* size / slots */
+    uint64_t probe_hist[16];     /* keys whose bucket is h buckets past its home, h = 0..14; 15 = more */
+    uint64_t max_probe;          /* largest such distance */
+} pshbm_stats;
+
+typedef struct pshbm_table pshbm_table;
+
+/* pull flags */
+#define PSHBM_PULL_INSERT_ON_MISS 1u /* init_store_value returns true: SparsePullOperator.h:217-225 */
+/* push flags */
+#define PSHBM_PUSH_NO_INSERT 1u      /* init_store_value returns false, item dropped: SparsePushOperator.h:250-251 */
+#define PSHBM_PUSH_ASSUME_UNIQUE 2u  /* caller guarantees distinct keys (a client batch after
+                                        SparsePushOperator.h:134-141): skips the aggregation */
+/* load flags */
+#define PSHBM_LOAD_UNIQUE 1u         /* a key already present is an error: LoadOperator.h:194,210 */
+
+/* Creates the storage of one shard. Replaces ShardStorageOperator::create_storage
+ * (pico-ps/operator/StorageOperator.h:106-109) -> PoolHashMapShardStorage::create_shard
+ * (pico-ps/storage/KVShardStorage.h:910-925). INVALID_CONFIG on a bad config, OUT_OF_MEMORY when
+ * the device cannot hold the table, ERROR when no HIP device answers. */
+int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out);
+
+/* Releases the table: the storage destructor (KVShardStorage.h:866-873 erase of each shard). */
+int32_t pshbm_destroy(pshbm_table* t);
+
+/* Message of the last failure on this table (owned by the table, valid until the next call). */
+const char* pshbm_last_error(const pshbm_table* t);
+
+/* Floats per stored value (weights + optimizer state) for a dim and optimizer; 0 if invalid. */
+uint32_t pshbm_value_floats(uint32_t dim, int32_t optimizer);
+
+/* Sparse pull. Replaces the per-key loop of SparseTablePullOperator::apply_request
+ * (pico-ps/operator/SparsePullOperator.h:208-228): for key i, out_rows[i*dim .. +dim) is the
+ * stored weights (fetch_pull_value) or zeros on a miss (init_store_value's value_type(), :307-310);
+ * hit[i] (may be NULL) is lock_find's return against the table as it was when the call began.
+ * With PSHBM_PULL_INSERT_ON_MISS (ignored on a read_only table) each distinct missing key is
+ * inserted with a fresh row. OUT_OF_MEMORY when the insertions do not fit (:245-253): then no key
+ * of the batch has been inserted and out_rows/hit are unspecified. */
+int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_rows, uint8_t* hit,
+                   uint32_t flags);
+int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* d_out_rows,
+                       uint8_t* d_hit, uint32_t flags, void* stream);
+
+/* Sparse push of one client batch. Replaces the duplicate aggregation of
+ * SparseTablePushOperator::generate_request_data (pico-ps/operator/SparsePushOperator.h:134-141:
+ * gradients of equal keys are summed) followed by the per-item loop of apply_async_push_request
+ * (:245-268: a missing key is inserted via init_store_value, a present key takes
+ * store_push_value = one optimizer step with the summed gradient). grads is n x dim.
+ * OUT_OF_MEMORY when the new keys do not fit: then the table is unchanged (the reference parks
+ * such items in the shard's overflow vector, :257-259; a fixed-capacity table refuses the batch).
+ * The *_dev form synchronizes only when the table is within n keys of its capacity. */
+int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, size_t n,
+                   uint32_t flags);
+int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
+                       uint32_t flags, void* stream);
+
+/* Same, from the wire layout of a push block: n records of std::pair<KEY, PUSH_VALUE> laid out
+ * back to back (SparsePushOperator.h:176-177,246-247), i.e. a uint64 key then dim floats, every
+ * `stride` bytes (stride >= 8 + 4*dim, a multiple of 4). */
+int32_t pshbm_push_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride, uint32_t flags);
+
+/* Sync push: queues a block without touching the table. Replaces apply_sync_push_request
+ * (SparsePushOperator.h:299-316, the per-shard MPSC queue of KVShardStorage.h:677-726). */
+int32_t pshbm_queue(pshbm_table* t, const uint64_t* keys, const float* grads, size_t n);
+int32_t pshbm_queue_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
+                        void* stream);
+/* Number of keys queued and not yet stored. */
+int32_t pshbm_queued(pshbm_table* t, uint64_t* n);
+
+/* Store: merges every queued block (merge_push_value sums equal keys, SparsePushOperator.h:377-386)
+ * and applies each distinct key once (:388-409). Replaces apply_store_request's work after its
+ * early acknowledgement. The queue is empty afterwards, also on failure. */
+int32_t pshbm_store(pshbm_table* t, uint32_t flags);
+int32_t pshbm_store_dev(pshbm_table* t, uint32_t flags, void* stream);
+
+/* Upsert of whole values: ht[key] = value for every item (safe_set, KVShardStorage.h:804-814).
+ * Replaces DirectPushOperator::apply_async_push_request (SparsePushOperator.h:520-574), where
+ * Load-with-rehash and the reshard shuffle land. values is n x pshbm_value_floats(); keys of one
+ * call must be distinct. OUT_OF_MEMORY (:568-573) leaves the table unchanged. */
+int32_t pshbm_set(pshbm_table* t, const uint64_t* keys, const float* values, size_t n);
+int32_t pshbm_set_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_values, size_t n,
+                      void* stream);
+
+/* Bulk load of n records {uint64 key; float value[pshbm_value_floats()]} from host memory,
+ * streamed to the device through pinned staging on a side stream and upserted block by block.
+ * Replaces BaseKVTextFileLoadOperator::restore (pico-ps/operator/LoadOperator.h:164-213) once the
+ * file is decoded; with PSHBM_LOAD_UNIQUE a key that is already present (or repeated) fails with
+ * PSHBM_ERROR the way restore aborts on it (:194,210), and the records loaded before the failing
+ * block stay. */
+int32_t pshbm_load(pshbm_table* t, const void* records, size_t n, uint32_t flags);
+
+/* Bulk dump of every (key, value) as the same records, in row-slab order, through the same
+ * staging. Replaces the shard walk of BaseKVTextFileDumpOperator::apply_request
+ * (pico-ps/operator/DumpOperator.h:163-174). *n_out = records written; ERROR if capacity_records
+ * is smaller than the table. The order is unspecified as the reference's is (map iteration order). */
+int32_t pshbm_dump(pshbm_table* t, void* records, size_t capacity_records, size_t* n_out);
+
+/* Resumable slice [offset, offset+batch) of that same record sequence. Replaces
+ * KVShardIterator::iterate_batch_as_binary_archive (pico-ps/storage/KVShardStorage.h:64-87).
+ * *n_out < batch marks the end. */
+int32_t pshbm_iterate(pshbm_table* t, size_t offset, size_t batch, void* records, size_t* n_out);
+
+/* Empties the table and keeps its memory: KVShardStorage.h:902-908. */
+int32_t pshbm_clear(pshbm_table* t);
+
+/* shard_size (KVShardStorage.h:927-935) and shard_memory_usage (:937-946). */
+int32_t pshbm_size(pshbm_table* t, uint64_t* n);
+int32_t pshbm_memory_usage(pshbm_table* t, uint64_t* bytes);
+
+/* Load factor and probe-distance histogram; the counterpart of StorageStatisticInfo
+ * (pico-ps/operator/StorageOperator.h:27-38,123-141). */
+int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out);
+
+/* Pinned host memory for request/response buffers of the host-pointer entry points. */
+int32_t pshbm_host_alloc(void** p, size_t bytes);
+int32_t pshbm_host_free(void* p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PSHBM_H */

@@ -1,0 +1,271 @@
+"""ctypes binding of libpshbm.so, the HBM-resident sparse table behind the Pull / Push / Load /
+Dump operators of one pico-ps server shard.
+
+The directory name contains a hyphen, so load it with
+``importlib.import_module("parameter-server_amd")``.
+
+There is no CPU fallback: if the library has not been built, or no HIP device answers, the calls
+raise.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libpshbm.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+OK, INVALID_CONFIG, INVALID_ID, OUT_OF_MEMORY, ERROR, FATAL = 0, 1, 2, 3, 10, 11
+OPT_SUM, OPT_SGD, OPT_ADAGRAD, OPT_FTRL = 0, 1, 2, 3
+PULL_INSERT_ON_MISS = 1
+PUSH_NO_INSERT = 1
+PUSH_ASSUME_UNIQUE = 2
+LOAD_UNIQUE = 1
+
+# every symbol include/pshbm.h declares
+SYMBOLS = [
+    "pshbm_create", "pshbm_destroy", "pshbm_last_error", "pshbm_value_floats",
+    "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
+    "pshbm_queue", "pshbm_queue_dev", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
+    "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
+    "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
+    "pshbm_host_alloc", "pshbm_host_free",
+]
+
+
+class Config(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("device", C.c_int32),
+        ("dim", C.c_uint32),
+        ("optimizer", C.c_int32),
+        ("lr", C.c_float),
+        ("init_acc", C.c_float),
+        ("alpha", C.c_float),
+        ("beta", C.c_float),
+        ("l1", C.c_float),
+        ("l2", C.c_float),
+        ("expected_max_items", C.c_uint64),
+        ("max_load_factor", C.c_float),
+        ("read_only", C.c_int32),
+        ("max_batch", C.c_uint64),
+    ]
+
+
+class Stats(C.Structure):
+    _fields_ = [
+        ("size", C.c_uint64),
+        ("capacity", C.c_uint64),
+        ("slots", C.c_uint64),
+        ("memory_usage", C.c_uint64),
+        ("load_factor", C.c_double),
+        ("probe_hist", C.c_uint64 * 16),
+        ("max_probe", C.c_uint64),
+    ]
+
+
+class PshbmError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"pshbm status {status}: {message}")
+        self.status = status
+
+
+def build(verbose=False):
+    """Compiles the HIP sources for gfx950 into libpshbm.so (hipcc; works without a GPU)."""
+    r = subprocess.run(["make", "-C", CSRC, "-B", "-j4"], capture_output=True, text=True)
+    if verbose or r.returncode != 0:
+        print(r.stdout[-4000:])
+        print(r.stderr[-4000:])
+    if r.returncode != 0:
+        raise RuntimeError("building libpshbm.so failed")
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                f"{LIB_PATH} is missing: build it with __graft_entry__.build() "
+                f"(make -C {CSRC}); there is no CPU fallback")
+        L = C.CDLL(LIB_PATH)
+        vp, sz, u32, i32 = C.c_void_p, C.c_size_t, C.c_uint32, C.c_int32
+        L.pshbm_create.argtypes = [C.POINTER(Config), C.POINTER(vp)]
+        L.pshbm_destroy.argtypes = [vp]
+        L.pshbm_last_error.argtypes = [vp]
+        L.pshbm_last_error.restype = C.c_char_p
+        L.pshbm_value_floats.argtypes = [u32, i32]
+        L.pshbm_value_floats.restype = u32
+        L.pshbm_pull.argtypes = [vp, vp, sz, vp, vp, u32]
+        L.pshbm_pull_dev.argtypes = [vp, vp, sz, vp, vp, u32, vp]
+        L.pshbm_push.argtypes = [vp, vp, vp, sz, u32]
+        L.pshbm_push_dev.argtypes = [vp, vp, vp, sz, u32, vp]
+        L.pshbm_push_pairs.argtypes = [vp, vp, sz, sz, u32]
+        L.pshbm_queue.argtypes = [vp, vp, vp, sz]
+        L.pshbm_queue_dev.argtypes = [vp, vp, vp, sz, vp]
+        L.pshbm_queued.argtypes = [vp, C.POINTER(C.c_uint64)]
+        L.pshbm_store.argtypes = [vp, u32]
+        L.pshbm_store_dev.argtypes = [vp, u32, vp]
+        L.pshbm_set.argtypes = [vp, vp, vp, sz]
+        L.pshbm_set_dev.argtypes = [vp, vp, vp, sz, vp]
+        L.pshbm_load.argtypes = [vp, vp, sz, u32]
+        L.pshbm_dump.argtypes = [vp, vp, sz, C.POINTER(sz)]
+        L.pshbm_iterate.argtypes = [vp, sz, sz, vp, C.POINTER(sz)]
+        L.pshbm_clear.argtypes = [vp]
+        L.pshbm_size.argtypes = [vp, C.POINTER(C.c_uint64)]
+        L.pshbm_memory_usage.argtypes = [vp, C.POINTER(C.c_uint64)]
+        L.pshbm_get_stats.argtypes = [vp, C.POINTER(Stats)]
+        L.pshbm_host_alloc.argtypes = [C.POINTER(vp), sz]
+        L.pshbm_host_free.argtypes = [vp]
+        for name in SYMBOLS:
+            if getattr(L, name).restype is C.c_int:
+                getattr(L, name).restype = i32
+        _lib = L
+    return _lib
+
+
+def value_floats(dim, optimizer):
+    return lib().pshbm_value_floats(dim, optimizer)
+
+
+def record_dtype(vf):
+    """Layout of one Load/Dump record: uint64 key then the value's floats, packed."""
+    return np.dtype([("key", "<u8"), ("value", "<f4", (vf,))])
+
+
+def _u64(a):
+    return np.ascontiguousarray(a, dtype=np.uint64)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+class Table:
+    """One shard's storage in HBM. Methods return the status code (and outputs); they raise only
+    on misuse. Host-array methods are synchronous; the ``*_dev`` methods take raw device pointers
+    and a hipStream_t value and enqueue."""
+
+    def __init__(self, dim, optimizer=OPT_SUM, lr=0.0, init_acc=0.0, alpha=0.0, beta=0.0, l1=0.0,
+                 l2=0.0, capacity=1 << 20, max_load_factor=0.0, read_only=False, max_batch=0,
+                 device=0):
+        self.dim = dim
+        self.optimizer = optimizer
+        self._h = C.c_void_p()
+        cfg = Config(C.sizeof(Config), device, dim, optimizer, lr, init_acc, alpha, beta, l1, l2,
+                     capacity, max_load_factor, int(read_only), max_batch)
+        st = lib().pshbm_create(C.byref(cfg), C.byref(self._h))
+        if st != OK:
+            raise PshbmError(st, (lib().pshbm_last_error(None) or b"").decode())
+        self.value_floats = value_floats(dim, optimizer)
+
+    # -- lifetime
+    def close(self):
+        if self._h:
+            lib().pshbm_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def last_error(self):
+        return (lib().pshbm_last_error(self._h) or b"").decode()
+
+    # -- host-array entry points
+    def pull(self, keys, flags=0):
+        k = _u64(keys)
+        out = np.empty((k.size, self.dim), dtype=np.float32)
+        hit = np.empty(k.size, dtype=np.uint8)
+        st = lib().pshbm_pull(self._h, k.ctypes.data, k.size, out.ctypes.data, hit.ctypes.data, flags)
+        return st, out, hit
+
+    def push(self, keys, grads, flags=0):
+        k, g = _u64(keys), _f32(grads)
+        assert g.size == k.size * self.dim
+        return lib().pshbm_push(self._h, k.ctypes.data, g.ctypes.data, k.size, flags)
+
+    def push_pairs(self, pairs, flags=0):
+        """pairs: structured array {key u8, value f4[dim]} (the wire layout of a push block)."""
+        p = np.ascontiguousarray(pairs)
+        return lib().pshbm_push_pairs(self._h, p.ctypes.data, p.size, p.dtype.itemsize, flags)
+
+    def queue(self, keys, grads):
+        k, g = _u64(keys), _f32(grads)
+        assert g.size == k.size * self.dim
+        return lib().pshbm_queue(self._h, k.ctypes.data, g.ctypes.data, k.size)
+
+    def queued(self):
+        n = C.c_uint64()
+        lib().pshbm_queued(self._h, C.byref(n))
+        return n.value
+
+    def store(self, flags=0):
+        return lib().pshbm_store(self._h, flags)
+
+    def set(self, keys, values):
+        k, v = _u64(keys), _f32(values)
+        assert v.size == k.size * self.value_floats
+        return lib().pshbm_set(self._h, k.ctypes.data, v.ctypes.data, k.size)
+
+    def load(self, records, flags=0):
+        r = np.ascontiguousarray(records, dtype=record_dtype(self.value_floats))
+        return lib().pshbm_load(self._h, r.ctypes.data, r.size, flags)
+
+    def dump(self):
+        n = self.size()
+        rec = np.empty(n, dtype=record_dtype(self.value_floats))
+        got = C.c_size_t()
+        st = lib().pshbm_dump(self._h, rec.ctypes.data, n, C.byref(got))
+        return st, rec[: got.value]
+
+    def iterate(self, offset, batch):
+        rec = np.empty(batch, dtype=record_dtype(self.value_floats))
+        got = C.c_size_t()
+        st = lib().pshbm_iterate(self._h, offset, batch, rec.ctypes.data, C.byref(got))
+        return st, rec[: got.value]
+
+    def clear(self):
+        return lib().pshbm_clear(self._h)
+
+    def size(self):
+        n = C.c_uint64()
+        st = lib().pshbm_size(self._h, C.byref(n))
+        if st != OK:
+            raise PshbmError(st, self.last_error())
+        return n.value
+
+    def memory_usage(self):
+        n = C.c_uint64()
+        lib().pshbm_memory_usage(self._h, C.byref(n))
+        return n.value
+
+    def stats(self):
+        s = Stats()
+        st = lib().pshbm_get_stats(self._h, C.byref(s))
+        if st != OK:
+            raise PshbmError(st, self.last_error())
+        return s
+
+    # -- device-pointer entry points (pointers and stream as integers)
+    def pull_dev(self, d_keys, n, d_out, d_hit=None, flags=0, stream=0):
+        return lib().pshbm_pull_dev(self._h, d_keys, n, d_out, d_hit, flags, stream)
+
+    def push_dev(self, d_keys, d_grads, n, flags=0, stream=0):
+        return lib().pshbm_push_dev(self._h, d_keys, d_grads, n, flags, stream)
+
+    def queue_dev(self, d_keys, d_grads, n, stream=0):
+        return lib().pshbm_queue_dev(self._h, d_keys, d_grads, n, stream)
+
+    def store_dev(self, flags=0, stream=0):
+        return lib().pshbm_store_dev(self._h, flags, stream)
+
+    def set_dev(self, d_keys, d_values, n, stream=0):
+        return lib().pshbm_set_dev(self._h, d_keys, d_values, n, stream)

@@ -1,0 +1,827 @@
+// C ABI of the HBM sparse table (include/pshbm.h): host-side state, capacity accounting, stream
+// ordering and staging around the kernels of kernels.hip / sort.hip.
+#include "../../include/pshbm.h"
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <shared_mutex>
+#include <string>
+
+#include "table.h"
+
+using namespace pshbm;
+
+namespace {
+
+constexpr size_t BULK_CHUNK_BYTES = 32u << 20;  // staging granule of load / dump
+constexpr uint32_t MAX_DIM = 16384;
+
+inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+struct DevBuf {
+    void* p = nullptr;
+    size_t bytes = 0;
+};
+
+}  // namespace
+
+struct pshbm_table {
+    pshbm_config cfg{};
+    TableDev d{};
+    int device = 0;
+    uint64_t nbuckets = 0;
+    uint32_t slot_bits = 0;
+    size_t slots_bytes = 0, rows_bytes = 0, keys_bytes = 0;
+
+    uint32_t* h_counters = nullptr;  // pinned, CNT_WORDS
+    unsigned long long* d_hist = nullptr;
+    unsigned long long* h_hist = nullptr;  // pinned, 17
+
+    // per-batch workspace of the mutating paths
+    size_t ws_cap = 0;
+    DevBuf ws_slot, ws_idx, ws_sslot, ws_sidx, ws_sort, ws_hdr, ws_pval;
+
+    // staging of the host-pointer entry points
+    std::mutex st_mu;
+    DevBuf st_keys, st_vals, st_out, st_hit, st_raw;
+
+    // sync-push queue
+    DevBuf q_keys, q_grads;
+    size_t q_n = 0;
+
+    // bulk staging (load / dump)
+    void* pin[2] = {nullptr, nullptr};
+    void* dbuf[2] = {nullptr, nullptr};
+    hipEvent_t ev_copy[2]{}, ev_done[2]{};
+
+    hipStream_t stream = nullptr, side = nullptr;
+    hipEvent_t order_ev{};
+    hipStream_t last_stream = nullptr;
+    bool has_last = false;
+
+    std::shared_mutex mu;
+    uint64_t size_bound = 0;  // upper bound of the rows handed out
+    std::string err;
+};
+
+namespace {
+
+struct DeviceGuard {
+    int prev = -1;
+    explicit DeviceGuard(int dev) {
+        if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+        if (prev != dev) (void)hipSetDevice(dev);
+    }
+    ~DeviceGuard() {
+        if (prev >= 0) (void)hipSetDevice(prev);
+    }
+};
+
+int32_t fail(pshbm_table* t, int32_t code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (t) t->err = buf;
+    return code;
+}
+
+int32_t hip_fail(pshbm_table* t, hipError_t e, const char* what) {
+    int32_t code = (e == hipErrorOutOfMemory) ? PSHBM_OUT_OF_MEMORY : PSHBM_ERROR;
+    return fail(t, code, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(t, expr)                                              \
+    do {                                                              \
+        hipError_t e__ = (expr);                                      \
+        if (e__ != hipSuccess) return hip_fail((t), e__, #expr);      \
+    } while (0)
+
+#define ST_TRY(expr)                          \
+    do {                                      \
+        int32_t s__ = (expr);                 \
+        if (s__ != PSHBM_OK) return s__;      \
+    } while (0)
+
+int32_t ensure(pshbm_table* t, DevBuf& b, size_t bytes) {
+    if (bytes <= b.bytes) return PSHBM_OK;
+    if (b.p) {
+        HIP_TRY(t, hipDeviceSynchronize());
+        HIP_TRY(t, hipFree(b.p));
+        b.p = nullptr;
+        b.bytes = 0;
+    }
+    size_t want = round_up(bytes + bytes / 4, 256);
+    HIP_TRY(t, hipMalloc(&b.p, want));
+    b.bytes = want;
+    return PSHBM_OK;
+}
+
+// scratch of the mutating paths for a batch of n keys
+int32_t ensure_workspace(pshbm_table* t, size_t n) {
+    if (n <= t->ws_cap) return PSHBM_OK;
+    size_t cap = std::max<size_t>(n, 1024);
+    ST_TRY(ensure(t, t->ws_slot, cap * 4));
+    ST_TRY(ensure(t, t->ws_idx, cap * 4));
+    ST_TRY(ensure(t, t->ws_sslot, cap * 4));
+    ST_TRY(ensure(t, t->ws_sidx, cap * 4));
+    ST_TRY(ensure(t, t->ws_sort, sort_pairs_temp_bytes(cap)));
+    // partial sums of the segmented reduce: size for the scalar layout, which has more chunks
+    SegGeom g1 = seg_geometry(t->d.dim, 1, cap);
+    SegGeom g4 = seg_geometry(t->d.dim, (t->d.dim % 4 == 0) ? 4 : 1, cap);
+    size_t chunks = std::max(g1.n_chunks, g4.n_chunks);
+    ST_TRY(ensure(t, t->ws_hdr, chunks * sizeof(uint4)));
+    ST_TRY(ensure(t, t->ws_pval, chunks * 2 * (size_t)t->d.dim * 4));
+    t->ws_cap = cap;
+    return PSHBM_OK;
+}
+
+// Orders this call after the table's previous call when that ran on another stream.
+int32_t begin_op(pshbm_table* t, hipStream_t s) {
+    if (t->has_last && t->last_stream != s) {
+        HIP_TRY(t, hipEventRecord(t->order_ev, t->last_stream));
+        HIP_TRY(t, hipStreamWaitEvent(s, t->order_ev, 0));
+    }
+    t->last_stream = s;
+    t->has_last = true;
+    return PSHBM_OK;
+}
+
+int32_t read_counters(pshbm_table* t, hipStream_t s) {
+    HIP_TRY(t, hipMemcpyAsync(t->h_counters, t->d.counters, CNT_WORDS * 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    return PSHBM_OK;
+}
+
+// Capacity accounting without a device round trip in the common case: `size_bound` is an upper
+// bound of the rows handed out (every inserting batch of n keys adds at most n). Only when the
+// bound would pass the capacity is the exact count read back; if even that leaves less than n
+// free rows the batch runs in checked mode (`*checked`), where the caller inspects the overflow
+// flag after the claim and rolls the batch back when it is set.
+int32_t reserve_rows(pshbm_table* t, size_t n, hipStream_t s, bool* checked, uint32_t* rows_before) {
+    *checked = false;
+    if (t->size_bound + n <= t->d.max_rows) {
+        t->size_bound += n;
+        return PSHBM_OK;
+    }
+    ST_TRY(read_counters(t, s));
+    t->size_bound = t->h_counters[CNT_ROWS];
+    if (t->size_bound + n <= t->d.max_rows) {
+        t->size_bound += n;
+        return PSHBM_OK;
+    }
+    *checked = true;
+    *rows_before = t->h_counters[CNT_ROWS];
+    return PSHBM_OK;
+}
+
+// After a claim in checked mode: OUT_OF_MEMORY (and the claim undone) if it did not fit.
+int32_t settle_rows(pshbm_table* t, const uint32_t* slot_idx, size_t n, hipStream_t s,
+                    uint32_t rows_before) {
+    ST_TRY(read_counters(t, s));
+    if (t->h_counters[CNT_OVERFLOW] || t->h_counters[CNT_ROWS] > t->d.max_rows) {
+        HIP_TRY(t, launch_rollback(t->d, slot_idx, n, rows_before, s));
+        HIP_TRY(t, hipStreamSynchronize(s));
+        t->size_bound = rows_before;
+        return fail(t, PSHBM_OUT_OF_MEMORY,
+                    "table full: %u keys stored, capacity %u, batch of %zu does not fit",
+                    rows_before, t->d.max_rows, n);
+    }
+    t->size_bound = t->h_counters[CNT_ROWS];
+    return PSHBM_OK;
+}
+
+bool has_reserved_key(const uint64_t* keys, size_t n) {
+    uint64_t bad = 0;
+    for (size_t i = 0; i < n; ++i) bad |= (uint64_t)(keys[i] >= KEY_DELETED);
+    return bad != 0;
+}
+
+int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
+                    uint32_t flags, hipStream_t s) {
+    if (n == 0) return PSHBM_OK;
+    ST_TRY(begin_op(t, s));
+    ST_TRY(ensure_workspace(t, n));
+    const bool insert = !(flags & PSHBM_PUSH_NO_INSERT);
+    const bool unique = (flags & PSHBM_PUSH_ASSUME_UNIQUE) != 0;
+    bool checked = false;
+    uint32_t rows_before = 0;
+    if (insert) ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
+    uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
+    uint32_t* idx = static_cast<uint32_t*>(t->ws_idx.p);
+    HIP_TRY(t, launch_locate(t->d, d_keys, n, slot, unique ? nullptr : idx, insert, true, false, s));
+    if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
+    if (unique) {
+        HIP_TRY(t, launch_update_unique(t->d, slot, n, d_grads, s));
+    } else {
+        uint32_t* sslot = static_cast<uint32_t*>(t->ws_sslot.p);
+        uint32_t* sidx = static_cast<uint32_t*>(t->ws_sidx.p);
+        HIP_TRY(t, sort_pairs(t->ws_sort.p, t->ws_sort.bytes, slot, sslot, idx, sidx, n,
+                              t->slot_bits + 1, s));
+        HIP_TRY(t, launch_segreduce_update(t->d, sslot, sidx, n, d_grads,
+                                           static_cast<uint4*>(t->ws_hdr.p),
+                                           static_cast<float*>(t->ws_pval.p), s));
+    }
+    return PSHBM_OK;
+}
+
+int32_t set_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_values, size_t n,
+                   bool count_dups, hipStream_t s) {
+    if (n == 0) return PSHBM_OK;
+    ST_TRY(begin_op(t, s));
+    ST_TRY(ensure_workspace(t, n));
+    bool checked = false;
+    uint32_t rows_before = 0;
+    ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
+    uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
+    HIP_TRY(t, launch_locate(t->d, d_keys, n, slot, nullptr, true, false, count_dups, s));
+    if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
+    HIP_TRY(t, launch_write_values(t->d, slot, n, d_values, s));
+    return PSHBM_OK;
+}
+
+int32_t ensure_bulk(pshbm_table* t) {
+    if (t->pin[0]) return PSHBM_OK;
+    for (int k = 0; k < 2; ++k) {
+        HIP_TRY(t, hipHostMalloc(&t->pin[k], BULK_CHUNK_BYTES, hipHostMallocDefault));
+        HIP_TRY(t, hipMalloc(&t->dbuf[k], BULK_CHUNK_BYTES));
+        HIP_TRY(t, hipEventCreateWithFlags(&t->ev_copy[k], hipEventDisableTiming));
+        HIP_TRY(t, hipEventCreateWithFlags(&t->ev_done[k], hipEventDisableTiming));
+    }
+    return PSHBM_OK;
+}
+
+void destroy_impl(pshbm_table* t) {
+    DeviceGuard g(t->device);
+    (void)hipDeviceSynchronize();
+    DevBuf* bufs[] = {&t->ws_slot, &t->ws_idx,  &t->ws_sslot, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
+                      &t->ws_pval, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
+                      &t->q_keys,  &t->q_grads};
+    for (DevBuf* b : bufs)
+        if (b->p) (void)hipFree(b->p);
+    for (int k = 0; k < 2; ++k) {
+        if (t->pin[k]) (void)hipHostFree(t->pin[k]);
+        if (t->dbuf[k]) (void)hipFree(t->dbuf[k]);
+        if (t->ev_copy[k]) (void)hipEventDestroy(t->ev_copy[k]);
+        if (t->ev_done[k]) (void)hipEventDestroy(t->ev_done[k]);
+    }
+    if (t->d.slots) (void)hipFree(t->d.slots);
+    if (t->d.rows) (void)hipFree(t->d.rows);
+    if (t->d.row_keys) (void)hipFree(t->d.row_keys);
+    if (t->d.counters) (void)hipFree(t->d.counters);
+    if (t->d_hist) (void)hipFree(t->d_hist);
+    if (t->h_counters) (void)hipHostFree(t->h_counters);
+    if (t->h_hist) (void)hipHostFree(t->h_hist);
+    if (t->order_ev) (void)hipEventDestroy(t->order_ev);
+    if (t->stream) (void)hipStreamDestroy(t->stream);
+    if (t->side) (void)hipStreamDestroy(t->side);
+    delete t;
+}
+
+thread_local std::string g_create_error;
+
+}  // namespace
+
+extern "C" {
+
+uint32_t pshbm_value_floats(uint32_t dim, int32_t optimizer) {
+    switch (optimizer) {
+        case PSHBM_OPT_SUM:
+        case PSHBM_OPT_SGD: return dim;
+        case PSHBM_OPT_ADAGRAD: return 2 * dim;
+        case PSHBM_OPT_FTRL: return 3 * dim;
+    }
+    return 0;
+}
+
+const char* pshbm_last_error(const pshbm_table* t) {
+    return t ? t->err.c_str() : g_create_error.c_str();
+}
+
+int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
+    if (!cfg || !out) return PSHBM_INVALID_CONFIG;
+    *out = nullptr;
+    auto bad = [&](const char* m) {
+        g_create_error = m;
+        return PSHBM_INVALID_CONFIG;
+    };
+    if (cfg->struct_size != sizeof(pshbm_config)) return bad("struct_size does not match this library");
+    if (cfg->dim == 0 || cfg->dim > MAX_DIM) return bad("dim must be in [1, 16384]");
+    const uint32_t vf = pshbm_value_floats(cfg->dim, cfg->optimizer);
+    if (vf == 0) return bad("unknown optimizer");
+    if (cfg->expected_max_items == 0 || cfg->expected_max_items > 0xFFFFFFF0ull)
+        return bad("expected_max_items must be in [1, 2^32-16]");
+    float lf = cfg->max_load_factor == 0.0f ? 0.5f : cfg->max_load_factor;
+    if (!(lf > 0.0f && lf <= 0.9f)) return bad("max_load_factor must be in (0, 0.9]");
+    if (cfg->optimizer == PSHBM_OPT_FTRL && !(cfg->alpha > 0.0f)) return bad("FTRL needs alpha > 0");
+
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess || ndev == 0) {
+        g_create_error = std::string("no HIP device: ") + hipGetErrorString(e);
+        return PSHBM_ERROR;
+    }
+    if (cfg->device < 0 || cfg->device >= ndev) return bad("device ordinal out of range");
+
+    pshbm_table* t = new (std::nothrow) pshbm_table();
+    if (!t) return PSHBM_OUT_OF_MEMORY;
+    t->cfg = *cfg;
+    t->cfg.max_load_factor = lf;
+    t->device = cfg->device;
+    DeviceGuard g(t->device);
+
+    const uint64_t max_rows = cfg->expected_max_items;
+    uint64_t want_slots = (uint64_t)((double)max_rows / lf) + 1;
+    uint64_t nb = 16;
+    while (nb * 4 < want_slots) nb <<= 1;
+    if (nb * 4 > (1ull << 31)) {
+        delete t;
+        return bad("table needs more than 2^31 slots");
+    }
+    t->nbuckets = nb;
+    t->slot_bits = 0;
+    while ((1ull << t->slot_bits) < nb * 4) ++t->slot_bits;
+
+    TableDev& d = t->d;
+    d.bucket_mask = (uint32_t)(nb - 1);
+    d.max_rows = (uint32_t)max_rows;
+    d.dim = cfg->dim;
+    d.vf = vf;
+    d.stride_f = (uint32_t)round_up(vf, 4);
+    d.opt = OptParams{cfg->optimizer, cfg->lr, cfg->init_acc, cfg->alpha, cfg->beta, cfg->l1, cfg->l2};
+    t->slots_bytes = nb * 64;
+    t->rows_bytes = max_rows * d.stride_f * 4;
+    t->keys_bytes = max_rows * 8;
+
+    auto bail = [&](hipError_t err, const char* what) {
+        g_create_error = std::string(what) + ": " + hipGetErrorString(err);
+        int32_t code = err == hipErrorOutOfMemory ? PSHBM_OUT_OF_MEMORY : PSHBM_ERROR;
+        destroy_impl(t);
+        return code;
+    };
+#define CREATE_TRY(expr)                              \
+    do {                                              \
+        hipError_t e__ = (expr);                      \
+        if (e__ != hipSuccess) return bail(e__, #expr); \
+    } while (0)
+    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.slots), t->slots_bytes));
+    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.rows), t->rows_bytes));
+    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.row_keys), t->keys_bytes));
+    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.counters), CNT_WORDS * 4));
+    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&t->d_hist), 17 * 8));
+    CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_counters), CNT_WORDS * 4, hipHostMallocDefault));
+    CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_hist), 17 * 8, hipHostMallocDefault));
+    CREATE_TRY(hipStreamCreateWithFlags(&t->stream, hipStreamNonBlocking));
+    CREATE_TRY(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));
+    CREATE_TRY(hipEventCreateWithFlags(&t->order_ev, hipEventDisableTiming));
+    CREATE_TRY(hipMemsetAsync(d.slots, 0xFF, t->slots_bytes, t->stream));
+    CREATE_TRY(hipMemsetAsync(d.counters, 0, CNT_WORDS * 4, t->stream));
+    CREATE_TRY(hipStreamSynchronize(t->stream));
+#undef CREATE_TRY
+    int32_t st = ensure_workspace(t, cfg->max_batch ? cfg->max_batch : 65536);
+    if (st != PSHBM_OK) {
+        g_create_error = t->err;
+        destroy_impl(t);
+        return st;
+    }
+    *out = t;
+    return PSHBM_OK;
+}
+
+int32_t pshbm_destroy(pshbm_table* t) {
+    if (!t) return PSHBM_OK;
+    destroy_impl(t);
+    return PSHBM_OK;
+}
+
+// ---- pull ------------------------------------------------------------------------------------
+int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* d_out_rows,
+                       uint8_t* d_hit, uint32_t flags, void* stream) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!d_keys || !d_out_rows) return fail(t, PSHBM_ERROR, "pull: null buffer");
+    if (n > 0x7FFFFFFFull) return fail(t, PSHBM_ERROR, "pull: batch larger than 2^31-1 keys");
+    DeviceGuard g(t->device);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool insert = (flags & PSHBM_PULL_INSERT_ON_MISS) && !t->cfg.read_only;
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    ST_TRY(begin_op(t, s));
+    if (!insert) {
+        HIP_TRY(t, launch_pull(t->d, d_keys, n, d_out_rows, d_hit, s));
+        return PSHBM_OK;
+    }
+    ST_TRY(ensure_workspace(t, n));
+    bool checked = false;
+    uint32_t rows_before = 0;
+    ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
+    uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
+    HIP_TRY(t, launch_snapshot_entry(t->d, s));
+    HIP_TRY(t, launch_locate(t->d, d_keys, n, slot, nullptr, true, true, false, s));
+    if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
+    HIP_TRY(t, launch_gather_slots(t->d, slot, n, d_out_rows, d_hit, s));
+    return PSHBM_OK;
+}
+
+int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_rows, uint8_t* hit,
+                   uint32_t flags) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!keys || !out_rows) return fail(t, PSHBM_ERROR, "pull: null buffer");
+    if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "pull: reserved key in batch");
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    const size_t out_bytes = n * (size_t)t->d.dim * 4;
+    ST_TRY(ensure(t, t->st_keys, n * 8));
+    ST_TRY(ensure(t, t->st_out, out_bytes));
+    ST_TRY(ensure(t, t->st_hit, n));
+    hipStream_t s = t->stream;
+    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, n * 8, hipMemcpyHostToDevice, s));
+    ST_TRY(pshbm_pull_dev(t, static_cast<const uint64_t*>(t->st_keys.p), n,
+                          static_cast<float*>(t->st_out.p), static_cast<uint8_t*>(t->st_hit.p), flags, s));
+    HIP_TRY(t, hipMemcpyAsync(out_rows, t->st_out.p, out_bytes, hipMemcpyDeviceToHost, s));
+    if (hit) HIP_TRY(t, hipMemcpyAsync(hit, t->st_hit.p, n, hipMemcpyDeviceToHost, s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    return PSHBM_OK;
+}
+
+// ---- push ------------------------------------------------------------------------------------
+int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
+                       uint32_t flags, void* stream) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!d_keys || !d_grads) return fail(t, PSHBM_ERROR, "push: null buffer");
+    if (n > 0x7FFFFFFFull) return fail(t, PSHBM_ERROR, "push: batch larger than 2^31-1 keys");
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    return push_locked(t, d_keys, d_grads, n, flags, static_cast<hipStream_t>(stream));
+}
+
+int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, size_t n, uint32_t flags) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!keys || !grads) return fail(t, PSHBM_ERROR, "push: null buffer");
+    if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "push: reserved key in batch");
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    const size_t gbytes = n * (size_t)t->d.dim * 4;
+    ST_TRY(ensure(t, t->st_keys, n * 8));
+    ST_TRY(ensure(t, t->st_vals, gbytes));
+    hipStream_t s = t->stream;
+    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, n * 8, hipMemcpyHostToDevice, s));
+    HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, grads, gbytes, hipMemcpyHostToDevice, s));
+    int32_t st = pshbm_push_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
+                                static_cast<const float*>(t->st_vals.p), n, flags, s);
+    HIP_TRY(t, hipStreamSynchronize(s));
+    return st;
+}
+
+int32_t pshbm_push_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride, uint32_t flags) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!pairs) return fail(t, PSHBM_ERROR, "push_pairs: null buffer");
+    const size_t used = 8 + (size_t)t->d.dim * 4;
+    if (stride < used || stride % 4) return fail(t, PSHBM_ERROR, "push_pairs: bad stride %zu", stride);
+    const char* p = static_cast<const char*>(pairs);
+    for (size_t i = 0; i < n; ++i) {
+        uint64_t k;
+        std::memcpy(&k, p + i * stride, 8);
+        if (k >= KEY_DELETED) return fail(t, PSHBM_ERROR, "push_pairs: reserved key in batch");
+    }
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    ST_TRY(ensure(t, t->st_raw, n * stride));
+    ST_TRY(ensure(t, t->st_keys, n * 8));
+    ST_TRY(ensure(t, t->st_vals, n * (size_t)t->d.dim * 4));
+    hipStream_t s = t->stream;
+    HIP_TRY(t, hipMemcpyAsync(t->st_raw.p, pairs, n * stride, hipMemcpyHostToDevice, s));
+    HIP_TRY(t, launch_unpack_records(static_cast<const uint32_t*>(t->st_raw.p), n,
+                                     (uint32_t)(stride / 4), t->d.dim,
+                                     static_cast<uint64_t*>(t->st_keys.p),
+                                     static_cast<float*>(t->st_vals.p), s));
+    int32_t st = pshbm_push_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
+                                static_cast<const float*>(t->st_vals.p), n, flags, s);
+    HIP_TRY(t, hipStreamSynchronize(s));
+    return st;
+}
+
+// ---- sync push: queue + store ----------------------------------------------------------------
+int32_t pshbm_queue_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
+                        void* stream) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!d_keys || !d_grads) return fail(t, PSHBM_ERROR, "queue: null buffer");
+    DeviceGuard g(t->device);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    if (t->q_n + n > 0x7FFFFFFFull) return fail(t, PSHBM_ERROR, "queue: more than 2^31-1 keys queued");
+    ST_TRY(begin_op(t, s));
+    const size_t gb = (size_t)t->d.dim * 4;
+    const size_t need = t->q_n + n;
+    if (need * 8 > t->q_keys.bytes) {  // grow, keeping what is queued
+        DevBuf nk, ng;
+        size_t cap = std::max(need * 2, (size_t)65536);
+        HIP_TRY(t, hipStreamSynchronize(s));
+        HIP_TRY(t, hipMalloc(&nk.p, cap * 8));
+        nk.bytes = cap * 8;
+        hipError_t e = hipMalloc(&ng.p, cap * gb);
+        if (e != hipSuccess) {
+            (void)hipFree(nk.p);
+            return hip_fail(t, e, "queue: hipMalloc");
+        }
+        ng.bytes = cap * gb;
+        if (t->q_n) {
+            HIP_TRY(t, hipMemcpy(nk.p, t->q_keys.p, t->q_n * 8, hipMemcpyDeviceToDevice));
+            HIP_TRY(t, hipMemcpy(ng.p, t->q_grads.p, t->q_n * gb, hipMemcpyDeviceToDevice));
+        }
+        if (t->q_keys.p) (void)hipFree(t->q_keys.p);
+        if (t->q_grads.p) (void)hipFree(t->q_grads.p);
+        t->q_keys = nk;
+        t->q_grads = ng;
+    }
+    HIP_TRY(t, hipMemcpyAsync(static_cast<uint64_t*>(t->q_keys.p) + t->q_n, d_keys, n * 8,
+                              hipMemcpyDeviceToDevice, s));
+    HIP_TRY(t, hipMemcpyAsync(static_cast<char*>(t->q_grads.p) + t->q_n * gb, d_grads, n * gb,
+                              hipMemcpyDeviceToDevice, s));
+    t->q_n += n;
+    return PSHBM_OK;
+}
+
+int32_t pshbm_queue(pshbm_table* t, const uint64_t* keys, const float* grads, size_t n) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!keys || !grads) return fail(t, PSHBM_ERROR, "queue: null buffer");
+    if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "queue: reserved key in batch");
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    const size_t gbytes = n * (size_t)t->d.dim * 4;
+    ST_TRY(ensure(t, t->st_keys, n * 8));
+    ST_TRY(ensure(t, t->st_vals, gbytes));
+    hipStream_t s = t->stream;
+    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, n * 8, hipMemcpyHostToDevice, s));
+    HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, grads, gbytes, hipMemcpyHostToDevice, s));
+    int32_t st = pshbm_queue_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
+                                 static_cast<const float*>(t->st_vals.p), n, s);
+    HIP_TRY(t, hipStreamSynchronize(s));
+    return st;
+}
+
+int32_t pshbm_queued(pshbm_table* t, uint64_t* n) {
+    if (!t || !n) return PSHBM_INVALID_ID;
+    std::shared_lock<std::shared_mutex> lk(t->mu);
+    *n = t->q_n;
+    return PSHBM_OK;
+}
+
+int32_t pshbm_store_dev(pshbm_table* t, uint32_t flags, void* stream) {
+    if (!t) return PSHBM_INVALID_ID;
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    const size_t n = t->q_n;
+    t->q_n = 0;
+    return push_locked(t, static_cast<const uint64_t*>(t->q_keys.p),
+                       static_cast<const float*>(t->q_grads.p), n,
+                       flags & ~PSHBM_PUSH_ASSUME_UNIQUE, static_cast<hipStream_t>(stream));
+}
+
+int32_t pshbm_store(pshbm_table* t, uint32_t flags) {
+    if (!t) return PSHBM_INVALID_ID;
+    DeviceGuard g(t->device);
+    int32_t st = pshbm_store_dev(t, flags, t->stream);
+    HIP_TRY(t, hipStreamSynchronize(t->stream));
+    return st;
+}
+
+// ---- set / load / dump / iterate ---------------------------------------------------------------
+int32_t pshbm_set_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_values, size_t n,
+                      void* stream) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!d_keys || !d_values) return fail(t, PSHBM_ERROR, "set: null buffer");
+    if (n > 0x7FFFFFFFull) return fail(t, PSHBM_ERROR, "set: batch larger than 2^31-1 keys");
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    return set_locked(t, d_keys, d_values, n, false, static_cast<hipStream_t>(stream));
+}
+
+int32_t pshbm_set(pshbm_table* t, const uint64_t* keys, const float* values, size_t n) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!keys || !values) return fail(t, PSHBM_ERROR, "set: null buffer");
+    if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "set: reserved key in batch");
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    const size_t vbytes = n * (size_t)t->d.vf * 4;
+    ST_TRY(ensure(t, t->st_keys, n * 8));
+    ST_TRY(ensure(t, t->st_vals, vbytes));
+    hipStream_t s = t->stream;
+    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, n * 8, hipMemcpyHostToDevice, s));
+    HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, values, vbytes, hipMemcpyHostToDevice, s));
+    int32_t st = pshbm_set_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
+                               static_cast<const float*>(t->st_vals.p), n, s);
+    HIP_TRY(t, hipStreamSynchronize(s));
+    return st;
+}
+
+int32_t pshbm_load(pshbm_table* t, const void* records, size_t n, uint32_t flags) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!records) return fail(t, PSHBM_ERROR, "load: null buffer");
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    ST_TRY(ensure_bulk(t));
+    const size_t rec = 8 + (size_t)t->d.vf * 4;
+    const size_t per_chunk = BULK_CHUNK_BYTES / rec;
+    if (per_chunk == 0) return fail(t, PSHBM_ERROR, "load: record larger than the staging chunk");
+    ST_TRY(ensure(t, t->st_keys, per_chunk * 8));
+    ST_TRY(ensure(t, t->st_vals, per_chunk * (size_t)t->d.vf * 4));
+    ST_TRY(ensure_workspace(t, per_chunk));
+    hipStream_t s = t->stream;
+    ST_TRY(begin_op(t, s));
+    const bool unique = (flags & PSHBM_LOAD_UNIQUE) != 0;
+    if (unique) HIP_TRY(t, hipMemsetAsync(t->d.counters + CNT_DUP, 0, 4, s));
+    const char* src = static_cast<const char*>(records);
+    int32_t status = PSHBM_OK;
+    size_t chunk = 0;
+    for (size_t off = 0; off < n; off += per_chunk, ++chunk) {
+        const size_t cnt = std::min(per_chunk, n - off);
+        const int k = (int)(chunk & 1);
+        if (chunk >= 2) {
+            HIP_TRY(t, hipEventSynchronize(t->ev_copy[k]));  // pinned chunk has left the host
+        }
+        const char* rp = src + off * rec;
+        for (size_t i = 0; i < cnt; ++i) {
+            uint64_t key;
+            std::memcpy(&key, rp + i * rec, 8);
+            if (key >= KEY_DELETED) {
+                status = fail(t, PSHBM_ERROR, "load: reserved key in record %zu", off + i);
+                break;
+            }
+        }
+        if (status != PSHBM_OK) break;
+        std::memcpy(t->pin[k], rp, cnt * rec);
+        if (chunk >= 2) HIP_TRY(t, hipStreamWaitEvent(t->side, t->ev_done[k], 0));  // device chunk consumed
+        HIP_TRY(t, hipMemcpyAsync(t->dbuf[k], t->pin[k], cnt * rec, hipMemcpyHostToDevice, t->side));
+        HIP_TRY(t, hipEventRecord(t->ev_copy[k], t->side));
+        HIP_TRY(t, hipStreamWaitEvent(s, t->ev_copy[k], 0));
+        HIP_TRY(t, launch_unpack_records(static_cast<const uint32_t*>(t->dbuf[k]), cnt,
+                                         (uint32_t)(rec / 4), t->d.vf,
+                                         static_cast<uint64_t*>(t->st_keys.p),
+                                         static_cast<float*>(t->st_vals.p), s));
+        HIP_TRY(t, hipEventRecord(t->ev_done[k], s));
+        status = set_locked(t, static_cast<const uint64_t*>(t->st_keys.p),
+                            static_cast<const float*>(t->st_vals.p), cnt, unique, s);
+        if (status != PSHBM_OK) break;
+    }
+    HIP_TRY(t, hipStreamSynchronize(t->side));
+    ST_TRY(read_counters(t, s));
+    if (status != PSHBM_OK) return status;
+    if (unique && t->h_counters[CNT_DUP])
+        return fail(t, PSHBM_ERROR, "load: %u keys were already present or repeated",
+                    t->h_counters[CNT_DUP]);
+    return PSHBM_OK;
+}
+
+static int32_t dump_range(pshbm_table* t, size_t first, size_t count, void* records) {
+    ST_TRY(ensure_bulk(t));
+    const size_t rec = 8 + (size_t)t->d.vf * 4;
+    const size_t per_chunk = BULK_CHUNK_BYTES / rec;
+    if (per_chunk == 0) return fail(t, PSHBM_ERROR, "dump: record larger than the staging chunk");
+    hipStream_t s = t->stream;
+    char* dst = static_cast<char*>(records);
+    size_t chunk = 0;
+    size_t pending_off[2] = {0, 0}, pending_cnt[2] = {0, 0};
+    for (size_t off = 0; off < count; off += per_chunk, ++chunk) {
+        const size_t cnt = std::min(per_chunk, count - off);
+        const int k = (int)(chunk & 1);
+        if (chunk >= 2) {  // drain the chunk that used this pair of buffers
+            HIP_TRY(t, hipEventSynchronize(t->ev_copy[k]));
+            std::memcpy(dst + pending_off[k] * rec, t->pin[k], pending_cnt[k] * rec);
+        }
+        HIP_TRY(t, launch_pack_records(t->d, (uint32_t)(first + off), cnt,
+                                       static_cast<uint32_t*>(t->dbuf[k]), s));
+        HIP_TRY(t, hipEventRecord(t->ev_done[k], s));
+        HIP_TRY(t, hipStreamWaitEvent(t->side, t->ev_done[k], 0));
+        HIP_TRY(t, hipMemcpyAsync(t->pin[k], t->dbuf[k], cnt * rec, hipMemcpyDeviceToHost, t->side));
+        HIP_TRY(t, hipEventRecord(t->ev_copy[k], t->side));
+        // dbuf[k] and pin[k] are reused two chunks later, after the host has waited for ev_copy[k]
+        pending_off[k] = off;
+        pending_cnt[k] = cnt;
+    }
+    const size_t nchunks = chunk;
+    for (size_t c = (nchunks >= 2 ? nchunks - 2 : 0); c < nchunks; ++c) {
+        const int k = (int)(c & 1);
+        HIP_TRY(t, hipEventSynchronize(t->ev_copy[k]));
+        std::memcpy(dst + pending_off[k] * rec, t->pin[k], pending_cnt[k] * rec);
+    }
+    HIP_TRY(t, hipStreamSynchronize(s));
+    return PSHBM_OK;
+}
+
+int32_t pshbm_iterate(pshbm_table* t, size_t offset, size_t batch, void* records, size_t* n_out) {
+    if (!t || !n_out) return PSHBM_INVALID_ID;
+    *n_out = 0;
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    ST_TRY(begin_op(t, t->stream));
+    ST_TRY(read_counters(t, t->stream));
+    const size_t size = t->h_counters[CNT_ROWS];
+    if (offset >= size || batch == 0) return PSHBM_OK;
+    if (!records) return fail(t, PSHBM_ERROR, "iterate: null buffer");
+    const size_t cnt = std::min(batch, size - offset);
+    ST_TRY(dump_range(t, offset, cnt, records));
+    *n_out = cnt;
+    return PSHBM_OK;
+}
+
+int32_t pshbm_dump(pshbm_table* t, void* records, size_t capacity_records, size_t* n_out) {
+    if (!t || !n_out) return PSHBM_INVALID_ID;
+    *n_out = 0;
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    ST_TRY(begin_op(t, t->stream));
+    ST_TRY(read_counters(t, t->stream));
+    const size_t size = t->h_counters[CNT_ROWS];
+    if (size == 0) return PSHBM_OK;
+    if (capacity_records < size)
+        return fail(t, PSHBM_ERROR, "dump: buffer holds %zu records, table has %zu", capacity_records, size);
+    if (!records) return fail(t, PSHBM_ERROR, "dump: null buffer");
+    ST_TRY(dump_range(t, 0, size, records));
+    *n_out = size;
+    return PSHBM_OK;
+}
+
+// ---- clear / size / stats ----------------------------------------------------------------------
+int32_t pshbm_clear(pshbm_table* t) {
+    if (!t) return PSHBM_INVALID_ID;
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    hipStream_t s = t->stream;
+    ST_TRY(begin_op(t, s));
+    HIP_TRY(t, hipMemsetAsync(t->d.slots, 0xFF, t->slots_bytes, s));
+    HIP_TRY(t, hipMemsetAsync(t->d.counters, 0, CNT_WORDS * 4, s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    t->size_bound = 0;
+    return PSHBM_OK;
+}
+
+int32_t pshbm_size(pshbm_table* t, uint64_t* n) {
+    if (!t || !n) return PSHBM_INVALID_ID;
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    ST_TRY(begin_op(t, t->stream));
+    ST_TRY(read_counters(t, t->stream));
+    t->size_bound = t->h_counters[CNT_ROWS];
+    *n = t->h_counters[CNT_ROWS];
+    return PSHBM_OK;
+}
+
+int32_t pshbm_memory_usage(pshbm_table* t, uint64_t* bytes) {
+    if (!t || !bytes) return PSHBM_INVALID_ID;
+    std::shared_lock<std::shared_mutex> lk(t->mu);
+    *bytes = t->slots_bytes + t->rows_bytes + t->keys_bytes;
+    return PSHBM_OK;
+}
+
+int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out) {
+    if (!t || !out) return PSHBM_INVALID_ID;
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    hipStream_t s = t->stream;
+    ST_TRY(begin_op(t, s));
+    ST_TRY(read_counters(t, s));
+    const uint32_t rows = t->h_counters[CNT_ROWS];
+    HIP_TRY(t, hipMemsetAsync(t->d_hist, 0, 17 * 8, s));
+    HIP_TRY(t, launch_probe_hist(t->d, rows, t->d_hist, s));
+    HIP_TRY(t, hipMemcpyAsync(t->h_hist, t->d_hist, 17 * 8, hipMemcpyDeviceToHost, s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    std::memset(out, 0, sizeof *out);
+    out->size = rows;
+    out->capacity = t->d.max_rows;
+    out->slots = t->nbuckets * 4;
+    out->memory_usage = t->slots_bytes + t->rows_bytes + t->keys_bytes;
+    out->load_factor = (double)rows / (double)(t->nbuckets * 4);
+    for (int i = 0; i < 16; ++i) out->probe_hist[i] = t->h_hist[i];
+    out->max_probe = t->h_hist[16];
+    return PSHBM_OK;
+}
+
+int32_t pshbm_host_alloc(void** p, size_t bytes) {
+    if (!p) return PSHBM_ERROR;
+    hipError_t e = hipHostMalloc(p, bytes, hipHostMallocDefault);
+    if (e == hipSuccess) return PSHBM_OK;
+    return e == hipErrorOutOfMemory ? PSHBM_OUT_OF_MEMORY : PSHBM_ERROR;
+}
+
+int32_t pshbm_host_free(void* p) {
+    return hipHostFree(p) == hipSuccess ? PSHBM_OK : PSHBM_ERROR;
+}
+
+}  // extern "C"

@@ -1,0 +1,708 @@
+// HIP kernels of the HBM sparse table, written for gfx950 (64-wide wavefronts).
+//
+// Work decomposition used throughout: a wavefront handles a group of keys per round. Probing
+// gives four lanes to a key — they read the four 16-byte slots of one 64-byte bucket with one
+// dwordx4 load each and agree on the outcome with a ballot. Row traffic gives `row units` lanes
+// to a key, so that consecutive lanes touch consecutive 16 bytes of a row or of the packed
+// response.
+#include "table.h"
+
+namespace pshbm {
+
+using u32 = uint32_t;
+using u64 = uint64_t;
+
+namespace {
+
+constexpr int BLOCK = 256;  // 4 wavefronts
+constexpr u32 KEYS_PER_ROUND = 16;
+
+// ---- small vector helpers ------------------------------------------------------------------
+__device__ __forceinline__ float vzero(float) { return 0.0f; }
+__device__ __forceinline__ float4 vzero(float4) { return make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ __forceinline__ float vadd(float a, float b) { return a + b; }
+__device__ __forceinline__ float4 vadd(float4 a, float4 b) {
+    return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+}
+__device__ __forceinline__ float vshfl(float v, u32 src) { return __shfl(v, (int)src); }
+__device__ __forceinline__ float4 vshfl(float4 v, u32 src) {
+    return make_float4(__shfl(v.x, (int)src), __shfl(v.y, (int)src), __shfl(v.z, (int)src),
+                       __shfl(v.w, (int)src));
+}
+__device__ __forceinline__ float vshfl_up(float v, u32 d) { return __shfl_up(v, d); }
+__device__ __forceinline__ float4 vshfl_up(float4 v, u32 d) {
+    return make_float4(__shfl_up(v.x, d), __shfl_up(v.y, d), __shfl_up(v.z, d), __shfl_up(v.w, d));
+}
+__device__ __forceinline__ u64 shfl64(u64 v, u32 src) {
+    u32 lo = __shfl((u32)v, (int)src);
+    u32 hi = __shfl((u32)(v >> 32), (int)src);
+    return ((u64)hi << 32) | lo;
+}
+
+// n / d for n*d < 2^32 by one multiply: m = ceil(2^32 / d) (d == 1 handled by m = 2^32).
+__device__ __forceinline__ u32 div_small(u32 n, u64 m) { return (u32)(((u64)n * m) >> 32); }
+// n / d for any 64-bit n by one multiply-high: m = ceil(2^64 / d), d >= 2.
+__device__ __forceinline__ u64 div_big(u64 n, u64 m, u32 d) { return d == 1 ? n : __umul64hi(n, m); }
+
+inline u64 magic32(u32 d) { return ((1ull << 32) + d - 1) / d; }
+inline u64 magic64(u32 d) { return d <= 1 ? 0 : (~0ull / d) + 1; }
+
+// ---- probing -------------------------------------------------------------------------------
+struct Found {
+    u32 slot;
+    u32 row;
+};
+
+// Four lanes (sub = 0..3 of group grp) look for `key`. Every lane of the wavefront must call
+// this; lanes whose `active` is false only take part in the ballots.
+__device__ __forceinline__ Found probe_find(const TableDev& t, u64 key, bool active, u32 grp,
+                                            u32 sub) {
+    Found f{SLOT_NONE, ROW_NONE};
+    u32 b = (u32)hash64(key) & t.bucket_mask;
+    bool done = !active;
+    u32 steps = 0;
+    while (__ballot(!done)) {
+        uint4 s = make_uint4(0u, 0u, 0u, 0u);
+        if (!done) s = t.slots[(u64)b * 4 + sub];
+        u64 skey = ((u64)s.y << 32) | s.x;
+        bool match = !done && skey == key;
+        bool empty = !done && skey == KEY_EMPTY;
+        u32 m4 = (u32)(__ballot(match) >> (grp * 4)) & 0xFu;
+        u32 e4 = (u32)(__ballot(empty) >> (grp * 4)) & 0xFu;
+        u32 src = grp * 4 + (m4 ? (u32)__ffs((int)m4) - 1u : 0u);
+        u32 row = __shfl(s.z, (int)src);
+        if (!done) {
+            if (m4) {
+                f.slot = b * 4 + (src & 3u);
+                f.row = row;
+                done = true;
+            } else if (e4) {
+                done = true;
+            } else {
+                b = (b + 1) & t.bucket_mask;
+                if (++steps > t.bucket_mask) done = true;
+            }
+        }
+    }
+    return f;
+}
+
+__device__ __forceinline__ float init_float(const TableDev& t, u32 f) {
+    return (t.opt.kind == 2 /*ADAGRAD*/ && f >= t.dim) ? t.opt.init_acc : 0.0f;
+}
+
+// ---- row gather into the packed response -----------------------------------------------------
+// `row` holds, in the lanes of group k, the row of key base + k (ROW_NONE = miss -> zeros).
+template <typename T>
+__device__ __forceinline__ void gather_round(const TableDev& t, u32 row, u64 base, u32 cnt,
+                                             T* __restrict__ out, u32 units, u32 stride_units,
+                                             u64 m32, u32 lane) {
+    const T* rows = reinterpret_cast<const T*>(t.rows);
+    const u32 total = cnt * units;
+    for (u32 j0 = 0; j0 < total; j0 += 64) {
+        u32 j = j0 + lane;
+        bool on = j < total;
+        u32 k = on ? div_small(j, m32) : 0u;
+        u32 c = j - k * units;
+        u32 r = __shfl(row, (int)(k * 4));
+        if (on) {
+            T v = vzero(T());
+            if (r != ROW_NONE) v = rows[(u64)r * stride_units + c];
+            out[base * units + j] = v;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void pull_kernel(TableDev t, const u64* __restrict__ keys,
+                                                      u32 n, T* __restrict__ out,
+                                                      uint8_t* __restrict__ hit, u32 units,
+                                                      u32 stride_units, u64 m32) {
+    const u32 lane = threadIdx.x & 63u;
+    const u32 grp = lane >> 2, sub = lane & 3u;
+    const u64 wave = ((u64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
+    const u64 nwaves = ((u64)gridDim.x * BLOCK) >> 6;
+    for (u64 base = wave * KEYS_PER_ROUND; base < n; base += nwaves * KEYS_PER_ROUND) {
+        u64 i = base + grp;
+        bool inb = i < n;
+        u64 key = inb ? keys[i] : KEY_EMPTY;
+        bool active = inb && key < KEY_DELETED;
+        Found f = probe_find(t, key, active, grp, sub);
+        if (hit && inb && sub == 0) hit[i] = f.row != ROW_NONE;
+        u32 cnt = (u32)((n - base) < KEYS_PER_ROUND ? (n - base) : KEYS_PER_ROUND);
+        gather_round<T>(t, f.row, base, cnt, out, units, stride_units, m32, lane);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void gather_slots_kernel(TableDev t,
+                                                              const u32* __restrict__ slot_idx,
+                                                              u32 n, T* __restrict__ out,
+                                                              uint8_t* __restrict__ hit, u32 units,
+                                                              u32 stride_units, u64 m32) {
+    const u32 lane = threadIdx.x & 63u;
+    const u32 grp = lane >> 2, sub = lane & 3u;
+    const u64 wave = ((u64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
+    const u64 nwaves = ((u64)gridDim.x * BLOCK) >> 6;
+    const u32 entry_rows = t.counters[CNT_ENTRY];
+    for (u64 base = wave * KEYS_PER_ROUND; base < n; base += nwaves * KEYS_PER_ROUND) {
+        u64 i = base + grp;
+        u32 row = ROW_NONE;
+        if (i < n) {
+            u32 s = slot_idx[i];
+            if (s != SLOT_NONE) row = reinterpret_cast<const u32*>(&t.slots[s])[2];
+            if (row >= t.max_rows) row = ROW_NONE;
+            if (hit && sub == 0) hit[i] = row < entry_rows;
+        }
+        u32 cnt = (u32)((n - base) < KEYS_PER_ROUND ? (n - base) : KEYS_PER_ROUND);
+        gather_round<T>(t, row, base, cnt, out, units, stride_units, m32, lane);
+    }
+}
+
+// ---- locate / claim ------------------------------------------------------------------------
+template <bool kInsert>
+__global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __restrict__ keys,
+                                                        u32 n, u32* __restrict__ slot_out,
+                                                        u32* __restrict__ idx_out, int init_rows,
+                                                        int count_dups) {
+    const u32 lane = threadIdx.x & 63u;
+    const u32 grp = lane >> 2, sub = lane & 3u;
+    const u64 wave = ((u64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
+    const u64 nwaves = ((u64)gridDim.x * BLOCK) >> 6;
+    for (u64 base = wave * KEYS_PER_ROUND; base < n; base += nwaves * KEYS_PER_ROUND) {
+        u64 i = base + grp;
+        bool inb = i < n;
+        u64 key = inb ? keys[i] : KEY_EMPTY;
+        bool active = inb && key < KEY_DELETED;
+        if (inb && !active && sub == 0) atomicAdd(&t.counters[CNT_BADKEY], 1u);
+        u32 slot = SLOT_NONE;
+        bool dup = false;
+        if constexpr (!kInsert) {
+            Found f = probe_find(t, key, active, grp, sub);
+            slot = f.slot;
+            dup = f.slot != SLOT_NONE;
+        } else {
+            bool won = false;
+            bool done = !active;
+            u32 b = (u32)hash64(key) & t.bucket_mask;
+            u32 steps = 0;
+            while (__ballot(!done)) {
+                u64 skey = 0;
+                // Coherent at the device level: a slot claimed by another compute unit during
+                // this launch must be seen, so the load bypasses the per-CU cache.
+                if (!done)
+                    skey = __hip_atomic_load(reinterpret_cast<u64*>(&t.slots[(u64)b * 4 + sub]),
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                bool match = !done && skey == key;
+                bool empty = !done && skey == KEY_EMPTY;
+                u32 m4 = (u32)(__ballot(match) >> (grp * 4)) & 0xFu;
+                u32 e4 = (u32)(__ballot(empty) >> (grp * 4)) & 0xFu;
+                u32 tgt = e4 ? (u32)__ffs((int)e4) - 1u : 0u;
+                bool do_cas = !done && !m4 && e4 && sub == tgt;
+                u64 old = 0;
+                if (do_cas)
+                    old = atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[(u64)b * 4 + tgt]),
+                                    (unsigned long long)KEY_EMPTY, (unsigned long long)key);
+                u64 oldb = shfl64(old, grp * 4 + tgt);
+                if (!done) {
+                    if (m4) {
+                        slot = b * 4 + (u32)__ffs((int)m4) - 1u;
+                        dup = true;
+                        done = true;
+                    } else if (e4) {
+                        if (oldb == KEY_EMPTY) {
+                            slot = b * 4 + tgt;
+                            won = true;
+                            done = true;
+                        } else if (oldb == key) {  // the same key, claimed by another group
+                            slot = b * 4 + tgt;
+                            dup = true;
+                            done = true;
+                        }
+                        // otherwise another key took the slot: look at this bucket again
+                    } else {
+                        b = (b + 1) & t.bucket_mask;
+                        if (++steps > t.bucket_mask) {
+                            done = true;
+                            if (sub == 0) t.counters[CNT_OVERFLOW] = 1u;
+                        }
+                    }
+                }
+            }
+            // Rows for the winners: one atomic per wavefront.
+            u64 wm = __ballot(won && sub == 0);
+            if (wm) {
+                u32 first = 0;
+                if (lane == 0) first = atomicAdd(&t.counters[CNT_ROWS], (u32)__popcll(wm));
+                first = __shfl(first, 0);
+                if (won) {
+                    u32 rank = (u32)__popcll(wm & ((1ull << (grp * 4)) - 1ull));
+                    u32 rid = first + rank;
+                    if (rid < t.max_rows) {
+                        if (sub == 0) {
+                            reinterpret_cast<u32*>(&t.slots[slot])[2] = rid;
+                            t.row_keys[rid] = key;
+                        }
+                        if (init_rows) {
+                            float4* r4 = reinterpret_cast<float4*>(t.rows + (u64)rid * t.stride_f);
+                            for (u32 c = sub; c < t.stride_f / 4; c += 4) {
+                                u32 f = c * 4;
+                                r4[c] = make_float4(init_float(t, f), init_float(t, f + 1),
+                                                    init_float(t, f + 2), init_float(t, f + 3));
+                            }
+                        }
+                    } else if (sub == 0) {
+                        t.counters[CNT_OVERFLOW] = 1u;
+                    }
+                }
+            }
+        }
+        if (inb && sub == 0) {
+            slot_out[i] = slot;
+            if (idx_out) idx_out[i] = (u32)i;
+            if (count_dups && dup) atomicAdd(&t.counters[CNT_DUP], 1u);
+        }
+    }
+}
+
+__global__ void snapshot_entry_kernel(TableDev t) { t.counters[CNT_ENTRY] = t.counters[CNT_ROWS]; }
+
+__global__ __launch_bounds__(BLOCK) void rollback_kernel(TableDev t, const u32* __restrict__ slot_idx,
+                                                          u32 n, u32 first_new_row) {
+    u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x;
+    if (i == 0) {
+        t.counters[CNT_ROWS] = first_new_row;
+        t.counters[CNT_OVERFLOW] = 0u;
+    }
+    if (i >= n) return;
+    u32 s = slot_idx[i];
+    if (s == SLOT_NONE) return;
+    u32 r = reinterpret_cast<const u32*>(&t.slots[s])[2];
+    if (r == ROW_NONE || r >= first_new_row)
+        t.slots[s] = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu);
+}
+
+__global__ __launch_bounds__(BLOCK) void fill_u32_kernel(u32* p, u64 n, u32 v) {
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (u64)gridDim.x * BLOCK) p[i] = v;
+}
+
+// ---- optimizer step ------------------------------------------------------------------------
+// One fp32 element; each operation rounds on its own (the file is compiled with
+// -ffp-contract=off and correctly rounded divide / sqrt).
+__device__ __forceinline__ void opt_step(const OptParams& o, float g, float& w, float& s1,
+                                         float& s2) {
+    switch (o.kind) {
+        case 0:  // SUM
+            w = w + g;
+            break;
+        case 1: {  // SGD
+            float step = o.lr * g;
+            w = w - step;
+        } break;
+        case 2: {  // ADAGRAD
+            float gg = g * g;
+            float nn = s1 + gg;
+            float num = o.lr * g;
+            float step = num / sqrtf(nn);
+            s1 = nn;
+            w = w - step;
+        } break;
+        default: {  // FTRL: s1 = z, s2 = n
+            float gg = g * g;
+            float n_new = s2 + gg;
+            float sq_new = sqrtf(n_new);
+            float sigma = (sq_new - sqrtf(s2)) / o.alpha;
+            float sw = sigma * w;
+            float z = (s1 + g) - sw;
+            float w_new;
+            if (fabsf(z) <= o.l1) {
+                w_new = 0.0f;
+            } else {
+                float shrunk = z > 0.0f ? z - o.l1 : z + o.l1;
+                float denom = (o.beta + sq_new) / o.alpha + o.l2;
+                w_new = -shrunk / denom;
+            }
+            w = w_new;
+            s1 = z;
+            s2 = n_new;
+        } break;
+    }
+}
+
+// Applies the aggregated gradient `g` (columns [col, col+1) in units of T) to the row in `slot`.
+template <typename T>
+__device__ __forceinline__ void finalize(const TableDev& t, u32 slot, u32 col, u32 units, T g) {
+    constexpr int N = sizeof(T) / 4;
+    u32 row = reinterpret_cast<const u32*>(&t.slots[slot])[2];
+    if (row >= t.max_rows) return;
+    T* r = reinterpret_cast<T*>(t.rows + (u64)row * t.stride_f);
+    const int kind = t.opt.kind;
+    T wv = r[col];
+    T av = vzero(T()), bv = vzero(T());
+    if (kind >= 2) av = r[units + col];
+    if (kind == 3) bv = r[2 * units + col];
+    float* gp = reinterpret_cast<float*>(&g);
+    float* wp = reinterpret_cast<float*>(&wv);
+    float* ap = reinterpret_cast<float*>(&av);
+    float* bp = reinterpret_cast<float*>(&bv);
+#pragma unroll
+    for (int e = 0; e < N; ++e) opt_step(t.opt, gp[e], wp[e], ap[e], bp[e]);
+    r[col] = wv;
+    if (kind >= 2) r[units + col] = av;
+    if (kind == 3) r[2 * units + col] = bv;
+}
+
+// ---- duplicate aggregation + update over slot-sorted pairs -------------------------------------
+// Each wavefront owns `wch` consecutive sorted positions (a chunk) and walks them in rounds of P
+// positions, `lp` lanes per position. Within a round equal slots are summed by a segmented
+// inclusive scan across lane groups; the running sum of the round's last position is carried into
+// the next round. A run that ends inside the chunk and began inside it is complete: its lanes
+// apply the optimizer step to the row at once. A run that crosses a chunk border leaves a partial
+// sum in part_val (entry 0: the run that entered from the left, entry 1: the run that leaves to
+// the right) for fixup_kernel to join.
+// part_hdr[w] = {slot of entry 0, flags of entry 0 (1 present, 2 run ends in this chunk),
+//               slot of entry 1, flags of entry 1 (1 present)}.
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void segreduce_kernel(
+    TableDev t, const u32* __restrict__ sslot, const u32* __restrict__ sidx, u32 n,
+    const T* __restrict__ grads, uint4* __restrict__ part_hdr, T* __restrict__ part_val, u32 units,
+    u32 lp_full, u32 P, u32 wch, u32 n_chunks) {
+    const u32 lane = threadIdx.x & 63u;
+    const u32 w = blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
+    if (w >= n_chunks) return;
+    const u32 col0 = blockIdx.y * 64u;
+    const u32 lp = (units - col0) < 64u ? (units - col0) : 64u;
+    const u32 g = lane / lp_full;
+    const u32 c = lane - g * lp_full;
+    const bool lane_on = g < P && c < lp;
+    const u32 cs = w * wch;
+    const u32 ce = (n - cs) < wch ? n : cs + wch;
+    const u32 pe = ce - 1;
+    const u32 first_slot = sslot[cs];
+    const bool open_left = cs > 0 && sslot[cs - 1] == first_slot;
+
+    u32 carry_slot = SLOT_NONE;
+    T carry_v = vzero(T());
+    bool l_present = false, l_ends = false, r_present = false;
+
+    for (u32 r0 = cs; r0 < ce; r0 += P) {
+        const u32 p = r0 + g;
+        const bool valid = lane_on && p < ce;
+        u32 slot = SLOT_NONE, nslot = SLOT_NONE;
+        T v = vzero(T());
+        if (valid) {
+            slot = sslot[p];
+            if (p + 1 < n) nslot = sslot[p + 1];
+            if (slot != SLOT_NONE) {
+                u32 i = sidx[p];
+                v = grads[(u64)i * units + col0 + c];
+            }
+        }
+        if (g == 0 && slot == carry_slot) v = vadd(v, carry_v);
+        // segmented inclusive scan over the P positions of the round (slots are sorted, so equal
+        // end points mean one run)
+        u32 prev = __shfl_up(slot, lp_full);
+        bool cont = valid && g > 0 && prev == slot;
+        if (__any(cont)) {
+            for (u32 off = 1; off < P; off <<= 1) {
+                u32 us = __shfl_up(slot, off * lp_full);
+                T uv = vshfl_up(v, off * lp_full);
+                if (g >= off && us == slot) v = vadd(v, uv);
+            }
+        }
+        const bool real = valid && slot != SLOT_NONE;
+        const bool is_tail = nslot != slot;
+        const bool first_run = open_left && slot == first_slot;
+        const bool do_l = real && first_run && (is_tail || p == pe);
+        const bool do_r = real && !first_run && !is_tail && p == pe;
+        if (real && !first_run && is_tail) finalize<T>(t, slot, col0 + c, units, v);
+        if (do_l) part_val[((u64)w * 2 + 0) * units + col0 + c] = v;
+        if (do_r) part_val[((u64)w * 2 + 1) * units + col0 + c] = v;
+        l_present |= __any(do_l) != 0;
+        l_ends |= __any(do_l && is_tail) != 0;
+        r_present |= __any(do_r) != 0;
+        // the running sum at the round's last position feeds the next round
+        const u32 left = ce - r0;
+        const u32 last_g = (left < P ? left : P) - 1u;
+        carry_slot = __shfl(slot, (int)(last_g * lp_full));
+        carry_v = vshfl(v, last_g * lp_full + c);
+    }
+    if (lane == 0 && blockIdx.y == 0)
+        part_hdr[w] = make_uint4(first_slot, (l_present ? 1u : 0u) | (l_ends ? 2u : 0u), sslot[pe],
+                                 r_present ? 1u : 0u);
+}
+
+// Joins the partial sums of runs that cross chunk borders: the lane group of the chunk where a
+// run leaves to the right walks the following chunks' left entries until the run ends, then
+// applies the step. The order of the additions is fixed by the chunk order, so results repeat.
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* __restrict__ part_hdr,
+                                                       const T* __restrict__ part_val, u32 units,
+                                                       u32 lp_full, u32 P, u32 n_chunks) {
+    const u32 lane = threadIdx.x & 63u;
+    const u32 wave = blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
+    const u32 col0 = blockIdx.y * 64u;
+    const u32 lp = (units - col0) < 64u ? (units - col0) : 64u;
+    const u32 g = lane / lp_full;
+    const u32 c = lane - g * lp_full;
+    const u64 w = (u64)wave * P + g;
+    if (!(g < P && c < lp) || w >= n_chunks) return;
+    const uint4 h = part_hdr[w];
+    if (!(h.w & 1u)) return;
+    const u32 col = col0 + c;
+    T acc = part_val[(w * 2 + 1) * units + col];
+    for (u64 x = w + 1; x < n_chunks; ++x) {
+        const uint4 hx = part_hdr[x];
+        if (!(hx.y & 1u) || hx.x != h.z) break;
+        acc = vadd(acc, part_val[(x * 2) * units + col]);
+        if (hx.y & 2u) break;
+    }
+    finalize<T>(t, h.z, col, units, acc);
+}
+
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void update_unique_kernel(TableDev t,
+                                                               const u32* __restrict__ slot_idx,
+                                                               u32 n, const T* __restrict__ grads,
+                                                               u32 units, u32 lp_full, u32 P) {
+    const u32 lane = threadIdx.x & 63u;
+    const u32 col0 = blockIdx.y * 64u;
+    const u32 lp = (units - col0) < 64u ? (units - col0) : 64u;
+    const u32 g = lane / lp_full;
+    const u32 c = lane - g * lp_full;
+    if (!(g < P && c < lp)) return;
+    const u64 wave = ((u64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
+    const u64 nwaves = ((u64)gridDim.x * BLOCK) >> 6;
+    for (u64 i = wave * P + g; i < n; i += nwaves * P) {
+        u32 s = slot_idx[i];
+        if (s == SLOT_NONE) continue;
+        T gv = grads[i * units + col0 + c];
+        finalize<T>(t, s, col0 + c, units, gv);
+    }
+}
+
+// ---- whole-value writes, record packing -------------------------------------------------------
+__global__ __launch_bounds__(BLOCK) void write_values_kernel(TableDev t,
+                                                              const u32* __restrict__ slot_idx,
+                                                              u64 total, const float* __restrict__ values,
+                                                              u64 m64) {
+    for (u64 q = (u64)blockIdx.x * BLOCK + threadIdx.x; q < total; q += (u64)gridDim.x * BLOCK) {
+        u64 i = div_big(q, m64, t.vf);
+        u32 f = (u32)(q - i * t.vf);
+        u32 s = slot_idx[i];
+        if (s == SLOT_NONE) continue;
+        u32 row = reinterpret_cast<const u32*>(&t.slots[s])[2];
+        if (row >= t.max_rows) continue;
+        t.rows[(u64)row * t.stride_f + f] = values[q];
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void pack_records_kernel(TableDev t, u32 first_row, u64 total,
+                                                              u32* __restrict__ rec, u32 rec_dw,
+                                                              u64 m64) {
+    const u32* rows = reinterpret_cast<const u32*>(t.rows);
+    const u32* rk = reinterpret_cast<const u32*>(t.row_keys);
+    for (u64 q = (u64)blockIdx.x * BLOCK + threadIdx.x; q < total; q += (u64)gridDim.x * BLOCK) {
+        u64 r = div_big(q, m64, rec_dw);
+        u32 off = (u32)(q - r * rec_dw);
+        u64 row = first_row + r;
+        rec[q] = off < 2 ? rk[row * 2 + off] : rows[row * t.stride_f + (off - 2)];
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void unpack_records_kernel(const u32* __restrict__ rec, u64 total,
+                                                                u32 stride_dw, u32 fpr, u32* keys,
+                                                                float* values, u64 m64) {
+    const u32 used = fpr + 2;
+    for (u64 q = (u64)blockIdx.x * BLOCK + threadIdx.x; q < total; q += (u64)gridDim.x * BLOCK) {
+        u64 r = div_big(q, m64, used);
+        u32 off = (u32)(q - r * used);
+        u32 v = rec[r * stride_dw + off];
+        if (off < 2)
+            keys[r * 2 + off] = v;
+        else
+            reinterpret_cast<u32*>(values)[r * fpr + (off - 2)] = v;
+    }
+}
+
+// distance, in buckets, between a stored key's home bucket and the bucket that holds it
+__global__ __launch_bounds__(BLOCK) void probe_hist_kernel(TableDev t, u32 n_rows,
+                                                            unsigned long long* hist) {
+    for (u64 r = (u64)blockIdx.x * BLOCK + threadIdx.x; r < n_rows; r += (u64)gridDim.x * BLOCK) {
+        u64 key = t.row_keys[r];
+        if (key >= KEY_DELETED) continue;
+        u32 b = (u32)hash64(key) & t.bucket_mask;
+        u32 dist = 0;
+        bool found = false;
+        while (!found && dist <= t.bucket_mask) {
+            for (u32 k = 0; k < 4 && !found; ++k) {
+                uint4 s = t.slots[(u64)b * 4 + k];
+                found = ((((u64)s.y) << 32) | s.x) == key;
+            }
+            if (!found) {
+                b = (b + 1) & t.bucket_mask;
+                ++dist;
+            }
+        }
+        if (!found) continue;
+        atomicAdd(&hist[dist < 15 ? dist : 15], 1ull);
+        atomicMax(&hist[16], (unsigned long long)dist);
+    }
+}
+
+inline u32 grid_for(u64 work_items, u32 per_block, u32 cap) {
+    u64 b = (work_items + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    if (b > cap) b = cap;
+    return (u32)b;
+}
+
+inline bool vec4_ok(const TableDev& t, const void* a, const void* b = nullptr) {
+    return (t.dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15u) == 0) &&
+           ((reinterpret_cast<uintptr_t>(b) & 15u) == 0);
+}
+
+}  // namespace
+
+// ---- launchers -----------------------------------------------------------------------------
+hipError_t launch_fill_u32(u32* p, size_t n, u32 v, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    fill_u32_kernel<<<grid_for(n, BLOCK, 65536), BLOCK, 0, s>>>(p, n, v);
+    return hipGetLastError();
+}
+
+hipError_t launch_snapshot_entry(const TableDev& t, hipStream_t s) {
+    snapshot_entry_kernel<<<1, 1, 0, s>>>(t);
+    return hipGetLastError();
+}
+
+hipError_t launch_pull(const TableDev& t, const u64* keys, size_t n, float* out, uint8_t* hit,
+                       hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const u32 grid = grid_for(n, KEYS_PER_ROUND * (BLOCK / 64), 16384);
+    if (vec4_ok(t, out)) {
+        u32 units = t.dim / 4;
+        pull_kernel<float4><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, reinterpret_cast<float4*>(out),
+                                                   hit, units, t.stride_f / 4, magic32(units));
+    } else {
+        pull_kernel<float><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, out, hit, t.dim, t.stride_f,
+                                                  magic32(t.dim));
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_gather_slots(const TableDev& t, const u32* slot_idx, size_t n, float* out,
+                               uint8_t* hit, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const u32 grid = grid_for(n, KEYS_PER_ROUND * (BLOCK / 64), 16384);
+    if (vec4_ok(t, out)) {
+        u32 units = t.dim / 4;
+        gather_slots_kernel<float4><<<grid, BLOCK, 0, s>>>(t, slot_idx, (u32)n,
+                                                           reinterpret_cast<float4*>(out), hit,
+                                                           units, t.stride_f / 4, magic32(units));
+    } else {
+        gather_slots_kernel<float><<<grid, BLOCK, 0, s>>>(t, slot_idx, (u32)n, out, hit, t.dim,
+                                                          t.stride_f, magic32(t.dim));
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_locate(const TableDev& t, const u64* keys, size_t n, u32* slot_out, u32* idx_out,
+                         bool insert, bool init_rows, bool count_dups, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const u32 grid = grid_for(n, KEYS_PER_ROUND * (BLOCK / 64), 16384);
+    if (insert)
+        locate_kernel<true><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, init_rows,
+                                                   count_dups);
+    else
+        locate_kernel<false><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, 0,
+                                                    count_dups);
+    return hipGetLastError();
+}
+
+hipError_t launch_rollback(const TableDev& t, const u32* slot_idx, size_t n, u32 first_new_row,
+                           hipStream_t s) {
+    rollback_kernel<<<grid_for(n ? n : 1, BLOCK, 1u << 30), BLOCK, 0, s>>>(t, slot_idx, (u32)n,
+                                                                           first_new_row);
+    return hipGetLastError();
+}
+
+hipError_t launch_segreduce_update(const TableDev& t, const u32* sorted_slot, const u32* sorted_idx,
+                                   size_t n, const float* grads, uint4* part_hdr, float* part_val,
+                                   hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const bool v4 = vec4_ok(t, grads, part_val);
+    const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
+    dim3 grid1((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);
+    const u32 fix_waves = (g.n_chunks + g.p - 1) / g.p;
+    dim3 grid2((fix_waves + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);
+    if (v4) {
+        segreduce_kernel<float4><<<grid1, BLOCK, 0, s>>>(
+            t, sorted_slot, sorted_idx, (u32)n, reinterpret_cast<const float4*>(grads), part_hdr,
+            reinterpret_cast<float4*>(part_val), g.units, g.lp, g.p, g.wch, g.n_chunks);
+        fixup_kernel<float4><<<grid2, BLOCK, 0, s>>>(t, part_hdr,
+                                                     reinterpret_cast<const float4*>(part_val),
+                                                     g.units, g.lp, g.p, g.n_chunks);
+    } else {
+        segreduce_kernel<float><<<grid1, BLOCK, 0, s>>>(t, sorted_slot, sorted_idx, (u32)n, grads,
+                                                        part_hdr, part_val, g.units, g.lp, g.p,
+                                                        g.wch, g.n_chunks);
+        fixup_kernel<float><<<grid2, BLOCK, 0, s>>>(t, part_hdr, part_val, g.units, g.lp, g.p,
+                                                    g.n_chunks);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_update_unique(const TableDev& t, const u32* slot_idx, size_t n, const float* grads,
+                                hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const bool v4 = vec4_ok(t, grads);
+    const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
+    dim3 grid(grid_for(n, g.p * (BLOCK / 64), 16384), g.col_blocks);
+    if (v4)
+        update_unique_kernel<float4><<<grid, BLOCK, 0, s>>>(
+            t, slot_idx, (u32)n, reinterpret_cast<const float4*>(grads), g.units, g.lp, g.p);
+    else
+        update_unique_kernel<float><<<grid, BLOCK, 0, s>>>(t, slot_idx, (u32)n, grads, g.units, g.lp,
+                                                           g.p);
+    return hipGetLastError();
+}
+
+hipError_t launch_write_values(const TableDev& t, const u32* slot_idx, size_t n, const float* values,
+                               hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const u64 total = (u64)n * t.vf;
+    write_values_kernel<<<grid_for(total, BLOCK * 4, 65536), BLOCK, 0, s>>>(t, slot_idx, total,
+                                                                            values, magic64(t.vf));
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_records(const TableDev& t, u32 first_row, size_t n, u32* records,
+                               hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const u32 rec_dw = t.vf + 2;
+    const u64 total = (u64)n * rec_dw;
+    pack_records_kernel<<<grid_for(total, BLOCK * 4, 65536), BLOCK, 0, s>>>(
+        t, first_row, total, records, rec_dw, magic64(rec_dw));
+    return hipGetLastError();
+}
+
+hipError_t launch_unpack_records(const u32* records, size_t n, u32 stride_dw, u32 floats_per_rec,
+                                 u64* keys, float* values, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const u32 used = floats_per_rec + 2;
+    const u64 total = (u64)n * used;
+    unpack_records_kernel<<<grid_for(total, BLOCK * 4, 65536), BLOCK, 0, s>>>(
+        records, total, stride_dw, floats_per_rec, reinterpret_cast<u32*>(keys), values,
+        magic64(used));
+    return hipGetLastError();
+}
+
+hipError_t launch_probe_hist(const TableDev& t, u32 n_rows, unsigned long long* hist,
+                             hipStream_t s) {
+    if (n_rows == 0) return hipSuccess;
+    probe_hist_kernel<<<grid_for(n_rows, BLOCK, 65536), BLOCK, 0, s>>>(t, n_rows, hist);
+    return hipGetLastError();
+}
+
+}  // namespace pshbm

@@ -1,0 +1,141 @@
+// Device-side layout of one HBM-resident shard and the launch interface of its kernels.
+//
+// Hash array: `nbuckets` (a power of two) buckets of 4 slots; a slot is 16 bytes
+// {uint64 key, uint32 row, uint32 aux}, so a bucket is one 64-byte line that four lanes read with
+// one dwordx4 load each. A key lives in the first bucket, walking linearly from its home bucket,
+// that had a free slot when it was inserted; buckets never lose keys while inserts run, so a
+// lookup stops at the first bucket that still has an empty slot.
+// Rows: dense slab `rows[row * stride_f]`, `vf` floats used per row (weights then optimizer
+// state), handed out by an atomic counter; `row_keys[row]` is the key that owns the row, which
+// makes Dump / iterate a linear walk of the slab.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pshbm {
+
+constexpr uint64_t KEY_EMPTY = 0xFFFFFFFFFFFFFFFFull;
+constexpr uint64_t KEY_DELETED = 0xFFFFFFFFFFFFFFFEull;
+constexpr uint32_t ROW_NONE = 0xFFFFFFFFu;
+constexpr uint32_t SLOT_NONE = 0xFFFFFFFFu;
+
+// indices into TableDev::counters
+enum {
+    CNT_ROWS = 0,      // rows handed out = keys stored
+    CNT_OVERFLOW = 1,  // set when an insert found no row or no slot
+    CNT_DUP = 2,       // keys that were already present (counted on request)
+    CNT_ENTRY = 3,     // CNT_ROWS as it was when the current pull began
+    CNT_BADKEY = 4,    // reserved keys met in a batch (skipped)
+    CNT_WORDS = 8
+};
+
+struct OptParams {
+    int32_t kind;  // PSHBM_OPT_*
+    float lr, init_acc, alpha, beta, l1, l2;
+};
+
+struct TableDev {
+    uint4* slots;        // nbuckets * 4
+    float* rows;         // max_rows * stride_f
+    uint64_t* row_keys;  // max_rows
+    uint32_t* counters;  // CNT_WORDS
+    uint32_t bucket_mask;
+    uint32_t max_rows;
+    uint32_t dim;       // weights per key
+    uint32_t vf;        // floats per value = dim * (1 + state blocks)
+    uint32_t stride_f;  // floats between rows, multiple of 4
+    OptParams opt;
+};
+
+__host__ __device__ inline uint64_t hash64(uint64_t h) {
+    h ^= h >> 33;
+    h *= 0xff51afd7ed558ccdull;
+    h ^= h >> 33;
+    h *= 0xc4ceb9fe1a85ec53ull;
+    h ^= h >> 33;
+    return h;
+}
+
+// Segment-reduce geometry shared by the kernels and the host that sizes their scratch.
+struct SegGeom {
+    uint32_t units;       // row length in elements of the vector type (dim / vec)
+    uint32_t col_blocks;  // ceil(units / 64)
+    uint32_t lp;          // lanes per position in a full column block
+    uint32_t p;           // positions per wave round
+    uint32_t wch;         // positions per wave chunk
+    uint32_t n_chunks;    // for a batch of n positions
+};
+constexpr uint32_t SEG_ROUNDS = 16;
+
+inline SegGeom seg_geometry(uint32_t dim, uint32_t vec, uint64_t n) {
+    SegGeom g;
+    g.units = dim / vec;
+    g.col_blocks = (g.units + 63) / 64;
+    g.lp = g.units < 64 ? g.units : 64;
+    g.p = 64 / g.lp;
+    g.wch = g.p * SEG_ROUNDS;
+    g.n_chunks = (uint32_t)((n + g.wch - 1) / g.wch);
+    return g;
+}
+
+// ---- launchers (kernels.hip) ---------------------------------------------------------------
+// All enqueue on `s` and return the hipError_t of the launch.
+
+hipError_t launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t s);
+hipError_t launch_snapshot_entry(const TableDev& t, hipStream_t s);
+
+// Fused probe + gather of pull without insertion. out is n x dim floats; hit may be null.
+hipError_t launch_pull(const TableDev& t, const uint64_t* keys, size_t n, float* out, uint8_t* hit,
+                       hipStream_t s);
+
+// slot_out[i] = slot holding keys[i] or SLOT_NONE; idx_out[i] = i when idx_out is not null.
+// insert: claim a slot and a row for each missing key (row initialised when init_rows).
+// count_dups: count keys that were found present or claimed by another lane into CNT_DUP.
+hipError_t launch_locate(const TableDev& t, const uint64_t* keys, size_t n, uint32_t* slot_out,
+                         uint32_t* idx_out, bool insert, bool init_rows, bool count_dups,
+                         hipStream_t s);
+
+// Gather through located slots (pull with insertion); hit = row existed when the pull began.
+hipError_t launch_gather_slots(const TableDev& t, const uint32_t* slot_idx, size_t n, float* out,
+                               uint8_t* hit, hipStream_t s);
+
+// Undo of a batch of claims: every located slot whose row is >= first_new_row (or unset) is
+// emptied, the counters are restored.
+hipError_t launch_rollback(const TableDev& t, const uint32_t* slot_idx, size_t n,
+                           uint32_t first_new_row, hipStream_t s);
+
+// Duplicate aggregation + update over pairs sorted by slot. part_hdr: n_chunks uint4;
+// part_val: n_chunks * 2 * dim floats.
+hipError_t launch_segreduce_update(const TableDev& t, const uint32_t* sorted_slot,
+                                   const uint32_t* sorted_idx, size_t n, const float* grads,
+                                   uint4* part_hdr, float* part_val, hipStream_t s);
+
+// One optimizer step per located key, no aggregation (keys distinct).
+hipError_t launch_update_unique(const TableDev& t, const uint32_t* slot_idx, size_t n,
+                                const float* grads, hipStream_t s);
+
+// rows[slot->row] = values[i] (whole value, vf floats).
+hipError_t launch_write_values(const TableDev& t, const uint32_t* slot_idx, size_t n,
+                               const float* values, hipStream_t s);
+
+// records [first_row, first_row + n) of the slab as {key, vf floats} packed records.
+hipError_t launch_pack_records(const TableDev& t, uint32_t first_row, size_t n, uint32_t* records,
+                               hipStream_t s);
+// the inverse split of packed records into a key array and a value matrix (n x floats_per_rec),
+// record stride in dwords.
+hipError_t launch_unpack_records(const uint32_t* records, size_t n, uint32_t stride_dw,
+                                 uint32_t floats_per_rec, uint64_t* keys, float* values,
+                                 hipStream_t s);
+
+// probe-distance histogram over the stored keys: hist[0..15], hist[16] = max distance.
+hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long long* hist,
+                             hipStream_t s);
+
+// ---- sort (sort.hip) -----------------------------------------------------------------------
+size_t sort_pairs_temp_bytes(size_t n);
+hipError_t sort_pairs(void* temp, size_t temp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
+                      const uint32_t* vals_in, uint32_t* vals_out, size_t n, unsigned end_bit,
+                      hipStream_t s);
+
+}  // namespace pshbm

@@ -1,0 +1,98 @@
+"""Writes tests/golden/reference_known_answers.json: the scenarios of the reference's own tests
+for the sparse-table path, restated as operation lists with the results those tests assert.
+
+Nothing here runs the reference or the oracle: every expected number is the closed form that the
+cited reference test checks (all integer valued). The reference's TestValue{sum,count}
+(pico-ps/test/TestOps.h:53-58) is modelled as a dim-2 row [sum, count] under the SUM optimizer, and
+a push of arg=key (apply_push_arg: sum += arg, count += 1, TestOps.h:98-103) as the gradient
+[key, 1].
+
+Run from the repository root:  python tests/golden/make_reference_known_answers.py
+"""
+import json
+import os
+
+TEST_KEY_NUM = 100  # pico-ps/test/TestOps.h:12
+
+
+def test_sparse(num_process):
+    """pico-ps/test/ps_service_test.cpp:77-184 (test_sparse) on one shard."""
+    ops = []
+    all_keys = []
+    for rank in range(num_process):
+        keys = list(range(rank * TEST_KEY_NUM, (rank + 1) * TEST_KEY_NUM))
+        grads = [[k, 1] for k in keys]
+        all_keys += keys
+        ops.append({"op": "push", "keys": keys, "grads": grads})          # async_push, :104
+        ops.append({"op": "queue", "keys": keys, "grads": grads})         # sync_push, :106
+        if rank % 2 == 0:
+            ops.append({"op": "queue", "keys": keys, "grads": grads})     # even ranks again, :108-111
+    ops.append({"op": "store"})                                           # :120
+    ops.append({"op": "expect_size", "value": TEST_KEY_NUM * num_process})  # :122
+
+    def row(k):
+        count = 2 + (1 if (k // TEST_KEY_NUM) % 2 == 0 else 0)  # TestOps.h:170-172
+        return [k * count, count]
+
+    # dump, load into a new storage, clear, restore (:125-156): same size, same pulls
+    ops.append({"op": "dump_load_roundtrip", "expect_size": TEST_KEY_NUM * num_process})
+    ops.append({"op": "expect_pull", "keys": all_keys, "rows": [row(k) for k in all_keys],
+                "hit": [1] * len(all_keys)})                              # :204-213 (x5: idempotent)
+    ops.append({"op": "expect_pull", "keys": all_keys, "rows": [row(k) for k in all_keys],
+                "hit": [1] * len(all_keys)})
+    # a key that is not stored pulls the default value 0 and is not inserted
+    # (pico-ps/operator/SparsePullOperator.h:307-310; ps_service_test.cpp:176-184 for erased keys)
+    missing = [TEST_KEY_NUM * num_process + i for i in range(10)]
+    ops.append({"op": "expect_pull", "keys": missing, "rows": [[0, 0]] * len(missing),
+                "hit": [0] * len(missing)})
+    ops.append({"op": "expect_size", "value": TEST_KEY_NUM * num_process})
+    ops.append({"op": "clear"})                                           # :153
+    ops.append({"op": "expect_size", "value": 0})                         # :154
+    return {"name": f"test_sparse_{num_process}", "dim": 2, "optimizer": "SUM",
+            "cite": "pico-ps/test/ps_service_test.cpp:77-184, pico-ps/test/TestOps.h:87-136,159-185",
+            "ops": ops}
+
+
+def pmem_three_pushes(num_keys=120):
+    """pico-ps/test/ps_pmem_test.cpp:395-439: key 2k is pushed arg=k three times (async), dumped
+    and loaded; pulling keys 0..NUM_KEYS-1 gives i odd ? 0 : i/2*3."""
+    keys = [2 * k for k in range(num_keys)]
+    grads = [[k, 1] for k in range(num_keys)]
+    ops = [{"op": "push", "keys": keys, "grads": grads} for _ in range(3)]
+    ops.append({"op": "dump_load_roundtrip", "expect_size": num_keys})
+    pull_keys = list(range(num_keys))
+    rows = [[0, 0] if i % 2 else [i // 2 * 3, 3] for i in pull_keys]
+    ops.append({"op": "expect_pull", "keys": pull_keys, "rows": rows,
+                "hit": [0 if i % 2 else 1 for i in pull_keys]})
+    return {"name": "pmem_three_pushes", "dim": 2, "optimizer": "SUM",
+            "cite": "pico-ps/test/ps_pmem_test.cpp:395-439", "ops": ops}
+
+
+def native_ps_roundtrip(num_process=2, per_rank=150):
+    """pico-ps/test/ps_predictor_native_ps_test.cpp:108-170: each key is pushed once with the value
+    (key+1, key+2), dumped, loaded through the in-process path; the pulled value is key+2.
+    (The reference uses 1000 keys per rank; the fixture keeps the stride and fewer keys.)"""
+    ops = []
+    keys = []
+    for rank in range(num_process):
+        ks = list(range(rank * 1000, rank * 1000 + per_rank))
+        keys += ks
+        ops.append({"op": "push", "keys": ks, "grads": [[k + 1, k + 2] for k in ks]})
+    ops.append({"op": "dump_load_roundtrip", "expect_size": len(keys)})
+    for _ in range(2):
+        ops.append({"op": "expect_pull", "keys": keys, "rows": [[k + 1, k + 2] for k in keys],
+                    "hit": [1] * len(keys)})
+    return {"name": "native_ps_roundtrip", "dim": 2, "optimizer": "SUM",
+            "cite": "pico-ps/test/ps_predictor_native_ps_test.cpp:108-170", "ops": ops}
+
+
+def main():
+    scenarios = [test_sparse(1), test_sparse(3), pmem_three_pushes(), native_ps_roundtrip()]
+    out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_known_answers.json")
+    with open(out, "w") as f:
+        json.dump({"scenarios": scenarios}, f, separators=(",", ":"))
+    print(out, os.path.getsize(out), "bytes")
+
+
+if __name__ == "__main__":
+    main()

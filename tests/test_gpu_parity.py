@@ -1,0 +1,324 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI (needs an MI355X).
+
+Bars: pulled rows, hit masks and stored key sets bit-exact; pushed values within 1e-6 relative /
+1e-7 absolute of the oracle (aggregation order differs), and bit-exact wherever every key of a
+batch is distinct or the gradients are integers.
+"""
+import numpy as np
+import pytest
+
+import scenario
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-6, 1e-7
+
+OPTS = {
+    "sum": dict(optimizer=0),
+    "sgd": dict(optimizer=1, lr=0.01),
+    "adagrad": dict(optimizer=2, lr=0.05, init_acc=0.1),
+    "ftrl": dict(optimizer=3, alpha=0.05, beta=1.0, l1=1e-4, l2=1e-5),
+}
+
+
+def pair(ps, orc, dim, opt, capacity=1 << 16, **kw):
+    o = OPTS[opt]
+    t = ps.Table(dim, capacity=capacity, **o, **kw)
+    r = orc.Oracle(dim, capacity=capacity, **o, **kw)
+    return t, r
+
+
+def sorted_dump(b):
+    st, rec = b.dump()
+    assert st == 0
+    return np.sort(rec, order="key")
+
+
+def assert_same_table(t, r, exact):
+    a, b = sorted_dump(t), sorted_dump(r)
+    np.testing.assert_array_equal(a["key"], b["key"])
+    if exact:
+        np.testing.assert_array_equal(a["value"], b["value"])
+    else:
+        np.testing.assert_allclose(a["value"], b["value"], rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("scn", scenario.load_scenarios(), ids=lambda s: s["name"])
+def test_reference_known_answers(ps, scn):
+    scenario.run(scn, lambda dim, opt: ps.Table(dim, opt, capacity=1 << 12))
+
+
+@pytest.mark.parametrize("dim", [1, 3, 4, 8, 16, 64, 128, 260])
+def test_pull_bit_exact(ps, orc, wl, dim):
+    rng = np.random.default_rng(dim)
+    t, r = pair(ps, orc, dim, "sgd", capacity=5000)
+    keys = wl.table_keys_np(0, 3000, seed=dim)
+    vals = rng.normal(0, 0.01, (3000, dim)).astype(np.float32)
+    assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+    assert t.size() == r.size() == 3000
+    # hits, misses and duplicates, in a length that is not a multiple of the wave's 16 keys
+    q = np.concatenate([keys[rng.integers(0, 3000, 777)], wl.fresh_keys_np(rng, 100), keys[:5], keys[:5]])
+    rng.shuffle(q)
+    st, rows, hit = t.pull(q)
+    st2, rows2, hit2 = r.pull(q)
+    assert st == st2 == 0
+    np.testing.assert_array_equal(hit, hit2)
+    np.testing.assert_array_equal(rows.view(np.uint32), rows2.view(np.uint32))
+    assert t.size() == 3000  # a pull without the insert flag never inserts
+    for n in (1, 15, 16, 17):
+        st, rows, hit = t.pull(q[:n])
+        np.testing.assert_array_equal(rows, rows2[:n])
+        np.testing.assert_array_equal(hit, hit2[:n])
+    t.close()
+
+
+def test_pull_empty_and_all_miss(ps, orc):
+    t, r = pair(ps, orc, 8, "sum", capacity=64)
+    st, rows, hit = t.pull(np.array([], np.uint64))
+    assert st == 0 and rows.shape == (0, 8)
+    st, rows, hit = t.pull(np.arange(40, dtype=np.uint64))
+    assert st == 0 and not rows.any() and not hit.any() and t.size() == 0
+    t.close()
+
+
+@pytest.mark.parametrize("dim", [2, 16])
+def test_pull_insert_on_miss(ps, orc, wl, dim):
+    rng = np.random.default_rng(3)
+    t, r = pair(ps, orc, dim, "adagrad", capacity=4000)
+    keys = wl.table_keys_np(0, 1000, seed=9)
+    vals = rng.normal(0, 0.01, (1000, 2 * dim)).astype(np.float32)
+    t.set(keys, vals), r.set(keys, vals)
+    fresh = wl.fresh_keys_np(rng, 300)
+    q = np.concatenate([keys[:200], fresh, fresh[:50], keys[100:150]])
+    rng.shuffle(q)
+    a = t.pull(q, ps.PULL_INSERT_ON_MISS)
+    b = r.pull(q, orc.PULL_INSERT_ON_MISS)
+    assert a[0] == b[0] == 0
+    np.testing.assert_array_equal(a[1], b[1])
+    np.testing.assert_array_equal(a[2], b[2])  # mask against the table at entry; duplicates share it
+    assert t.size() == r.size() == 1300
+    assert_same_table(t, r, exact=True)        # fresh rows: zero weights, accumulator = init_acc
+    a, b = t.pull(q), r.pull(q)
+    np.testing.assert_array_equal(a[2], b[2])
+    assert a[2].all()
+    # a read-only table ignores the flag
+    t2 = ps.Table(dim, capacity=100, read_only=True)
+    st, rows, hit = t2.pull(q[:50], ps.PULL_INSERT_ON_MISS)
+    assert st == 0 and t2.size() == 0
+    t.close(), t2.close()
+
+
+@pytest.mark.parametrize("opt", ["sum", "sgd", "adagrad", "ftrl"])
+@pytest.mark.parametrize("dim", [1, 3, 8, 16, 64, 128, 260])
+def test_push_unique_keys_bit_exact(ps, orc, wl, opt, dim):
+    """With distinct keys there is nothing to aggregate: every value must match bit for bit."""
+    rng = np.random.default_rng(dim * 7 + len(opt))
+    t, r = pair(ps, orc, dim, opt, capacity=4000)
+    keys = wl.table_keys_np(0, 1500, seed=1)
+    for it in range(3):
+        sel = rng.permutation(1500)[: 700 + it]
+        g = rng.normal(0, 1e-2, (sel.size, dim)).astype(np.float32)
+        assert t.push(keys[sel], g) == 0 and r.push(keys[sel], g) == 0
+    assert t.push(keys[:300], g[:300], ps.PUSH_ASSUME_UNIQUE) == 0 and r.push(keys[:300], g[:300]) == 0
+    assert_same_table(t, r, exact=True)
+    t.close()
+
+
+@pytest.mark.parametrize("dim", [1, 2, 3, 16, 64, 260])
+def test_aggregation_exact_with_integer_gradients(ps, orc, dim):
+    """The reference's own test operator: integer sums do not depend on the order of addition
+    (pico-ps/test/TestOps.h:98-117), so heavy duplication must still match bit for bit."""
+    rng = np.random.default_rng(dim)
+    t, r = pair(ps, orc, dim, "sum", capacity=3000)
+    for it in range(4):
+        n = 5000 + 17 * it
+        keys = rng.zipf(1.3, n).astype(np.uint64) % np.uint64(2000)   # a few keys repeat thousands of times
+        g = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+        assert t.push(keys, g) == 0 and r.push(keys, g) == 0
+    assert_same_table(t, r, exact=True)
+    # one key only: a single run spanning every chunk of the segmented reduction
+    keys = np.full(9000, 77, np.uint64)
+    g = rng.integers(-3, 4, (9000, dim)).astype(np.float32)
+    assert t.push(keys, g) == 0 and r.push(keys, g) == 0
+    assert_same_table(t, r, exact=True)
+    t.close()
+
+
+@pytest.mark.parametrize("opt", ["sgd", "adagrad", "ftrl"])
+@pytest.mark.parametrize("dim,s", [(16, 1.05), (64, 1.2), (8, 1.1), (128, 1.1)])
+def test_push_zipf_within_tolerance(ps, orc, wl, opt, dim, s):
+    rng = np.random.default_rng(11)
+    n_table, batch = 20000, 30000
+    t, r = pair(ps, orc, dim, opt, capacity=n_table + 4000)
+    keys = wl.table_keys_np(0, n_table, seed=2)
+    vf = t.value_floats
+    vals = rng.normal(0, 0.01, (n_table, vf)).astype(np.float32)
+    if opt == "adagrad":
+        vals[:, dim:] = 0.1
+    if opt == "ftrl":
+        vals[:, 2 * dim:] = vals[:, dim:2 * dim] ** 2
+    assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+    for step in range(3):
+        q = wl.zipf_batch_np(rng, n_table, s, batch, seed=2)
+        q[:500] = wl.fresh_keys_np(rng, 500)            # insert-on-miss inside a push
+        q[500:600] = q[:100]                            # duplicated fresh keys
+        g = rng.normal(0, 1e-3, (batch, dim)).astype(np.float32)
+        assert t.push(q, g) == 0 and r.push(q, g) == 0
+        st, rows, hit = t.pull(q[:4000])
+        st2, rows2, hit2 = r.pull(q[:4000])
+        np.testing.assert_array_equal(hit, hit2)
+        np.testing.assert_allclose(rows, rows2, rtol=RTOL, atol=ATOL)
+    assert t.size() == r.size()
+    assert_same_table(t, r, exact=False)
+    t.close()
+
+
+def test_push_no_insert_drops_missing_keys(ps, orc, wl):
+    rng = np.random.default_rng(4)
+    t, r = pair(ps, orc, 4, "sgd", capacity=1000)
+    keys = wl.table_keys_np(0, 100, seed=3)
+    t.set(keys, np.zeros((100, 4), np.float32)), r.set(keys, np.zeros((100, 4), np.float32))
+    q = np.concatenate([keys[:50], wl.fresh_keys_np(rng, 50)])
+    g = rng.normal(0, 1, (100, 4)).astype(np.float32)
+    assert t.push(q, g, ps.PUSH_NO_INSERT) == 0 and r.push(q, g, orc.PUSH_NO_INSERT) == 0
+    assert t.size() == 100
+    assert_same_table(t, r, exact=True)
+    t.close()
+
+
+def test_capacity_is_all_or_nothing(ps, orc):
+    t, r = pair(ps, orc, 2, "sum", capacity=8)
+    keys = np.arange(6, dtype=np.uint64)
+    ones = lambda n: np.ones((n, 2), np.float32)
+    assert t.push(keys, ones(6)) == 0 and r.push(keys, ones(6)) == 0
+    for b in (t, r):
+        assert b.push(np.array([0, 1, 10, 11, 12], np.uint64), ones(5)) == 3
+        assert b.pull(np.array([20, 21, 22], np.uint64), 1)[0] == 3
+        assert b.set(np.array([30, 31, 32], np.uint64), ones(3)) == 3
+    assert "capacity" in t.last_error()
+    assert_same_table(t, r, exact=True)
+    for b in (t, r):
+        assert b.push(np.array([0, 10, 11, 10], np.uint64), ones(4)) == 0
+        assert b.size() == 8
+        assert b.push(keys, ones(6)) == 0                      # present keys always fit
+        assert b.push(np.array([99], np.uint64), ones(1)) == 3
+    assert_same_table(t, r, exact=True)
+    # the table keeps working after refusals: missing keys pull zeros
+    st, rows, hit = t.pull(np.array([10, 12, 99], np.uint64))
+    np.testing.assert_array_equal(hit, [1, 0, 0])
+    t.close()
+
+
+def test_sync_push_and_store(ps, orc, wl):
+    rng = np.random.default_rng(6)
+    t, r = pair(ps, orc, 8, "sgd", capacity=4000)
+    for _ in range(5):
+        k = rng.integers(0, 900, 1000).astype(np.uint64)
+        g = rng.normal(0, 1e-3, (1000, 8)).astype(np.float32)
+        assert t.queue(k, g) == 0 and r.queue(k, g) == 0
+    assert t.size() == 0 and t.queued() == r.queued() == 5000
+    assert t.store() == 0 and r.store() == 0
+    assert t.queued() == 0
+    assert_same_table(t, r, exact=False)
+    assert t.store() == 0   # nothing queued: a plain acknowledgement
+    t.close()
+
+
+def test_push_pairs_wire_layout(ps, orc):
+    rng = np.random.default_rng(8)
+    t, r = pair(ps, orc, 6, "sgd", capacity=1000)
+    pairs = np.zeros(300, dtype=np.dtype([("key", "<u8"), ("value", "<f4", (6,))]))
+    pairs["key"] = rng.permutation(1000)[:300]
+    pairs["value"] = rng.normal(0, 1, (300, 6))
+    assert t.push_pairs(pairs) == 0 and r.push(pairs["key"], pairs["value"]) == 0
+    assert_same_table(t, r, exact=True)
+    t.close()
+
+
+@pytest.mark.parametrize("opt,dim", [("sgd", 16), ("ftrl", 8), ("adagrad", 128)])
+def test_dump_load_iterate_roundtrip(ps, orc, wl, opt, dim):
+    rng = np.random.default_rng(12)
+    n = 90000 if dim == 128 else 20000       # 90000 x 1032 B = 3 staging chunks
+    t, r = pair(ps, orc, dim, opt, capacity=n + 10)
+    keys = wl.table_keys_np(0, n, seed=5)
+    vals = rng.normal(0, 0.01, (n, t.value_floats)).astype(np.float32)
+    assert t.set(keys, vals) == 0
+    rec = sorted_dump(t)
+    order = np.argsort(keys)
+    np.testing.assert_array_equal(rec["key"], keys[order])
+    np.testing.assert_array_equal(rec["value"], vals[order])
+    # iterate in slices reproduces the dump, a short slice marks the end
+    st, whole = t.dump()
+    got, off = [], 0
+    while True:
+        st, part = t.iterate(off, 7001)
+        assert st == 0
+        got.append(part.copy())
+        off += part.size
+        if part.size < 7001:
+            break
+    np.testing.assert_array_equal(np.concatenate(got), whole)
+    # load into a new table; restore semantics refuse keys that are already there
+    t2 = ps.Table(dim, capacity=n + 10, **OPTS[opt])
+    assert t2.load(whole, ps.LOAD_UNIQUE) == 0
+    np.testing.assert_array_equal(sorted_dump(t2), rec)
+    assert t2.load(whole[:10], ps.LOAD_UNIQUE) == ps.ERROR
+    assert t2.load(whole[:10]) == 0 and t2.size() == n
+    assert t2.clear() == 0 and t2.size() == 0
+    st, rows, hit = t2.pull(keys[:100])
+    assert not hit.any()
+    assert t2.load(whole[:100], ps.LOAD_UNIQUE) == 0 and t2.size() == 100
+    t.close(), t2.close()
+
+
+def test_reserved_keys_and_stats(ps, orc, wl):
+    t, r = pair(ps, orc, 4, "sum", capacity=20000, max_load_factor=0.8)
+    bad = np.array([1, 0xFFFFFFFFFFFFFFFF], np.uint64)
+    assert t.push(bad, np.ones((2, 4), np.float32)) == ps.ERROR
+    assert t.pull(bad)[0] == ps.ERROR and t.size() == 0
+    keys = wl.table_keys_np(0, 20000, seed=7)
+    assert t.set(keys, np.zeros((20000, 4), np.float32)) == 0
+    s = t.stats()
+    assert s.size == 20000 and s.capacity == 20000 and s.slots == 32768
+    assert sum(s.probe_hist) == 20000 and s.probe_hist[0] > 15000
+    assert abs(s.load_factor - 20000 / 32768) < 1e-9
+    assert t.memory_usage() == s.memory_usage == 32768 * 16 + 20000 * (16 + 8)
+    t.close()
+
+
+def test_device_pointer_entry_points(ps, orc, wl):
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(21)
+    dim, n_table, batch = 16, 50000, 40000
+    t, r = pair(ps, orc, dim, "sgd", capacity=n_table + batch)
+    keys = wl.table_keys_np(0, n_table, seed=4)
+    vals = rng.normal(0, 0.01, (n_table, dim)).astype(np.float32)
+    dk = torch.from_numpy(keys.view(np.int64)).cuda()
+    dv = torch.from_numpy(vals).cuda()
+    stream = torch.cuda.current_stream().cuda_stream
+    assert t.set_dev(dk.data_ptr(), dv.data_ptr(), n_table, stream) == 0
+    assert r.set(keys, vals) == 0
+    q = wl.zipf_batch_np(rng, n_table, 1.05, batch, seed=4)
+    g = rng.normal(0, 1e-3, (batch, dim)).astype(np.float32)
+    dq = torch.from_numpy(q.view(np.int64)).cuda()
+    dg = torch.from_numpy(g).cuda()
+    out = torch.empty(batch, dim, device="cuda")
+    hit = torch.empty(batch, dtype=torch.uint8, device="cuda")
+    for step in range(2):
+        assert t.pull_dev(dq.data_ptr(), batch, out.data_ptr(), hit.data_ptr(), 0, stream) == 0
+        assert t.push_dev(dq.data_ptr(), dg.data_ptr(), batch, 0, stream) == 0
+        torch.cuda.synchronize()
+        st, rows, h = r.pull(q)
+        np.testing.assert_allclose(out.cpu().numpy(), rows, rtol=RTOL, atol=ATOL)
+        assert hit.all()
+        assert r.push(q, g) == 0
+    # queue_dev / store_dev on another stream: the table orders itself across streams
+    s2 = torch.cuda.Stream()
+    assert t.queue_dev(dq.data_ptr(), dg.data_ptr(), batch, s2.cuda_stream) == 0
+    assert t.store_dev(0, s2.cuda_stream) == 0
+    assert t.pull_dev(dq.data_ptr(), batch, out.data_ptr(), None, 0, stream) == 0
+    torch.cuda.synchronize()
+    assert r.queue(q, g) == 0 and r.store() == 0
+    np.testing.assert_allclose(out.cpu().numpy(), r.pull(q)[1], rtol=RTOL, atol=ATOL)
+    assert_same_table(t, r, exact=False)
+    t.close()
