@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-table hot path on one MI355X.
+
+A step = one pull of a key batch followed by one push of gradients for the same batch, both
+through the device-pointer C ABI with every input already resident in HBM. The default workload
+is BASELINE.json's configs[1] ("c2": 100M uint64 keys, dim-16 fp32 rows, plain SGD lr 0.01, 1M-key
+Zipf(1.05) batches, duplicates summed before the update).
+
+Prints ONE JSON line: metric/value (pulled + pushed keys per second), the roofline of the kernel
+that takes the most time, and the same workload timed on the host CPU with the oracle.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+CONFIGS = {
+    # name: table keys, dim, optimizer kwargs, batch, zipf s, fresh fraction, grad sigma
+    "c1": dict(n=1_000_000, dim=8, opt=dict(optimizer=1, lr=0.01), batch=65_536, s=None, fresh=0.0,
+               sigma=1e-3, pull_only=True,
+               desc="C1: 1M keys dim8, pull only, 65536-key uniform batches"),
+    "c2": dict(n=100_000_000, dim=16, opt=dict(optimizer=1, lr=0.01), batch=1_000_000, s=1.05,
+               fresh=0.0, sigma=1e-3, pull_only=False,
+               desc="C2: 100M keys dim16 SGD lr0.01, pull+push of 1M-key Zipf(1.05) batches"),
+    "c3": dict(n=50_000_000, dim=64, opt=dict(optimizer=2, lr=0.05, init_acc=0.1), batch=2_000_000,
+               s=1.2, fresh=0.0, sigma=1e-3, pull_only=False,
+               desc="C3: 50M keys dim64 Adagrad, pull+push of 2M-key Zipf(1.2) batches"),
+    "c4": dict(n=500_000_000, dim=8, opt=dict(optimizer=3, alpha=0.05, beta=1.0, l1=1e-4, l2=1e-5),
+               batch=4_000_000, s=1.1, fresh=0.05, sigma=1e-2, pull_only=False,
+               desc="C4: 500M keys dim8 FTRL, pull+push of 4M-key batches (95% Zipf(1.1), 5% fresh)"),
+    "c5": dict(n=200_000_000, dim=128, opt=dict(optimizer=2, lr=0.05, init_acc=0.1), batch=4_000_000,
+               s=1.1, fresh=0.0, sigma=1e-3, pull_only=False,
+               desc="C5: 200M keys dim128 Adagrad, pull+push of 4M-key Zipf(1.1) batches"),
+}
+STATE_BLOCKS = {0: 1, 1: 1, 2: 2, 3: 3}
+
+
+def algorithmic_bytes(cfg, phase, k, u):
+    """Bytes of keys, gradients, rows and state one launch must move (probe, sort and scratch
+    traffic excluded): k = keys in the batch, u = distinct keys."""
+    d4 = 4 * cfg["dim"]
+    r = d4 * STATE_BLOCKS[cfg["opt"]["optimizer"]]
+    if phase == "pull":
+        return k * (8 + d4 + d4)            # key, row read (weights), response write
+    if phase == "locate":
+        return k * 8                        # key read
+    if phase == "segreduce":
+        return k * d4 + u * 2 * r           # gradient read, row+state read and write
+    return 0                                # sort, fixup: pure overhead
+
+
+def build_table(ps, wl, torch, cfg, n_table, seed=0):
+    dim = cfg["dim"]
+    cap = n_table + max(n_table // 4, 32 * cfg["batch"])
+    t = ps.Table(dim, capacity=cap, max_batch=cfg["batch"], **cfg["opt"])
+    vf = t.value_floats
+    stream = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    chunk = 4_000_000
+    for start in range(0, n_table, chunk):
+        cnt = min(chunk, n_table - start)
+        keys = wl.table_keys_torch(start, cnt, seed=seed)
+        vals = torch.randn(cnt, vf, device="cuda", generator=gen) * 0.01
+        if cfg["opt"]["optimizer"] == 2:
+            vals[:, dim:] = cfg["opt"]["init_acc"]
+        if cfg["opt"]["optimizer"] == 3:   # self-consistent FTRL state: n = z^2
+            vals[:, 2 * dim:] = vals[:, dim:2 * dim] ** 2
+        st = t.set_dev(keys.data_ptr(), vals.data_ptr(), cnt, stream)
+        if st != 0:
+            raise RuntimeError(f"set_dev failed: {st} {t.last_error()}")
+        torch.cuda.synchronize()
+    assert t.size() == n_table, (t.size(), n_table)
+    return t
+
+
+def make_batches(wl, torch, cfg, n_table, n_batches, seed=0):
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(2)
+    out = []
+    for b in range(n_batches):
+        k = cfg["batch"]
+        if cfg["s"] is None:
+            idx = torch.randint(0, n_table, (k,), device="cuda", generator=gen)
+            keys = wl.keys_of_index_torch(idx, seed)
+        else:
+            keys = wl.zipf_batch_torch(gen, n_table, cfg["s"], k, seed=seed)
+        nf = int(k * cfg["fresh"])
+        if nf:
+            fresh = torch.randint(0, 1 << 62, (nf,), device="cuda", generator=gen) * 2 + 1
+            pos = torch.randperm(k, device="cuda", generator=gen)[:nf]
+            keys[pos] = fresh
+        grads = torch.randn(k, cfg["dim"], device="cuda", generator=gen) * cfg["sigma"]
+        out.append((keys.contiguous(), grads.contiguous(), int(torch.unique(keys).numel())))
+    return out
+
+
+def run_steps(t, torch, cfg, batches, out, steps, first=0):
+    stream = torch.cuda.current_stream().cuda_stream
+    k = cfg["batch"]
+    for i in range(first, first + steps):
+        keys, grads, _ = batches[i % len(batches)]
+        st = t.pull_dev(keys.data_ptr(), k, out.data_ptr(), None, 0, stream)
+        if st == 0 and not cfg["pull_only"]:
+            st = t.push_dev(keys.data_ptr(), grads.data_ptr(), k, 0, stream)
+        if st != 0:
+            raise RuntimeError(f"step {i} failed: {st} {t.last_error()}")
+
+
+def cpu_baseline(cfg, wl, budget_keys):
+    """The oracle (a scalar port of the reference's operator loops) on a bounded sample of the same
+    workload: a table of budget_keys keys and a few batches of the configured size, one thread."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import oracle
+    n = min(cfg["n"], budget_keys)
+    dim, k = cfg["dim"], cfg["batch"]
+    o = oracle.Oracle(dim, capacity=n + 8 * k, **cfg["opt"])
+    vf = o.value_floats
+    rng = np.random.default_rng(1)
+    chunk = 1_000_000
+    for start in range(0, n, chunk):
+        cnt = min(chunk, n - start)
+        vals = (rng.standard_normal((cnt, vf), dtype=np.float32) * np.float32(0.01))
+        if cfg["opt"]["optimizer"] == 2:
+            vals[:, dim:] = cfg["opt"]["init_acc"]
+        if cfg["opt"]["optimizer"] == 3:
+            vals[:, 2 * dim:] = vals[:, dim:2 * dim] ** 2
+        assert o.set(wl.table_keys_np(start, cnt, seed=0), vals) == 0
+    steps, times = 4, []
+    for s in range(steps):
+        if cfg["s"] is None:
+            keys = wl.keys_of_index_np(rng.integers(0, n, k), 0)
+        else:
+            keys = wl.zipf_batch_np(rng, n, cfg["s"], k, seed=0)
+        grads = rng.standard_normal((k, dim), dtype=np.float32) * np.float32(cfg["sigma"])
+        t0 = time.perf_counter()
+        st, rows, hit = o.pull(keys)
+        if not cfg["pull_only"]:
+            assert o.push(keys, grads) == 0
+        times.append(time.perf_counter() - t0)
+    per_step = sorted(times[1:])[len(times[1:]) // 2]   # first step warms the caches
+    keys_per_step = k * (1 if cfg["pull_only"] else 2)
+    o.close()
+    return {
+        "value": keys_per_step / per_step, "unit": "keys/s", "cores": 1, "kind": "port",
+        "sample": f"{n}-key table (of {cfg['n']}), median of {steps - 1} steps of {k}-key batches, "
+                  f"oracle/ps_oracle.cpp single thread",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--table-keys", type=int, default=0, help="override the table size (testing)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-keys", type=int, default=10_000_000, help="table size of the CPU sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    import torch
+    ps = importlib.import_module("parameter-server_amd")
+    wl = importlib.import_module("parameter-server_amd.workload")
+    ps.lib()  # fails loudly if the HIP library has not been built
+    cfg = dict(CONFIGS[args.config])
+    n_table = args.table_keys or cfg["n"]
+    torch.cuda.set_device(0)
+
+    t = build_table(ps, wl, torch, cfg, n_table)
+    batches = make_batches(wl, torch, cfg, n_table, n_batches=8)
+    out = torch.empty(cfg["batch"], cfg["dim"], device="cuda")
+    k = cfg["batch"]
+    keys_per_step = k * (1 if cfg["pull_only"] else 2)
+
+    # timed region: W warm-up steps, then exactly K steps between two device synchronisations
+    run_steps(t, torch, cfg, batches, out, args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_steps(t, torch, cfg, batches, out, args.steps, first=args.warmup)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = keys_per_step * args.steps / elapsed
+
+    # the same K steps again with HIP events around every kernel launch (on the launch stream)
+    t.profile_enable(True)
+    run_steps(t, torch, cfg, batches, out, args.steps, first=args.warmup)
+    torch.cuda.synchronize()
+    prof = t.profile_read()
+    t.profile_enable(False)
+    u_mean = sum(b[2] for b in batches) / len(batches)
+    phases = {}
+    for name, (ms, launches) in prof.items():
+        if launches:
+            avg_ms = ms / launches
+            by = algorithmic_bytes(cfg, name, k, u_mean)
+            phases[name] = {"avg_ms": round(avg_ms, 5), "launches": int(launches),
+                            "algorithmic_GBps": round(by / avg_ms / 1e6, 1)}
+    dominant = max(phases, key=lambda p: phases[p]["avg_ms"])
+    achieved = phases[dominant]["algorithmic_GBps"]
+    roofline = {"kernel": dominant, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "avg_ms": phases[dominant]["avg_ms"]}
+    step_bytes = sum(algorithmic_bytes(cfg, p, k, u_mean) for p in ("pull",) if True)
+    if not cfg["pull_only"]:
+        step_bytes += algorithmic_bytes(cfg, "locate", k, u_mean) + algorithmic_bytes(cfg, "segreduce", k, u_mean)
+
+    result = {
+        "metric": "pulled+pushed keys/sec on 1 MI355X; achieved HBM GB/s as % of peak",
+        "value": value, "unit": "keys/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": cfg["desc"], "table_keys": n_table, "batch": k, "dim": cfg["dim"],
+                   "unique_keys_per_batch": round(u_mean)},
+        "step_algorithmic_GBps": round(step_bytes / (ms_per_step * 1e6), 1),
+        "step_frac_of_hbm_peak": round(step_bytes / (ms_per_step * 1e6) / HBM_PEAK_GBS, 4),
+        "roofline": roofline,
+        "phases": phases,
+    }
+    t.close()
+    del out, batches
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg, wl, args.cpu_keys)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -193,6 +193,26 @@ int32_t pshbm_memory_usage(pshbm_table* t, uint64_t* bytes);
  * (pico-ps/operator/StorageOperator.h:27-38,123-141). */
 int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out);
 
+/* Per-kernel timing. While enabled, every kernel launch of a pull or push is bracketed by HIP
+ * events on the stream it runs on; pshbm_profile_read waits for them, returns the milliseconds and
+ * launch counts accumulated per phase since the last read, and starts over. The counterpart of the
+ * VTIMER scopes at the top of the reference's operator halves (SparsePullOperator.h:160,
+ * SparsePushOperator.h:202,328). Costs two event records per launch; leave it off in production. */
+#define PSHBM_PHASE_PULL 0          /* fused probe + gather of a pull */
+#define PSHBM_PHASE_LOCATE 1        /* probe (+ claim) of a push, a set or an inserting pull */
+#define PSHBM_PHASE_SORT 2          /* (slot, index) radix sort */
+#define PSHBM_PHASE_SEGREDUCE 3     /* duplicate aggregation + update inside wave chunks */
+#define PSHBM_PHASE_FIXUP 4         /* runs that cross chunk borders */
+#define PSHBM_PHASE_UPDATE_UNIQUE 5 /* update of a batch declared duplicate-free */
+#define PSHBM_PHASE_GATHER 6        /* row gather of an inserting pull */
+#define PSHBM_PHASES 8
+typedef struct pshbm_profile {
+    double ms[PSHBM_PHASES];
+    uint64_t launches[PSHBM_PHASES];
+} pshbm_profile;
+int32_t pshbm_profile_enable(pshbm_table* t, int32_t on);
+int32_t pshbm_profile_read(pshbm_table* t, pshbm_profile* out);
+
 /* Pinned host memory for request/response buffers of the host-pointer entry points. */
 int32_t pshbm_host_alloc(void** p, size_t bytes);
 int32_t pshbm_host_free(void* p);

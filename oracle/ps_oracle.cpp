@@ -45,6 +45,10 @@ constexpr uint64_t KEY_DELETED = 0xFFFFFFFFFFFFFFFEull;
 enum { ST_OK = 0, ST_INVALID_CONFIG = 1, ST_OOM = 3, ST_ERROR = 10 };  // Status.h:15-29
 enum { OPT_SUM = 0, OPT_SGD = 1, OPT_ADAGRAD = 2, OPT_FTRL = 3 };
 enum { PULL_INSERT_ON_MISS = 1u, PUSH_NO_INSERT = 1u, LOAD_UNIQUE = 1u };
+// Oracle-only push flag: sum duplicates in float64 and round once. This is not what the reference
+// computes; it is the exactly rounded sum, against which tests judge which of two fp32 summation
+// orders (the reference's sequential one, the kernels' tree) is closer for heavily repeated keys.
+enum { PUSH_EXACT_AGGREGATION = 0x100u };
 
 struct Config {
     uint32_t dim;
@@ -149,21 +153,30 @@ uint32_t append_row(Oracle& o, uint64_t key) {
 // -> apply_push_arg adds each occurrence in input order. Unique keys come out in first-occurrence
 // order (the reference's wire order is EasyHashMap bucket order, which fixes no value).
 void aggregate(uint32_t dim, const uint64_t* keys, const float* grads, size_t n,
-               std::vector<uint64_t>& ukeys, std::vector<float>& usum) {
+               std::vector<uint64_t>& ukeys, std::vector<float>& usum, bool exact = false) {
     std::unordered_map<uint64_t, size_t> whole_map;
     whole_map.reserve(n * 2);
     ukeys.clear();
     usum.clear();
+    std::vector<double> dsum;  // exact mode only
     for (size_t i = 0; i < n; ++i) {
         auto rit = whole_map.try_emplace(keys[i], ukeys.size());
         if (rit.second) {
             ukeys.push_back(keys[i]);
             usum.resize(usum.size() + dim, 0.0f);
+            if (exact) dsum.resize(dsum.size() + dim, 0.0);
         }
-        float* acc = &usum[rit.first->second * dim];
         const float* g = grads + i * dim;
-        for (uint32_t j = 0; j < dim; ++j) acc[j] = acc[j] + g[j];
+        if (exact) {
+            double* acc = &dsum[rit.first->second * dim];
+            for (uint32_t j = 0; j < dim; ++j) acc[j] += (double)g[j];
+        } else {
+            float* acc = &usum[rit.first->second * dim];
+            for (uint32_t j = 0; j < dim; ++j) acc[j] = acc[j] + g[j];
+        }
     }
+    if (exact)
+        for (size_t k = 0; k < dsum.size(); ++k) usum[k] = (float)dsum[k];
 }
 
 // The per-item loop of apply_async_push_request, SparsePushOperator.h:245-268, over unique items.
@@ -279,7 +292,7 @@ int32_t pso_push(void* h, const uint64_t* keys, const float* grads, size_t n, ui
         if (reserved(keys[i])) return ST_ERROR;
     std::vector<uint64_t> uk;
     std::vector<float> us;
-    aggregate(o.c.dim, keys, grads, n, uk, us);
+    aggregate(o.c.dim, keys, grads, n, uk, us, (flags & PUSH_EXACT_AGGREGATION) != 0);
     return apply_unique(o, uk, us, flags);
 }
 

@@ -31,8 +31,9 @@ SYMBOLS = [
     "pshbm_queue", "pshbm_queue_dev", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
     "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
-    "pshbm_host_alloc", "pshbm_host_free",
+    "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
+PHASES = ["pull", "locate", "sort", "segreduce", "fixup", "update_unique", "gather"]
 
 
 class Config(C.Structure):
@@ -66,6 +67,10 @@ class Stats(C.Structure):
     ]
 
 
+class Profile(C.Structure):
+    _fields_ = [("ms", C.c_double * 8), ("launches", C.c_uint64 * 8)]
+
+
 class PshbmError(RuntimeError):
     def __init__(self, status, message):
         super().__init__(f"pshbm status {status}: {message}")
@@ -93,6 +98,13 @@ def lib():
             raise FileNotFoundError(
                 f"{LIB_PATH} is missing: build it with __graft_entry__.build() "
                 f"(make -C {CSRC}); there is no CPU fallback")
+        # PyTorch wheels bundle their own HIP runtime under the same SONAME. A process must hold
+        # one runtime only (streams and device pointers are handed between torch and this
+        # library), and whichever loads first wins: let torch load first when it is installed.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = C.CDLL(LIB_PATH)
         vp, sz, u32, i32 = C.c_void_p, C.c_size_t, C.c_uint32, C.c_int32
         L.pshbm_create.argtypes = [C.POINTER(Config), C.POINTER(vp)]
@@ -122,6 +134,8 @@ def lib():
         L.pshbm_get_stats.argtypes = [vp, C.POINTER(Stats)]
         L.pshbm_host_alloc.argtypes = [C.POINTER(vp), sz]
         L.pshbm_host_free.argtypes = [vp]
+        L.pshbm_profile_enable.argtypes = [vp, i32]
+        L.pshbm_profile_read.argtypes = [vp, C.POINTER(Profile)]
         for name in SYMBOLS:
             if getattr(L, name).restype is C.c_int:
                 getattr(L, name).restype = i32
@@ -253,6 +267,17 @@ class Table:
         if st != OK:
             raise PshbmError(st, self.last_error())
         return s
+
+    def profile_enable(self, on=True):
+        return lib().pshbm_profile_enable(self._h, int(on))
+
+    def profile_read(self):
+        """{phase: (total ms, launches)} since the last read."""
+        p = Profile()
+        st = lib().pshbm_profile_read(self._h, C.byref(p))
+        if st != OK:
+            raise PshbmError(st, self.last_error())
+        return {name: (p.ms[i], p.launches[i]) for i, name in enumerate(PHASES)}
 
     # -- device-pointer entry points (pointers and stream as integers)
     def pull_dev(self, d_keys, n, d_out, d_hit=None, flags=0, stream=0):

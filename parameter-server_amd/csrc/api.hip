@@ -10,6 +10,7 @@
 #include <new>
 #include <shared_mutex>
 #include <string>
+#include <vector>
 
 #include "table.h"
 
@@ -66,6 +67,11 @@ struct pshbm_table {
     std::shared_mutex mu;
     uint64_t size_bound = 0;  // upper bound of the rows handed out
     std::string err;
+
+    // optional per-kernel timing (pshbm_profile_*)
+    bool prof_on = false;
+    std::vector<hipEvent_t> prof_ev;  // start/stop pairs
+    std::vector<int> prof_phase;      // phase of each pair in use
 };
 
 namespace {
@@ -102,11 +108,37 @@ int32_t hip_fail(pshbm_table* t, hipError_t e, const char* what) {
         if (e__ != hipSuccess) return hip_fail((t), e__, #expr);      \
     } while (0)
 
+// Times `expr` (a kernel launch on stream s) as `phase` when profiling is on.
+#define HIP_TRY_PROF(t, s, phase, expr)                               \
+    do {                                                              \
+        prof_begin((t), (s), (phase));                                \
+        hipError_t e__ = (expr);                                      \
+        prof_end((t), (s));                                           \
+        if (e__ != hipSuccess) return hip_fail((t), e__, #expr);      \
+    } while (0)
+
 #define ST_TRY(expr)                          \
     do {                                      \
         int32_t s__ = (expr);                 \
         if (s__ != PSHBM_OK) return s__;      \
     } while (0)
+
+void prof_begin(pshbm_table* t, hipStream_t s, int phase) {
+    if (!t->prof_on) return;
+    const size_t k = t->prof_phase.size();
+    while (t->prof_ev.size() < 2 * (k + 1)) {
+        hipEvent_t e = nullptr;
+        if (hipEventCreate(&e) != hipSuccess) return;
+        t->prof_ev.push_back(e);
+    }
+    t->prof_phase.push_back(phase);
+    (void)hipEventRecord(t->prof_ev[2 * k], s);
+}
+
+void prof_end(pshbm_table* t, hipStream_t s) {
+    if (!t->prof_on || t->prof_phase.empty()) return;
+    (void)hipEventRecord(t->prof_ev[2 * (t->prof_phase.size() - 1) + 1], s);
+}
 
 int32_t ensure(pshbm_table* t, DevBuf& b, size_t bytes) {
     if (bytes <= b.bytes) return PSHBM_OK;
@@ -214,18 +246,22 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
     if (insert) ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
     uint32_t* idx = static_cast<uint32_t*>(t->ws_idx.p);
-    HIP_TRY(t, launch_locate(t->d, d_keys, n, slot, unique ? nullptr : idx, insert, true, false, s));
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE,
+                 launch_locate(t->d, d_keys, n, slot, unique ? nullptr : idx, insert, true, false, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
     if (unique) {
-        HIP_TRY(t, launch_update_unique(t->d, slot, n, d_grads, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_UPDATE_UNIQUE, launch_update_unique(t->d, slot, n, d_grads, s));
     } else {
         uint32_t* sslot = static_cast<uint32_t*>(t->ws_sslot.p);
         uint32_t* sidx = static_cast<uint32_t*>(t->ws_sidx.p);
-        HIP_TRY(t, sort_pairs(t->ws_sort.p, t->ws_sort.bytes, slot, sslot, idx, sidx, n,
-                              t->slot_bits + 1, s));
-        HIP_TRY(t, launch_segreduce_update(t->d, sslot, sidx, n, d_grads,
-                                           static_cast<uint4*>(t->ws_hdr.p),
-                                           static_cast<float*>(t->ws_pval.p), s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT,
+                     sort_pairs(t->ws_sort.p, t->ws_sort.bytes, slot, sslot, idx, sidx, n,
+                                t->slot_bits + 1, s));
+        uint4* hdr = static_cast<uint4*>(t->ws_hdr.p);
+        float* pval = static_cast<float*>(t->ws_pval.p);
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_SEGREDUCE,
+                     launch_segreduce(t->d, sslot, sidx, n, d_grads, hdr, pval, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP, launch_fixup(t->d, n, d_grads, hdr, pval, s));
     }
     return PSHBM_OK;
 }
@@ -278,6 +314,7 @@ void destroy_impl(pshbm_table* t) {
     if (t->h_counters) (void)hipHostFree(t->h_counters);
     if (t->h_hist) (void)hipHostFree(t->h_hist);
     if (t->order_ev) (void)hipEventDestroy(t->order_ev);
+    for (hipEvent_t e : t->prof_ev) (void)hipEventDestroy(e);
     if (t->stream) (void)hipStreamDestroy(t->stream);
     if (t->side) (void)hipStreamDestroy(t->side);
     delete t;
@@ -412,7 +449,7 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     std::unique_lock<std::shared_mutex> lk(t->mu);
     ST_TRY(begin_op(t, s));
     if (!insert) {
-        HIP_TRY(t, launch_pull(t->d, d_keys, n, d_out_rows, d_hit, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_PULL, launch_pull(t->d, d_keys, n, d_out_rows, d_hit, s));
         return PSHBM_OK;
     }
     ST_TRY(ensure_workspace(t, n));
@@ -421,9 +458,10 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
     HIP_TRY(t, launch_snapshot_entry(t->d, s));
-    HIP_TRY(t, launch_locate(t->d, d_keys, n, slot, nullptr, true, true, false, s));
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE,
+                 launch_locate(t->d, d_keys, n, slot, nullptr, true, true, false, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
-    HIP_TRY(t, launch_gather_slots(t->d, slot, n, d_out_rows, d_hit, s));
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_GATHER, launch_gather_slots(t->d, slot, n, d_out_rows, d_hit, s));
     return PSHBM_OK;
 }
 
@@ -810,6 +848,30 @@ int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out) {
     out->load_factor = (double)rows / (double)(t->nbuckets * 4);
     for (int i = 0; i < 16; ++i) out->probe_hist[i] = t->h_hist[i];
     out->max_probe = t->h_hist[16];
+    return PSHBM_OK;
+}
+
+int32_t pshbm_profile_enable(pshbm_table* t, int32_t on) {
+    if (!t) return PSHBM_INVALID_ID;
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    t->prof_on = on != 0;
+    return PSHBM_OK;
+}
+
+int32_t pshbm_profile_read(pshbm_table* t, pshbm_profile* out) {
+    if (!t || !out) return PSHBM_INVALID_ID;
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    std::memset(out, 0, sizeof *out);
+    for (size_t k = 0; k < t->prof_phase.size(); ++k) {
+        HIP_TRY(t, hipEventSynchronize(t->prof_ev[2 * k + 1]));
+        float ms = 0.f;
+        HIP_TRY(t, hipEventElapsedTime(&ms, t->prof_ev[2 * k], t->prof_ev[2 * k + 1]));
+        const int ph = t->prof_phase[k];
+        out->ms[ph] += ms;
+        out->launches[ph] += 1;
+    }
+    t->prof_phase.clear();
     return PSHBM_OK;
 }
 

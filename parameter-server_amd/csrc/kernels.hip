@@ -432,32 +432,65 @@ __global__ __launch_bounds__(BLOCK) void segreduce_kernel(
                                  r_present ? 1u : 0u);
 }
 
-// Joins the partial sums of runs that cross chunk borders: the lane group of the chunk where a
-// run leaves to the right walks the following chunks' left entries until the run ends, then
-// applies the step. The order of the additions is fixed by the chunk order, so results repeat.
+__device__ __forceinline__ float vshfl_down(float v, u32 d) { return __shfl_down(v, d); }
+__device__ __forceinline__ float4 vshfl_down(float4 v, u32 d) {
+    return make_float4(__shfl_down(v.x, d), __shfl_down(v.y, d), __shfl_down(v.z, d),
+                       __shfl_down(v.w, d));
+}
+
+// Joins the partial sums of runs that cross chunk borders. One wavefront per chunk: if a run
+// leaves that chunk to the right, the wavefront finds where the run ends (the first following
+// chunk whose left entry is marked as the run's end), its P lane groups add the left entries of
+// the chunks in between in a strided fashion, a shuffle tree joins the P sums, and group 0
+// applies the step. The order of the additions depends only on the chunk layout, so results
+// repeat from run to run.
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* __restrict__ part_hdr,
                                                        const T* __restrict__ part_val, u32 units,
                                                        u32 lp_full, u32 P, u32 n_chunks) {
     const u32 lane = threadIdx.x & 63u;
-    const u32 wave = blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
+    const u32 w = blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
+    if (w >= n_chunks) return;
+    const uint4 h = part_hdr[w];
+    if (!(h.w & 1u)) return;  // wave-uniform
     const u32 col0 = blockIdx.y * 64u;
     const u32 lp = (units - col0) < 64u ? (units - col0) : 64u;
     const u32 g = lane / lp_full;
     const u32 c = lane - g * lp_full;
-    const u64 w = (u64)wave * P + g;
-    if (!(g < P && c < lp) || w >= n_chunks) return;
-    const uint4 h = part_hdr[w];
-    if (!(h.w & 1u)) return;
+    const bool lane_on = g < P && c < lp;
     const u32 col = col0 + c;
-    T acc = part_val[(w * 2 + 1) * units + col];
-    for (u64 x = w + 1; x < n_chunks; ++x) {
-        const uint4 hx = part_hdr[x];
-        if (!(hx.y & 1u) || hx.x != h.z) break;
-        acc = vadd(acc, part_val[(x * 2) * units + col]);
-        if (hx.y & 2u) break;
+    // last chunk of the run: 64 headers per step
+    u32 last = w;
+    for (u32 base = w + 1; base < n_chunks; base += 64) {
+        const u32 x = base + lane;
+        bool ends = false, brk = true;
+        if (x < n_chunks) {
+            const uint4 hx = part_hdr[x];
+            const bool same = (hx.y & 1u) && hx.x == h.z;
+            ends = same && (hx.y & 2u);
+            brk = !same;
+        }
+        const u64 em = __ballot(ends), bm = __ballot(brk);
+        const u64 any = em | bm;
+        if (any) {
+            const u32 f = (u32)__ffsll((unsigned long long)any) - 1u;
+            last = ((em >> f) & 1ull) ? base + f : base + f - 1u;
+            break;
+        }
+        last = base + 63u;
     }
-    finalize<T>(t, h.z, col, units, acc);
+    T acc = vzero(T());
+    if (lane_on) {
+        if (g == 0) acc = part_val[((u64)w * 2 + 1) * units + col];
+        for (u64 x = (u64)w + 1 + g; x <= last; x += P) acc = vadd(acc, part_val[(x * 2) * units + col]);
+    }
+    u32 top = 1;
+    while (top < P) top <<= 1;
+    for (u32 off = top >> 1; off >= 1; off >>= 1) {
+        T o = vshfl_down(acc, off * lp_full);
+        if (g + off < P) acc = vadd(acc, o);
+    }
+    if (lane_on && g == 0) finalize<T>(t, h.z, col, units, acc);
 }
 
 template <typename T>
@@ -627,29 +660,36 @@ hipError_t launch_rollback(const TableDev& t, const u32* slot_idx, size_t n, u32
     return hipGetLastError();
 }
 
-hipError_t launch_segreduce_update(const TableDev& t, const u32* sorted_slot, const u32* sorted_idx,
-                                   size_t n, const float* grads, uint4* part_hdr, float* part_val,
-                                   hipStream_t s) {
+hipError_t launch_segreduce(const TableDev& t, const u32* sorted_slot, const u32* sorted_idx, size_t n,
+                            const float* grads, uint4* part_hdr, float* part_val, hipStream_t s) {
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads, part_val);
     const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
-    dim3 grid1((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);
-    const u32 fix_waves = (g.n_chunks + g.p - 1) / g.p;
-    dim3 grid2((fix_waves + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);
-    if (v4) {
-        segreduce_kernel<float4><<<grid1, BLOCK, 0, s>>>(
+    dim3 grid((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);
+    if (v4)
+        segreduce_kernel<float4><<<grid, BLOCK, 0, s>>>(
             t, sorted_slot, sorted_idx, (u32)n, reinterpret_cast<const float4*>(grads), part_hdr,
             reinterpret_cast<float4*>(part_val), g.units, g.lp, g.p, g.wch, g.n_chunks);
-        fixup_kernel<float4><<<grid2, BLOCK, 0, s>>>(t, part_hdr,
-                                                     reinterpret_cast<const float4*>(part_val),
-                                                     g.units, g.lp, g.p, g.n_chunks);
-    } else {
-        segreduce_kernel<float><<<grid1, BLOCK, 0, s>>>(t, sorted_slot, sorted_idx, (u32)n, grads,
-                                                        part_hdr, part_val, g.units, g.lp, g.p,
-                                                        g.wch, g.n_chunks);
-        fixup_kernel<float><<<grid2, BLOCK, 0, s>>>(t, part_hdr, part_val, g.units, g.lp, g.p,
-                                                    g.n_chunks);
-    }
+    else
+        segreduce_kernel<float><<<grid, BLOCK, 0, s>>>(t, sorted_slot, sorted_idx, (u32)n, grads,
+                                                       part_hdr, part_val, g.units, g.lp, g.p,
+                                                       g.wch, g.n_chunks);
+    return hipGetLastError();
+}
+
+hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
+                        const float* part_val, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const bool v4 = vec4_ok(t, grads, part_val);  // the layout launch_segreduce chose
+    const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
+    dim3 grid((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per chunk
+    if (v4)
+        fixup_kernel<float4><<<grid, BLOCK, 0, s>>>(t, part_hdr,
+                                                    reinterpret_cast<const float4*>(part_val),
+                                                    g.units, g.lp, g.p, g.n_chunks);
+    else
+        fixup_kernel<float><<<grid, BLOCK, 0, s>>>(t, part_hdr, part_val, g.units, g.lp, g.p,
+                                                   g.n_chunks);
     return hipGetLastError();
 }
 

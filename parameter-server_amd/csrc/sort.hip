@@ -8,10 +8,15 @@
 
 namespace pshbm {
 
+// rocPRIM's default switches to a merge sort (about twenty launches) below 2^20 items; batches
+// here are that size, and the Onesweep radix path is several times faster for them.
+using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                              rocprim::default_config, 8192>;
+
 size_t sort_pairs_temp_bytes(size_t n) {
     size_t bytes = 0;
     uint32_t* k = nullptr;
-    (void)rocprim::radix_sort_pairs(nullptr, bytes, k, k, k, k, n, 0, 32, hipStreamDefault);
+    (void)rocprim::radix_sort_pairs<SortConfig>(nullptr, bytes, k, k, k, k, n, 0, 32, hipStreamDefault);
     return bytes;
 }
 
@@ -19,7 +24,7 @@ hipError_t sort_pairs(void* temp, size_t temp_bytes, const uint32_t* keys_in, ui
                       const uint32_t* vals_in, uint32_t* vals_out, size_t n, unsigned end_bit,
                       hipStream_t s) {
     if (n == 0) return hipSuccess;
-    return rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, vals_in, vals_out, n, 0,
+    return rocprim::radix_sort_pairs<SortConfig>(temp, temp_bytes, keys_in, keys_out, vals_in, vals_out, n, 0,
                                      end_bit, s);
 }
 

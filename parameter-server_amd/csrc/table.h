@@ -105,11 +105,15 @@ hipError_t launch_gather_slots(const TableDev& t, const uint32_t* slot_idx, size
 hipError_t launch_rollback(const TableDev& t, const uint32_t* slot_idx, size_t n,
                            uint32_t first_new_row, hipStream_t s);
 
-// Duplicate aggregation + update over pairs sorted by slot. part_hdr: n_chunks uint4;
+// Duplicate aggregation + update over pairs sorted by slot, in two launches: launch_segreduce
+// sums runs of equal slots inside each wavefront's chunk and applies the complete ones;
+// launch_fixup joins the runs that cross chunk borders. part_hdr: n_chunks uint4;
 // part_val: n_chunks * 2 * dim floats.
-hipError_t launch_segreduce_update(const TableDev& t, const uint32_t* sorted_slot,
-                                   const uint32_t* sorted_idx, size_t n, const float* grads,
-                                   uint4* part_hdr, float* part_val, hipStream_t s);
+hipError_t launch_segreduce(const TableDev& t, const uint32_t* sorted_slot, const uint32_t* sorted_idx,
+                            size_t n, const float* grads, uint4* part_hdr, float* part_val,
+                            hipStream_t s);
+hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
+                        const float* part_val, hipStream_t s);
 
 // One optimizer step per located key, no aggregation (keys distinct).
 hipError_t launch_update_unique(const TableDev& t, const uint32_t* slot_idx, size_t n,

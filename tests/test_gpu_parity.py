@@ -144,12 +144,37 @@ def test_aggregation_exact_with_integer_gradients(ps, orc, dim):
     t.close()
 
 
+LOW_MULTIPLICITY = 32
+
+
+def assert_push_parity(gpu, seq, exact, multiplicity):
+    """gpu / seq / exact: key-sorted dumps after the same push from the same state, through the
+    kernels, the oracle (sums duplicates sequentially in fp32, the reference's order) and the
+    oracle with exactly rounded sums. Every value must be within RTOL/ATOL of the reference-order
+    result. The one excuse: a key repeated more than LOW_MULTIPLICITY times in the batch, where
+    the order of the fp32 additions alone moves the sum by more than the tolerance (the
+    sequential sum of thousands of terms is itself that far from the exact sum); such a value
+    must then be at least as close to the exactly rounded result as the reference-order one."""
+    np.testing.assert_array_equal(gpu["key"], seq["key"])
+    np.testing.assert_array_equal(gpu["key"], exact["key"])
+    g, s, e = (x["value"].astype(np.float64) for x in (gpu, seq, exact))
+    ok = np.abs(g - s) <= ATOL + RTOL * np.abs(s)
+    if ok.all():
+        return
+    bad_rows = np.unique(np.nonzero(~ok)[0])
+    assert (multiplicity[bad_rows] > LOW_MULTIPLICITY).all(), \
+        "a key of low multiplicity misses the tolerance"
+    closer = np.abs(g - e) <= np.abs(s - e) + ATOL + RTOL * np.abs(e)
+    assert (ok | closer).all(), "a heavily repeated key is further from the exact sum than the reference order"
+
+
 @pytest.mark.parametrize("opt", ["sgd", "adagrad", "ftrl"])
 @pytest.mark.parametrize("dim,s", [(16, 1.05), (64, 1.2), (8, 1.1), (128, 1.1)])
 def test_push_zipf_within_tolerance(ps, orc, wl, opt, dim, s):
     rng = np.random.default_rng(11)
     n_table, batch = 20000, 30000
     t, r = pair(ps, orc, dim, opt, capacity=n_table + 4000)
+    x = orc.Oracle(dim, capacity=n_table + 4000, **OPTS[opt])   # exactly rounded aggregation
     keys = wl.table_keys_np(0, n_table, seed=2)
     vf = t.value_floats
     vals = rng.normal(0, 0.01, (n_table, vf)).astype(np.float32)
@@ -157,19 +182,26 @@ def test_push_zipf_within_tolerance(ps, orc, wl, opt, dim, s):
         vals[:, dim:] = 0.1
     if opt == "ftrl":
         vals[:, 2 * dim:] = vals[:, dim:2 * dim] ** 2
-    assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+    for b in (t, r, x):
+        assert b.set(keys, vals) == 0
     for step in range(3):
         q = wl.zipf_batch_np(rng, n_table, s, batch, seed=2)
         q[:500] = wl.fresh_keys_np(rng, 500)            # insert-on-miss inside a push
         q[500:600] = q[:100]                            # duplicated fresh keys
         g = rng.normal(0, 1e-3, (batch, dim)).astype(np.float32)
         assert t.push(q, g) == 0 and r.push(q, g) == 0
+        assert x.push(q, g, orc.PUSH_EXACT_AGGREGATION) == 0
         st, rows, hit = t.pull(q[:4000])
         st2, rows2, hit2 = r.pull(q[:4000])
         np.testing.assert_array_equal(hit, hit2)
-        np.testing.assert_allclose(rows, rows2, rtol=RTOL, atol=ATOL)
+        a, b, c = sorted_dump(t), sorted_dump(r), sorted_dump(x)
+        uk, cnt = np.unique(q, return_counts=True)
+        mult = np.zeros(a.size, np.int64)
+        mult[np.searchsorted(a["key"], uk)] = cnt
+        assert_push_parity(a, b, c, mult)
+        # next step: everyone restarts from the reference-order state
+        assert t.set(b["key"], b["value"]) == 0 and x.set(b["key"], b["value"]) == 0
     assert t.size() == r.size()
-    assert_same_table(t, r, exact=False)
     t.close()
 
 
@@ -272,7 +304,7 @@ def test_dump_load_iterate_roundtrip(ps, orc, wl, opt, dim):
 
 
 def test_reserved_keys_and_stats(ps, orc, wl):
-    t, r = pair(ps, orc, 4, "sum", capacity=20000, max_load_factor=0.8)
+    t = ps.Table(4, capacity=20000, max_load_factor=0.8)
     bad = np.array([1, 0xFFFFFFFFFFFFFFFF], np.uint64)
     assert t.push(bad, np.ones((2, 4), np.float32)) == ps.ERROR
     assert t.pull(bad)[0] == ps.ERROR and t.size() == 0
