@@ -44,6 +44,7 @@ struct pshbm_table {
 
     // per-batch workspace of the mutating paths
     size_t ws_cap = 0;
+    unsigned sort_parity = 0;  // which half of the sort head the next sort uses
     DevBuf ws_slot, ws_idx, ws_sslot, ws_sidx, ws_sort, ws_hdr, ws_pval;
 
     // staging of the host-pointer entry points
@@ -163,6 +164,8 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     ST_TRY(ensure(t, t->ws_sslot, cap * 4));
     ST_TRY(ensure(t, t->ws_sidx, cap * 4));
     ST_TRY(ensure(t, t->ws_sort, sort_pairs_temp_bytes(cap)));
+    HIP_TRY(t, hipMemset(t->ws_sort.p, 0, sort_pairs_head_bytes()));
+    t->sort_parity = 0;
     // partial sums of the segmented reduce: size for the scalar layout, which has more chunks
     SegGeom g1 = seg_geometry(t->d.dim, 1, cap);
     SegGeom g4 = seg_geometry(t->d.dim, (t->d.dim % 4 == 0) ? 4 : 1, cap);
@@ -187,6 +190,9 @@ int32_t begin_op(pshbm_table* t, hipStream_t s) {
 int32_t read_counters(pshbm_table* t, hipStream_t s) {
     HIP_TRY(t, hipMemcpyAsync(t->h_counters, t->d.counters, CNT_WORDS * 4, hipMemcpyDeviceToHost, s));
     HIP_TRY(t, hipStreamSynchronize(s));
+    if (t->h_counters[CNT_SORT_ERR])
+        return fail(t, PSHBM_FATAL, "a radix-sort tile timed out waiting for its predecessor; "
+                                    "the last push may be wrong");
     return PSHBM_OK;
 }
 
@@ -254,13 +260,16 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
     } else {
         uint32_t* sslot = static_cast<uint32_t*>(t->ws_sslot.p);
         uint32_t* sidx = static_cast<uint32_t*>(t->ws_sidx.p);
+        bool in_b = false;
         HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT,
-                     sort_pairs(t->ws_sort.p, t->ws_sort.bytes, slot, sslot, idx, sidx, n,
-                                t->slot_bits + 1, s));
+                     sort_pairs(t->ws_sort.p, t->ws_sort.bytes, t->sort_parity++, slot, sslot, idx, sidx, n,
+                                t->slot_bits + 1, &in_b, t->d.counters + CNT_SORT_ERR, s));
+        const uint32_t* fs = in_b ? sslot : slot;
+        const uint32_t* fi = in_b ? sidx : idx;
         uint4* hdr = static_cast<uint4*>(t->ws_hdr.p);
         float* pval = static_cast<float*>(t->ws_pval.p);
         HIP_TRY_PROF(t, s, PSHBM_PHASE_SEGREDUCE,
-                     launch_segreduce(t->d, sslot, sidx, n, d_grads, hdr, pval, s));
+                     launch_segreduce(t->d, fs, fi, n, d_grads, hdr, pval, s));
         HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP, launch_fixup(t->d, n, d_grads, hdr, pval, s));
     }
     return PSHBM_OK;

@@ -1,31 +1,285 @@
-// Sort of (slot, batch index) pairs by slot: the grouping step of duplicate-key aggregation.
-// The passes are rocPRIM's LSD radix sort restricted to the bits a slot index can have.
+// Stable LSD radix sort of (slot, batch index) pairs by slot: the grouping step of duplicate-key
+// aggregation. Written for batches of 10^5..10^7 pairs, where launch count and latency matter more
+// than bandwidth: one histogram launch, then ONE launch per 8-bit digit.
+//
+// A digit pass cuts the input into tiles of 4096 pairs, one per 1024-thread workgroup:
+//   1. each of the 16 wavefronts ranks its 256 pairs, 64 at a time: eight ballots give every lane
+//      the set of lanes holding the same digit; its rank is the wave's running count for that
+//      digit plus the number of lower lanes in that set (equal digits keep their input order);
+//   2. thread b < 256 owns digit b: it chains the 16 wave counts into the tile count, publishes it
+//      in status[tile][b], looks back over the predecessors' published counts -- 16 words per
+//      round trip -- until it meets one that already carries a running total ("decoupled
+//      look-back"), and publishes its own running total;
+//   3. the pairs are first put in digit order in LDS, then written out by consecutive lanes, so
+//      that each run of equal digits is a contiguous, coalesced store.
+// The look-back spin is bounded: if a predecessor does not publish within SPIN_LIMIT polls the
+// tile raises *err_flag and goes on with what it has, so the grid always drains.
 #include "table.h"
-
-#include <cstring>
-
-#include <rocprim/device/device_radix_sort.hpp>
 
 namespace pshbm {
 
-// rocPRIM's default switches to a merge sort (about twenty launches) below 2^20 items; batches
-// here are that size, and the Onesweep radix path is several times faster for them.
-using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
-                                              rocprim::default_config, 8192>;
+namespace {
 
-size_t sort_pairs_temp_bytes(size_t n) {
-    size_t bytes = 0;
-    uint32_t* k = nullptr;
-    (void)rocprim::radix_sort_pairs<SortConfig>(nullptr, bytes, k, k, k, k, n, 0, 32, hipStreamDefault);
-    return bytes;
+using u32 = uint32_t;
+using u64 = uint64_t;
+
+constexpr u32 SORT_BLOCK = 1024;
+constexpr u32 SORT_WAVES = SORT_BLOCK / 64;  // 16
+constexpr u32 SORT_ITEMS = 4;
+constexpr u32 SORT_TILE = SORT_BLOCK * SORT_ITEMS;  // 4096
+constexpr u32 SORT_WAVE_SPAN = 64 * SORT_ITEMS;     // 256 pairs per wavefront
+constexpr u32 RADIX = 256;
+constexpr u32 MAX_PASSES = 4;
+constexpr u32 FLAG_AGG = 1u << 30, FLAG_PREFIX = 2u << 30, COUNT_MASK = (1u << 30) - 1u;
+constexpr u32 SPIN_LIMIT = 1u << 24;
+constexpr u32 LOOKBACK = 16;  // predecessor words fetched per round trip
+
+// temp layout in 32-bit words: two heads {digit totals [MAX_PASSES][RADIX], tile counters
+// [MAX_PASSES] (+ pad)} used by alternate sorts -- each sort zeroes the other one for its
+// successor, which saves a fill launch -- then status [MAX_PASSES][n_tiles][RADIX].
+constexpr size_t HEAD_TOTALS = 0;
+constexpr size_t HEAD_COUNTERS = MAX_PASSES * RADIX;
+constexpr size_t HEAD_WORDS = HEAD_COUNTERS + 16;
+constexpr size_t OFF_STATUS = 2 * HEAD_WORDS;
+
+__global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(const u32* __restrict__ keys, u32 n,
+                                                                u32 n_tiles, u32 passes,
+                                                                u32* __restrict__ totals,
+                                                                u32* __restrict__ status,
+                                                                u32* __restrict__ next_head) {
+    // Counts the lowest digit only; every digit pass counts the next digit of the pairs it holds.
+    __shared__ u32 h[RADIX];
+    const u32 tid = threadIdx.x;
+    if (tid < RADIX) h[tid] = 0;
+    const u32 tile = blockIdx.x;
+    const u64 base = (u64)tile * SORT_TILE;
+    u32 k[SORT_ITEMS];
+#pragma unroll
+    for (u32 j = 0; j < SORT_ITEMS; ++j) {  // all loads in flight before the first LDS atomic
+        const u64 i = base + (u64)j * SORT_BLOCK + tid;
+        k[j] = i < n ? keys[i] : 0u;
+    }
+    __syncthreads();
+#pragma unroll
+    for (u32 j = 0; j < SORT_ITEMS; ++j)
+        if (base + (u64)j * SORT_BLOCK + tid < n) atomicAdd(&h[k[j] & 255u], 1u);
+    __syncthreads();
+    {
+        const u32 p = tid >> 8, b = tid & 255u;  // 1024 threads = MAX_PASSES x RADIX
+        if (p == 0 && h[b]) atomicAdd(&totals[b], h[b]);
+        if (p < passes)
+            status[((size_t)p * n_tiles + tile) * RADIX + b] = 0;  // this tile's look-back words
+    }
+    // the totals and tile counters of the NEXT sort (the other half of the head) start at zero
+    if (tile == 0)
+        for (u32 x = tid; x < HEAD_WORDS; x += SORT_BLOCK) next_head[x] = 0;
 }
 
-hipError_t sort_pairs(void* temp, size_t temp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
-                      const uint32_t* vals_in, uint32_t* vals_out, size_t n, unsigned end_bit,
-                      hipStream_t s) {
+// exclusive scan over the 256 values held by threads 0..255 (4 wavefronts); all threads of the
+// block must call it (it contains a barrier). `sums` is LDS scratch of 4 words.
+__device__ __forceinline__ u32 scan256_exclusive(u32 v, u32 tid, u32* sums) {
+    const u32 lane = tid & 63u, w = tid >> 6;
+    u32 incl = v;
+    for (u32 off = 1; off < 64; off <<= 1) {
+        const u32 o = __shfl_up(incl, off);
+        if (lane >= off) incl += o;
+    }
+    if (lane == 63 && w < 4) sums[w] = incl;
+    __syncthreads();
+    u32 r = incl - v;
+    for (u32 x = 0; x < w && x < 4; ++x) r += sums[x];
+    return r;
+}
+
+__global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
+    const u32* __restrict__ kin, const u32* __restrict__ vin, u32* __restrict__ kout,
+    u32* __restrict__ vout, u32 n, u32 shift, const u32* __restrict__ totals,
+    u32* __restrict__ totals_next, u32* status, u32* err_flag) {
+    __shared__ volatile u32 wcnt[SORT_WAVES][RADIX];  // per-wave digit counts, then offsets
+    __shared__ u32 hnext[RADIX];                      // this tile's counts of the next digit
+    __shared__ u32 binpos[RADIX];                     // global position of a digit's run - its place in the tile
+    __shared__ u32 tile_start[RADIX];                 // place of a digit's run in the tile
+    __shared__ u32 skey[SORT_TILE], sval[SORT_TILE];
+    __shared__ u32 sums_a[4], sums_b[4];
+    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    // Tiles are taken in workgroup order. The hardware starts workgroups in that order, so a
+    // tile's predecessors are running (or done) when it looks back; should that ever not hold,
+    // the bounded spin below turns a would-be hang into an error flag.
+    const u32 tile = blockIdx.x;
+    const u32 tot = tid < RADIX ? totals[tid] : 0u;  // needed late; fetched with the pairs
+#pragma unroll
+    for (u32 x = 0; x < SORT_WAVES * RADIX / SORT_BLOCK; ++x)
+        (&wcnt[0][0])[x * SORT_BLOCK + tid] = 0;
+    if (tid < RADIX) hnext[tid] = 0;
+    __syncthreads();
+    const u64 tile_base = (u64)tile * SORT_TILE;
+    const u64 base = tile_base + (u64)w * SORT_WAVE_SPAN;
+    const u64 lt_mask = (1ull << lane) - 1ull;
+
+    u32 key[SORT_ITEMS], val[SORT_ITEMS], rnk[SORT_ITEMS];
+#pragma unroll
+    for (u32 j = 0; j < SORT_ITEMS; ++j) {
+        const u64 i = base + (u64)j * 64 + lane;
+        const bool valid = i < n;
+        key[j] = valid ? kin[i] : 0xFFFFFFFFu;
+        val[j] = valid ? vin[i] : 0u;
+    }
+    // 1. rank inside the wavefront, keeping input order among equal digits
+#pragma unroll
+    for (u32 j = 0; j < SORT_ITEMS; ++j) {
+        const bool valid = base + (u64)j * 64 + lane < n;
+        const u32 d = (key[j] >> shift) & 255u;
+        u64 peers = __ballot(valid);
+#pragma unroll
+        for (u32 b = 0; b < 8; ++b) {
+            const bool bit = (d >> b) & 1u;
+            const u64 m = __ballot(valid && bit);
+            peers &= bit ? m : ~m;
+        }
+        const u32 before = (u32)__popcll(peers & lt_mask);
+        u32 running = 0;
+        if (valid) {
+            running = wcnt[w][d];
+            if (before == 0) wcnt[w][d] = running + (u32)__popcll(peers);
+        }
+        rnk[j] = running + before;
+        if (valid && totals_next) atomicAdd(&hnext[(key[j] >> (shift + 8)) & 255u], 1u);
+    }
+    __syncthreads();
+    // 2. thread b < 256 owns digit b: wave offsets, tile count, digit base, look-back
+    u32 tile_count = 0;
+    if (tid < RADIX) {
+        u32 run = 0;
+#pragma unroll
+        for (u32 x = 0; x < SORT_WAVES; ++x) {
+            const u32 c = wcnt[x][tid];
+            wcnt[x][tid] = run;
+            run += c;
+        }
+        tile_count = run;
+        if (totals_next && hnext[tid]) atomicAdd(&totals_next[tid], hnext[tid]);
+        // publish early, so that successors can start adding
+        __hip_atomic_store(status + (size_t)tile * RADIX + tid,
+                           (tile == 0 ? FLAG_PREFIX : FLAG_AGG) | tile_count, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const u32 digit_base = scan256_exclusive(tot, tid, sums_a);       // over the whole input
+    const u32 local_start = scan256_exclusive(tile_count, tid, sums_b);  // inside this tile
+    if (tid < RADIX) {
+        const u32 b = tid;
+        u32 excl = 0;
+        if (tile != 0) {
+            // Walk back over the predecessors, LOOKBACK words per round trip: add counts until a
+            // word with a running total is met; a word not yet published stops the batch there.
+            int t = (int)tile - 1;
+            u32 spins = 0;
+            bool done = false;
+            while (!done) {
+                u32 sw[LOOKBACK];
+#pragma unroll
+                for (u32 q = 0; q < LOOKBACK; ++q)
+                    sw[q] = (t - (int)q >= 0)
+                                ? __hip_atomic_load(status + (size_t)(t - (int)q) * RADIX + b,
+                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                : FLAG_PREFIX;
+                u32 used = 0;
+                bool stalled = false;
+#pragma unroll
+                for (u32 q = 0; q < LOOKBACK; ++q) {
+                    if (!done && !stalled) {
+                        const u32 f = sw[q] >> 30;
+                        if (f == 0) {
+                            stalled = true;
+                        } else {
+                            excl += sw[q] & COUNT_MASK;
+                            ++used;
+                            if (f == 2) done = true;
+                        }
+                    }
+                }
+                t -= (int)used;
+                if (!done && used == 0) {
+                    if (++spins > SPIN_LIMIT) {  // never expected; keeps the grid from hanging
+                        *err_flag = 1u;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+            __hip_atomic_store(status + (size_t)tile * RADIX + b,
+                               FLAG_PREFIX | ((excl + tile_count) & COUNT_MASK), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+        tile_start[b] = local_start;
+        binpos[b] = digit_base + excl - local_start;  // wraps; undone by adding the place in the tile
+    }
+    __syncthreads();
+    // 3. digit order in LDS, then coalesced stores
+#pragma unroll
+    for (u32 j = 0; j < SORT_ITEMS; ++j) {
+        const bool valid = base + (u64)j * 64 + lane < n;
+        if (valid) {
+            const u32 d = (key[j] >> shift) & 255u;
+            const u32 place = tile_start[d] + wcnt[w][d] + rnk[j];
+            skey[place] = key[j];
+            sval[place] = val[j];
+        }
+    }
+    __syncthreads();
+    const u32 tile_n = (n - tile_base) < SORT_TILE ? (u32)(n - tile_base) : SORT_TILE;
+#pragma unroll
+    for (u32 j = 0; j < SORT_ITEMS; ++j) {
+        const u32 place = j * SORT_BLOCK + tid;
+        if (place < tile_n) {
+            const u32 k = skey[place];
+            const u32 pos = binpos[(k >> shift) & 255u] + place;
+            kout[pos] = k;
+            vout[pos] = sval[place];
+        }
+    }
+}
+
+}  // namespace
+
+size_t sort_pairs_temp_bytes(size_t n) {
+    const size_t n_tiles = (n + SORT_TILE - 1) / SORT_TILE;
+    return (OFF_STATUS + (size_t)MAX_PASSES * (n_tiles ? n_tiles : 1) * RADIX) * 4;
+}
+
+size_t sort_pairs_head_bytes() { return OFF_STATUS * 4; }
+
+hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys_a,
+                      uint32_t* keys_b, uint32_t* vals_a, uint32_t* vals_b, size_t n,
+                      unsigned end_bit, bool* result_in_b, uint32_t* err_flag, hipStream_t s) {
+    *result_in_b = false;
     if (n == 0) return hipSuccess;
-    return rocprim::radix_sort_pairs<SortConfig>(temp, temp_bytes, keys_in, keys_out, vals_in, vals_out, n, 0,
-                                     end_bit, s);
+    if (n > COUNT_MASK || temp_bytes < sort_pairs_temp_bytes(n)) return hipErrorInvalidValue;
+    const u32 passes = (end_bit + 7) / 8;
+    if (passes == 0 || passes > MAX_PASSES) return hipErrorInvalidValue;
+    const u32 n_tiles = (u32)((n + SORT_TILE - 1) / SORT_TILE);
+    u32* words = static_cast<u32*>(temp);
+    u32* head = words + (parity & 1u) * HEAD_WORDS;
+    u32* next_head = words + ((parity & 1u) ^ 1u) * HEAD_WORDS;
+    u32* totals = head + HEAD_TOTALS;
+    u32* status = words + OFF_STATUS;
+    sort_hist_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys_a, (u32)n, n_tiles, passes, totals, status,
+                                                    next_head);
+    u32 *kin = keys_a, *vin = vals_a, *kout = keys_b, *vout = vals_b;
+    for (u32 p = 0; p < passes; ++p) {
+        sort_pass_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(kin, vin, kout, vout, (u32)n, 8 * p,
+                                                        totals + p * RADIX,
+                                                        p + 1 < passes ? totals + (p + 1) * RADIX : nullptr,
+                                                        status + (size_t)p * n_tiles * RADIX,
+                                                        err_flag);
+        u32* tk = kin;
+        u32* tv = vin;
+        kin = kout;
+        vin = vout;
+        kout = tk;
+        vout = tv;
+    }
+    *result_in_b = (passes & 1u) != 0;
+    return hipGetLastError();
 }
 
 }  // namespace pshbm

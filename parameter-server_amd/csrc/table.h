@@ -27,6 +27,7 @@ enum {
     CNT_DUP = 2,       // keys that were already present (counted on request)
     CNT_ENTRY = 3,     // CNT_ROWS as it was when the current pull began
     CNT_BADKEY = 4,    // reserved keys met in a batch (skipped)
+    CNT_SORT_ERR = 5,  // a sort tile gave up waiting for its predecessor
     CNT_WORDS = 8
 };
 
@@ -137,9 +138,16 @@ hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long l
                              hipStream_t s);
 
 // ---- sort (sort.hip) -----------------------------------------------------------------------
+// Stable radix sort of (key, value) pairs on the low `end_bit` bits (rounded up to whole bytes).
+// Both buffer pairs are scratch: the sorted pairs end in (keys_b, vals_b) when *result_in_b, else
+// in (keys_a, vals_a). *err_flag (device) is raised if a tile's bounded wait for its predecessor
+// ran out, in which case the output is not sorted.
+// `temp` starts with a head of sort_pairs_head_bytes() that must be zero before the first sort
+// and is kept zeroed by the sorts themselves as long as `parity` alternates 0,1,0,1,...
 size_t sort_pairs_temp_bytes(size_t n);
-hipError_t sort_pairs(void* temp, size_t temp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
-                      const uint32_t* vals_in, uint32_t* vals_out, size_t n, unsigned end_bit,
-                      hipStream_t s);
+size_t sort_pairs_head_bytes();
+hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys_a,
+                      uint32_t* keys_b, uint32_t* vals_a, uint32_t* vals_b, size_t n,
+                      unsigned end_bit, bool* result_in_b, uint32_t* err_flag, hipStream_t s);
 
 }  // namespace pshbm
