@@ -6,14 +6,15 @@
 //   1. each of the 16 wavefronts ranks its 256 pairs, 64 at a time: eight ballots give every lane
 //      the set of lanes holding the same digit; its rank is the wave's running count for that
 //      digit plus the number of lower lanes in that set (equal digits keep their input order);
-//   2. thread b < 256 owns digit b: it chains the 16 wave counts into the tile count, publishes it
-//      in status[tile][b], looks back over the predecessors' published counts -- 16 words per
-//      round trip -- until it meets one that already carries a running total ("decoupled
-//      look-back"), and publishes its own running total;
+//   2. thread b < 256 owns digit b: it chains the 16 wave counts into the tile count and publishes
+//      it; the last tile of every group of 16 tiles also publishes the group's count. The number
+//      of pairs with digit b in earlier tiles is then the sum of at most 15 tile words and of the
+//      group words before -- two or three batches of loads that wait only for published counts,
+//      never for another tile's finished prefix, so no chain forms across the tiles;
 //   3. the pairs are first put in digit order in LDS, then written out by consecutive lanes, so
 //      that each run of equal digits is a contiguous, coalesced store.
-// The look-back spin is bounded: if a predecessor does not publish within SPIN_LIMIT polls the
-// tile raises *err_flag and goes on with what it has, so the grid always drains.
+// The wait is bounded: if a word is not published within SPIN_LIMIT polls the tile raises
+// *err_flag and goes on with what it has, so the grid always drains.
 #include "table.h"
 
 namespace pshbm {
@@ -30,13 +31,14 @@ constexpr u32 SORT_TILE = SORT_BLOCK * SORT_ITEMS;  // 4096
 constexpr u32 SORT_WAVE_SPAN = 64 * SORT_ITEMS;     // 256 pairs per wavefront
 constexpr u32 RADIX = 256;
 constexpr u32 MAX_PASSES = 4;
-constexpr u32 FLAG_AGG = 1u << 30, FLAG_PREFIX = 2u << 30, COUNT_MASK = (1u << 30) - 1u;
+constexpr u32 FLAG_READY = 1u << 30, COUNT_MASK = (1u << 30) - 1u;
 constexpr u32 SPIN_LIMIT = 1u << 24;
-constexpr u32 LOOKBACK = 16;  // predecessor words fetched per round trip
+constexpr u32 GROUP = 16;  // tiles per group of the two-level tile prefix
 
 // temp layout in 32-bit words: two heads {digit totals [MAX_PASSES][RADIX], tile counters
 // [MAX_PASSES] (+ pad)} used by alternate sorts -- each sort zeroes the other one for its
-// successor, which saves a fill launch -- then status [MAX_PASSES][n_tiles][RADIX].
+// successor, which saves a fill launch -- then, per pass, [n_tiles][RADIX] tile words and
+// [n_groups][RADIX] group words.
 constexpr size_t HEAD_TOTALS = 0;
 constexpr size_t HEAD_COUNTERS = MAX_PASSES * RADIX;
 constexpr size_t HEAD_WORDS = HEAD_COUNTERS + 16;
@@ -67,8 +69,11 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(const u32* __rest
     {
         const u32 p = tid >> 8, b = tid & 255u;  // 1024 threads = MAX_PASSES x RADIX
         if (p == 0 && h[b]) atomicAdd(&totals[b], h[b]);
-        if (p < passes)
-            status[((size_t)p * n_tiles + tile) * RADIX + b] = 0;  // this tile's look-back words
+        if (p < passes) {  // this tile's published words, and its group's if it opens the group
+            const size_t rows = n_tiles + (n_tiles + GROUP - 1) / GROUP;
+            status[(p * rows + tile) * RADIX + b] = 0;
+            if (tile % GROUP == 0) status[(p * rows + n_tiles + tile / GROUP) * RADIX + b] = 0;
+        }
     }
     // the totals and tile counters of the NEXT sort (the other half of the head) start at zero
     if (tile == 0)
@@ -91,10 +96,38 @@ __device__ __forceinline__ u32 scan256_exclusive(u32 v, u32 tid, u32* sums) {
     return r;
 }
 
+// Sum of `count` (<= GROUP) published words spaced RADIX apart, starting at `words`. The loads of a
+// batch are issued together; the batch is fetched again until every word carries FLAG_READY. The
+// wait is bounded: past SPIN_LIMIT polls the caller gets what is there and *err_flag is raised.
+__device__ __forceinline__ u32 wait_sum(const u32* words, u32 count, u32* err_flag) {
+    if (count == 0) return 0;
+    u32 spins = 0;
+    while (true) {
+        u32 sw[GROUP];
+#pragma unroll
+        for (u32 q = 0; q < GROUP; ++q)
+            sw[q] = q < count ? __hip_atomic_load(words + (size_t)q * RADIX, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT)
+                              : FLAG_READY;
+        u32 ready = FLAG_READY, sum = 0;
+#pragma unroll
+        for (u32 q = 0; q < GROUP; ++q) {
+            ready &= sw[q];
+            sum += sw[q] & COUNT_MASK;
+        }
+        if (ready & FLAG_READY) return sum;
+        if (++spins > SPIN_LIMIT) {  // never expected; keeps the grid from hanging
+            *err_flag = 1u;
+            return sum;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
 __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
     const u32* __restrict__ kin, const u32* __restrict__ vin, u32* __restrict__ kout,
     u32* __restrict__ vout, u32 n, u32 shift, const u32* __restrict__ totals,
-    u32* __restrict__ totals_next, u32* status, u32* err_flag) {
+    u32* __restrict__ totals_next, u32* status, u32* group_status, u32 n_tiles, u32* err_flag) {
     __shared__ volatile u32 wcnt[SORT_WAVES][RADIX];  // per-wave digit counts, then offsets
     __shared__ u32 hnext[RADIX];                      // this tile's counts of the next digit
     __shared__ u32 binpos[RADIX];                     // global position of a digit's run - its place in the tile
@@ -158,58 +191,27 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
         }
         tile_count = run;
         if (totals_next && hnext[tid]) atomicAdd(&totals_next[tid], hnext[tid]);
-        // publish early, so that successors can start adding
-        __hip_atomic_store(status + (size_t)tile * RADIX + tid,
-                           (tile == 0 ? FLAG_PREFIX : FLAG_AGG) | tile_count, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
+        // publish early: successors only ever wait for these per-tile counts
+        __hip_atomic_store(status + (size_t)tile * RADIX + tid, FLAG_READY | tile_count,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     const u32 digit_base = scan256_exclusive(tot, tid, sums_a);       // over the whole input
     const u32 local_start = scan256_exclusive(tile_count, tid, sums_b);  // inside this tile
     if (tid < RADIX) {
         const u32 b = tid;
-        u32 excl = 0;
-        if (tile != 0) {
-            // Walk back over the predecessors, LOOKBACK words per round trip: add counts until a
-            // word with a running total is met; a word not yet published stops the batch there.
-            int t = (int)tile - 1;
-            u32 spins = 0;
-            bool done = false;
-            while (!done) {
-                u32 sw[LOOKBACK];
-#pragma unroll
-                for (u32 q = 0; q < LOOKBACK; ++q)
-                    sw[q] = (t - (int)q >= 0)
-                                ? __hip_atomic_load(status + (size_t)(t - (int)q) * RADIX + b,
-                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                : FLAG_PREFIX;
-                u32 used = 0;
-                bool stalled = false;
-#pragma unroll
-                for (u32 q = 0; q < LOOKBACK; ++q) {
-                    if (!done && !stalled) {
-                        const u32 f = sw[q] >> 30;
-                        if (f == 0) {
-                            stalled = true;
-                        } else {
-                            excl += sw[q] & COUNT_MASK;
-                            ++used;
-                            if (f == 2) done = true;
-                        }
-                    }
-                }
-                t -= (int)used;
-                if (!done && used == 0) {
-                    if (++spins > SPIN_LIMIT) {  // never expected; keeps the grid from hanging
-                        *err_flag = 1u;
-                        break;
-                    }
-                    __builtin_amdgcn_s_sleep(1);
-                }
-            }
-            __hip_atomic_store(status + (size_t)tile * RADIX + b,
-                               FLAG_PREFIX | ((excl + tile_count) & COUNT_MASK), __ATOMIC_RELAXED,
+        const u32 grp = tile / GROUP, first = grp * GROUP;
+        // (a) the tiles before this one in its group of GROUP: one batch of loads
+        const u32 in_group = wait_sum(status + (size_t)first * RADIX + b, tile - first, err_flag);
+        // the last tile of a group (or of the input) publishes the group's total
+        if (tile + 1 == first + GROUP || tile + 1 == n_tiles)
+            __hip_atomic_store(group_status + (size_t)grp * RADIX + b,
+                               FLAG_READY | ((in_group + tile_count) & COUNT_MASK), __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
-        }
+        // (b) the groups before this one, GROUP words per round trip
+        u32 excl = in_group;
+        for (u32 g0 = 0; g0 < grp; g0 += GROUP)
+            excl += wait_sum(group_status + (size_t)g0 * RADIX + b, (grp - g0) < GROUP ? grp - g0 : GROUP,
+                             err_flag);
         tile_start[b] = local_start;
         binpos[b] = digit_base + excl - local_start;  // wraps; undone by adding the place in the tile
     }
@@ -243,7 +245,8 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
 
 size_t sort_pairs_temp_bytes(size_t n) {
     const size_t n_tiles = (n + SORT_TILE - 1) / SORT_TILE;
-    return (OFF_STATUS + (size_t)MAX_PASSES * (n_tiles ? n_tiles : 1) * RADIX) * 4;
+    const size_t rows = (n_tiles ? n_tiles : 1) + (n_tiles + GROUP - 1) / GROUP + 1;
+    return (OFF_STATUS + (size_t)MAX_PASSES * rows * RADIX) * 4;
 }
 
 size_t sort_pairs_head_bytes() { return OFF_STATUS * 4; }
@@ -262,6 +265,7 @@ hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* 
     u32* next_head = words + ((parity & 1u) ^ 1u) * HEAD_WORDS;
     u32* totals = head + HEAD_TOTALS;
     u32* status = words + OFF_STATUS;
+    const size_t rows = n_tiles + (n_tiles + GROUP - 1) / GROUP;  // per pass: tile words, group words
     sort_hist_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys_a, (u32)n, n_tiles, passes, totals, status,
                                                     next_head);
     u32 *kin = keys_a, *vin = vals_a, *kout = keys_b, *vout = vals_b;
@@ -269,7 +273,9 @@ hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* 
         sort_pass_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(kin, vin, kout, vout, (u32)n, 8 * p,
                                                         totals + p * RADIX,
                                                         p + 1 < passes ? totals + (p + 1) * RADIX : nullptr,
-                                                        status + (size_t)p * n_tiles * RADIX,
+                                                        status + (size_t)p * rows * RADIX,
+                                                        status + ((size_t)p * rows + n_tiles) * RADIX,
+                                                        n_tiles,
                                                         err_flag);
         u32* tk = kin;
         u32* tv = vin;
