@@ -40,6 +40,13 @@ CONFIGS = {
                desc="C5: 200M keys dim128 Adagrad, pull+push of 4M-key Zipf(1.1) batches"),
 }
 STATE_BLOCKS = {0: 1, 1: 1, 2: 2, 3: 3}
+KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist": "sort_hist_kernel",
+                   "sort_pass": "sort_pass_kernel", "segreduce": "segreduce_kernel",
+                   "fixup": "fixup_kernel", "update_unique": "update_unique_kernel",
+                   "gather": "gather_slots_kernel"}
+# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by the factors a plain
+# copy of known size gave), measured on an MI355X; the summaries are under profiles/.
+MEASURED_TRAFFIC_BYTES = {}
 
 
 def algorithmic_bytes(cfg, phase, k, u):
@@ -165,6 +172,9 @@ def main():
     ap.add_argument("--table-keys", type=int, default=0, help="override the table size (testing)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-keys", type=int, default=10_000_000, help="table size of the CPU sample")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one 256 MiB device copy, a kernel of known HBM traffic that "
+                         "rocprofv3 --pmc runs of this script use to scale FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -177,6 +187,13 @@ def main():
     n_table = args.table_keys or cfg["n"]
     torch.cuda.set_device(0)
 
+    if args.calibration_copy:
+        a = torch.empty(64 << 20, dtype=torch.float32, device="cuda").normal_()
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
     t = build_table(ps, wl, torch, cfg, n_table)
     batches = make_batches(wl, torch, cfg, n_table, n_batches=8)
     out = torch.empty(cfg["batch"], cfg["dim"], device="cuda")
@@ -207,11 +224,14 @@ def main():
             by = algorithmic_bytes(cfg, name, k, u_mean)
             phases[name] = {"avg_ms": round(avg_ms, 5), "launches": int(launches),
                             "algorithmic_GBps": round(by / avg_ms / 1e6, 1)}
+    # the kernel with the longest average launch
     dominant = max(phases, key=lambda p: phases[p]["avg_ms"])
     achieved = phases[dominant]["algorithmic_GBps"]
-    roofline = {"kernel": dominant, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "avg_ms": phases[dominant]["avg_ms"]}
+    roofline = {"kernel": KERNEL_OF_PHASE[dominant], "bound": "hbm", "achieved": achieved,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dominant)) if not args.table_keys else None,
+                "avg_ms": phases[dominant]["avg_ms"],
+                "algorithmic_bytes": int(algorithmic_bytes(cfg, dominant, k, u_mean))}
     step_bytes = sum(algorithmic_bytes(cfg, p, k, u_mean) for p in ("pull",) if True)
     if not cfg["pull_only"]:
         step_bytes += algorithmic_bytes(cfg, "locate", k, u_mean) + algorithmic_bytes(cfg, "segreduce", k, u_mean)

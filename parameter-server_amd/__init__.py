@@ -33,7 +33,7 @@ SYMBOLS = [
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
-PHASES = ["pull", "locate", "sort", "segreduce", "fixup", "update_unique", "gather"]
+PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass"]
 
 
 class Config(C.Structure):

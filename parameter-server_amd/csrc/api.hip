@@ -260,10 +260,18 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
     } else {
         uint32_t* sslot = static_cast<uint32_t*>(t->ws_sslot.p);
         uint32_t* sidx = static_cast<uint32_t*>(t->ws_sidx.p);
-        bool in_b = false;
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT,
-                     sort_pairs(t->ws_sort.p, t->ws_sort.bytes, t->sort_parity++, slot, sslot, idx, sidx, n,
-                                t->slot_bits + 1, &in_b, t->d.counters + CNT_SORT_ERR, s));
+        SortPlan plan;
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_HIST,
+                     sort_begin(t->ws_sort.p, t->ws_sort.bytes, t->sort_parity++, slot, n,
+                                t->slot_bits + 1, &plan, s));
+        uint32_t *kin = slot, *vin = idx, *kout = sslot, *vout = sidx;
+        for (uint32_t p = 0; p < plan.passes; ++p) {
+            HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_PASS,
+                         sort_pass(plan, p, kin, vin, kout, vout, t->d.counters + CNT_SORT_ERR, s));
+            std::swap(kin, kout);
+            std::swap(vin, vout);
+        }
+        const bool in_b = (plan.passes & 1u) != 0;
         const uint32_t* fs = in_b ? sslot : slot;
         const uint32_t* fi = in_b ? sidx : idx;
         uint4* hdr = static_cast<uint4*>(t->ws_hdr.p);

@@ -251,10 +251,10 @@ size_t sort_pairs_temp_bytes(size_t n) {
 
 size_t sort_pairs_head_bytes() { return OFF_STATUS * 4; }
 
-hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys_a,
-                      uint32_t* keys_b, uint32_t* vals_a, uint32_t* vals_b, size_t n,
-                      unsigned end_bit, bool* result_in_b, uint32_t* err_flag, hipStream_t s) {
-    *result_in_b = false;
+hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, const uint32_t* keys, size_t n,
+                      unsigned end_bit, SortPlan* plan, hipStream_t s) {
+    plan->n = 0;
+    plan->passes = 0;
     if (n == 0) return hipSuccess;
     if (n > COUNT_MASK || temp_bytes < sort_pairs_temp_bytes(n)) return hipErrorInvalidValue;
     const u32 passes = (end_bit + 7) / 8;
@@ -263,20 +263,40 @@ hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* 
     u32* words = static_cast<u32*>(temp);
     u32* head = words + (parity & 1u) * HEAD_WORDS;
     u32* next_head = words + ((parity & 1u) ^ 1u) * HEAD_WORDS;
-    u32* totals = head + HEAD_TOTALS;
-    u32* status = words + OFF_STATUS;
-    const size_t rows = n_tiles + (n_tiles + GROUP - 1) / GROUP;  // per pass: tile words, group words
-    sort_hist_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys_a, (u32)n, n_tiles, passes, totals, status,
-                                                    next_head);
+    plan->n = (u32)n;
+    plan->n_tiles = n_tiles;
+    plan->passes = passes;
+    plan->totals = head + HEAD_TOTALS;
+    plan->status = words + OFF_STATUS;
+    plan->rows = n_tiles + (n_tiles + GROUP - 1) / GROUP;  // per pass: tile words, group words
+    sort_hist_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys, (u32)n, n_tiles, passes, plan->totals,
+                                                    plan->status, next_head);
+    return hipGetLastError();
+}
+
+hipError_t sort_pass(const SortPlan& plan, unsigned p, const uint32_t* kin, const uint32_t* vin,
+                     uint32_t* kout, uint32_t* vout, uint32_t* err_flag, hipStream_t s) {
+    if (plan.n == 0) return hipSuccess;
+    if (p >= plan.passes) return hipErrorInvalidValue;
+    sort_pass_kernel<<<plan.n_tiles, SORT_BLOCK, 0, s>>>(
+        kin, vin, kout, vout, plan.n, 8 * p, plan.totals + p * RADIX,
+        p + 1 < plan.passes ? plan.totals + (p + 1) * RADIX : nullptr,
+        plan.status + (size_t)p * plan.rows * RADIX,
+        plan.status + ((size_t)p * plan.rows + plan.n_tiles) * RADIX, plan.n_tiles, err_flag);
+    return hipGetLastError();
+}
+
+hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys_a,
+                      uint32_t* keys_b, uint32_t* vals_a, uint32_t* vals_b, size_t n,
+                      unsigned end_bit, bool* result_in_b, uint32_t* err_flag, hipStream_t s) {
+    *result_in_b = false;
+    SortPlan plan;
+    hipError_t e = sort_begin(temp, temp_bytes, parity, keys_a, n, end_bit, &plan, s);
+    if (e != hipSuccess) return e;
     u32 *kin = keys_a, *vin = vals_a, *kout = keys_b, *vout = vals_b;
-    for (u32 p = 0; p < passes; ++p) {
-        sort_pass_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(kin, vin, kout, vout, (u32)n, 8 * p,
-                                                        totals + p * RADIX,
-                                                        p + 1 < passes ? totals + (p + 1) * RADIX : nullptr,
-                                                        status + (size_t)p * rows * RADIX,
-                                                        status + ((size_t)p * rows + n_tiles) * RADIX,
-                                                        n_tiles,
-                                                        err_flag);
+    for (u32 p = 0; p < plan.passes; ++p) {
+        e = sort_pass(plan, p, kin, vin, kout, vout, err_flag, s);
+        if (e != hipSuccess) return e;
         u32* tk = kin;
         u32* tv = vin;
         kin = kout;
@@ -284,8 +304,8 @@ hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* 
         kout = tk;
         vout = tv;
     }
-    *result_in_b = (passes & 1u) != 0;
-    return hipGetLastError();
+    *result_in_b = (plan.passes & 1u) != 0;
+    return hipSuccess;
 }
 
 }  // namespace pshbm

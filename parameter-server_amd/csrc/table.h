@@ -146,6 +146,18 @@ hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long l
 // and is kept zeroed by the sorts themselves as long as `parity` alternates 0,1,0,1,...
 size_t sort_pairs_temp_bytes(size_t n);
 size_t sort_pairs_head_bytes();
+// The same sort launch by launch (the histogram, then one launch per 8-bit digit p = 0 .. passes-1,
+// alternating between the two buffer pairs), for callers that time or interleave the launches.
+struct SortPlan {
+    uint32_t n, n_tiles, passes;
+    uint32_t* totals;
+    uint32_t* status;
+    size_t rows;
+};
+hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, const uint32_t* keys, size_t n,
+                      unsigned end_bit, SortPlan* plan, hipStream_t s);
+hipError_t sort_pass(const SortPlan& plan, unsigned p, const uint32_t* kin, const uint32_t* vin,
+                     uint32_t* kout, uint32_t* vout, uint32_t* err_flag, hipStream_t s);
 hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys_a,
                       uint32_t* keys_b, uint32_t* vals_a, uint32_t* vals_b, size_t n,
                       unsigned end_bit, bool* result_in_b, uint32_t* err_flag, hipStream_t s);
