@@ -46,7 +46,10 @@ KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist"
                    "gather": "gather_slots_kernel"}
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by the factors a plain
 # copy of known size gave), measured on an MI355X; the summaries are under profiles/.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    ("c2", "pull"): 191_700_000, ("c2", "locate"): 71_500_000, ("c2", "sort_hist"): 5_400_000,
+    ("c2", "sort_pass"): 21_200_000, ("c2", "segreduce"): 235_500_000, ("c2", "fixup"): 1_400_000,
+}
 
 
 def algorithmic_bytes(cfg, phase, k, u):

@@ -146,6 +146,8 @@ int32_t pshbm_push_pairs(pshbm_table* t, const void* pairs, size_t n, size_t str
 int32_t pshbm_queue(pshbm_table* t, const uint64_t* keys, const float* grads, size_t n);
 int32_t pshbm_queue_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
                         void* stream);
+/* Same, from the wire layout of a push block (see pshbm_push_pairs). */
+int32_t pshbm_queue_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride);
 /* Number of keys queued and not yet stored. */
 int32_t pshbm_queued(pshbm_table* t, uint64_t* n);
 

@@ -28,7 +28,7 @@ LOAD_UNIQUE = 1
 SYMBOLS = [
     "pshbm_create", "pshbm_destroy", "pshbm_last_error", "pshbm_value_floats",
     "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
-    "pshbm_queue", "pshbm_queue_dev", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
+    "pshbm_queue", "pshbm_queue_dev", "pshbm_queue_pairs", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
     "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
@@ -120,6 +120,7 @@ def lib():
         L.pshbm_push_pairs.argtypes = [vp, vp, sz, sz, u32]
         L.pshbm_queue.argtypes = [vp, vp, vp, sz]
         L.pshbm_queue_dev.argtypes = [vp, vp, vp, sz, vp]
+        L.pshbm_queue_pairs.argtypes = [vp, vp, sz, sz]
         L.pshbm_queued.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pshbm_store.argtypes = [vp, u32]
         L.pshbm_store_dev.argtypes = [vp, u32, vp]
@@ -215,6 +216,10 @@ class Table:
         k, g = _u64(keys), _f32(grads)
         assert g.size == k.size * self.dim
         return lib().pshbm_queue(self._h, k.ctypes.data, g.ctypes.data, k.size)
+
+    def queue_pairs(self, pairs):
+        p = np.ascontiguousarray(pairs)
+        return lib().pshbm_queue_pairs(self._h, p.ctypes.data, p.size, p.dtype.itemsize)
 
     def queued(self):
         n = C.c_uint64()

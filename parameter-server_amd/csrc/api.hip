@@ -535,20 +535,18 @@ int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, siz
     return st;
 }
 
-int32_t pshbm_push_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride, uint32_t flags) {
-    if (!t) return PSHBM_INVALID_ID;
-    if (n == 0) return PSHBM_OK;
-    if (!pairs) return fail(t, PSHBM_ERROR, "push_pairs: null buffer");
+// Copies n wire pairs {uint64 key, dim floats} to the device and splits them into the staged key
+// and gradient arrays (st_keys, st_vals). The caller holds st_mu.
+static int32_t stage_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride, const char* what) {
+    if (!pairs) return fail(t, PSHBM_ERROR, "%s: null buffer", what);
     const size_t used = 8 + (size_t)t->d.dim * 4;
-    if (stride < used || stride % 4) return fail(t, PSHBM_ERROR, "push_pairs: bad stride %zu", stride);
+    if (stride < used || stride % 4) return fail(t, PSHBM_ERROR, "%s: bad stride %zu", what, stride);
     const char* p = static_cast<const char*>(pairs);
     for (size_t i = 0; i < n; ++i) {
         uint64_t k;
         std::memcpy(&k, p + i * stride, 8);
-        if (k >= KEY_DELETED) return fail(t, PSHBM_ERROR, "push_pairs: reserved key in batch");
+        if (k >= KEY_DELETED) return fail(t, PSHBM_ERROR, "%s: reserved key in batch", what);
     }
-    DeviceGuard g(t->device);
-    std::lock_guard<std::mutex> sl(t->st_mu);
     ST_TRY(ensure(t, t->st_raw, n * stride));
     ST_TRY(ensure(t, t->st_keys, n * 8));
     ST_TRY(ensure(t, t->st_vals, n * (size_t)t->d.dim * 4));
@@ -558,9 +556,30 @@ int32_t pshbm_push_pairs(pshbm_table* t, const void* pairs, size_t n, size_t str
                                      (uint32_t)(stride / 4), t->d.dim,
                                      static_cast<uint64_t*>(t->st_keys.p),
                                      static_cast<float*>(t->st_vals.p), s));
+    return PSHBM_OK;
+}
+
+int32_t pshbm_push_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride, uint32_t flags) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    ST_TRY(stage_pairs(t, pairs, n, stride, "push_pairs"));
     int32_t st = pshbm_push_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
-                                static_cast<const float*>(t->st_vals.p), n, flags, s);
-    HIP_TRY(t, hipStreamSynchronize(s));
+                                static_cast<const float*>(t->st_vals.p), n, flags, t->stream);
+    HIP_TRY(t, hipStreamSynchronize(t->stream));
+    return st;
+}
+
+int32_t pshbm_queue_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    ST_TRY(stage_pairs(t, pairs, n, stride, "queue_pairs"));
+    int32_t st = pshbm_queue_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
+                                 static_cast<const float*>(t->st_vals.p), n, t->stream);
+    HIP_TRY(t, hipStreamSynchronize(t->stream));
     return st;
 }
 

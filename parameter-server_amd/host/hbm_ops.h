@@ -1,0 +1,412 @@
+// Host-side mirror of the pico-ps operator interface for the sparse-table path, on top of the
+// C ABI of include/pshbm.h. Each class stands where the reference class of the same role stands
+// and keeps its method names, argument order and error behaviour; only the body differs: instead
+// of walking a hash map key by key, it hands the decoded block to the HBM table.
+//
+//   HbmShardStorage        <- KVShardStorage / PoolHashMapShardStorage (storage/KVShardStorage.h:22-49, 844-952)
+//   HbmStorageOperator     <- ShardStorageOperator                     (operator/StorageOperator.h:78-158)
+//   HbmSparsePullOperator  <- SparseTablePullOperator::apply_request   (operator/SparsePullOperator.h:156-254)
+//   HbmSparsePushOperator  <- SparseTablePushOperator server halves    (operator/SparsePushOperator.h:197-416)
+//   HbmDirectPushOperator  <- DirectPushOperator                       (operator/SparsePushOperator.h:520-574)
+//   HbmDumpOperator        <- BaseKVTextFileDumpOperator::apply_request (operator/DumpOperator.h:137-183)
+//   HbmLoadOperator        <- BaseKVTextFileLoadOperator::restore      (operator/LoadOperator.h:164-213)
+//
+// The client halves (generate_request, apply_response, ...) are not here: they run in the
+// application process and are inherited unchanged from the reference's templates.
+#pragma once
+
+#include <functional>
+#include <memory>
+
+#include "../../include/pshbm.h"
+#include "standin.h"
+
+namespace pshbm_host {
+
+// op_config keys of an HBM table: dim, optimizer (sum|sgd|adagrad|ftrl), lr, init_acc, alpha, beta,
+// l1, l2, hbm_table.expected_max_items, hbm_table.max_load_factor, hbm_table.max_batch, read_only,
+// device. The learning rate lives in the operator config, as pico-ps/operator/Operator.h:55 expects.
+inline pshbm_config table_config(const Configure& c) {
+    pshbm_config cfg{};
+    cfg.struct_size = sizeof(cfg);
+    cfg.device = (int32_t)c.number("device", 0);
+    cfg.dim = (uint32_t)c.number("dim", 0);
+    const std::string opt = c.str("optimizer", "sum");
+    cfg.optimizer = opt == "sgd" ? PSHBM_OPT_SGD : opt == "adagrad" ? PSHBM_OPT_ADAGRAD
+                  : opt == "ftrl" ? PSHBM_OPT_FTRL : opt == "sum" ? PSHBM_OPT_SUM : -1;
+    cfg.lr = (float)c.number("lr", 0.0);
+    cfg.init_acc = (float)c.number("init_acc", 0.0);
+    cfg.alpha = (float)c.number("alpha", 0.0);
+    cfg.beta = (float)c.number("beta", 0.0);
+    cfg.l1 = (float)c.number("l1", 0.0);
+    cfg.l2 = (float)c.number("l2", 0.0);
+    cfg.expected_max_items = (uint64_t)c.number("hbm_table.expected_max_items", 1 << 20);
+    cfg.max_load_factor = (float)c.number("hbm_table.max_load_factor", 0.0);
+    cfg.max_batch = (uint64_t)c.number("hbm_table.max_batch", 0);
+    cfg.read_only = (int32_t)c.number("read_only", 0);
+    return cfg;
+}
+
+// One pshbm_table per local shard id, the way PmemHashMapShardStorage keeps one handle per shard
+// (storage/DCPmemory.h:400-442). HBM is volatile: need_remote_restore() is true.
+class HbmShardStorage : public Storage {
+public:
+    HbmShardStorage(const std::set<int32_t>& shard_ids, const Configure& config) : _config(config) {
+        for (int32_t id : shard_ids) PSHBM_SCHECK(create_shard(id), "create_shard failed: " + _error);
+    }
+    ~HbmShardStorage() override {
+        for (auto& p : _shards) pshbm_destroy(p.second);
+    }
+    HbmShardStorage(const HbmShardStorage&) = delete;
+    HbmShardStorage& operator=(const HbmShardStorage&) = delete;
+
+    bool need_remote_restore() override { return true; }
+    pshbm_table* get(int32_t shard_id) {
+        auto it = _shards.find(shard_id);
+        return it == _shards.end() ? nullptr : it->second;
+    }
+    bool create_shard(int32_t shard_id) {  // KVShardStorage.h:910-925
+        if (_shards.count(shard_id)) return false;
+        pshbm_config cfg = table_config(_config);
+        pshbm_table* t = nullptr;
+        int32_t st = pshbm_create(&cfg, &t);
+        if (st != PSHBM_OK) {
+            _error = pshbm_last_error(nullptr);
+            return false;
+        }
+        _shards[shard_id] = t;
+        _vf = pshbm_value_floats(cfg.dim, cfg.optimizer);
+        _dim = cfg.dim;
+        return true;
+    }
+    bool erase_shard(int32_t shard_id) {
+        auto it = _shards.find(shard_id);
+        if (it == _shards.end()) return false;
+        pshbm_destroy(it->second);
+        _shards.erase(it);
+        return true;
+    }
+    void clear() {  // KVShardStorage.h:902-908: every shard emptied, the shards stay
+        for (auto& p : _shards) pshbm_clear(p.second);
+    }
+    std::vector<int32_t> shard_list() const {
+        std::vector<int32_t> ids;
+        for (auto& p : _shards) ids.push_back(p.first);
+        return ids;
+    }
+    size_t shard_size(int32_t shard_id) {  // :927-935
+        uint64_t n = 0;
+        pshbm_size(_shards.at(shard_id), &n);
+        return n;
+    }
+    size_t shard_memory_usage(int32_t shard_id) {  // :937-946
+        uint64_t n = 0;
+        pshbm_memory_usage(_shards.at(shard_id), &n);
+        return n;
+    }
+    // KVShardIterator::iterate_batch_as_binary_archive (:64-87): records [offset, offset+batch) of a
+    // shard as {uint64 key, value} pairs appended to `ar`; returns how many (fewer than batch = end).
+    size_t iterate_batch_as_binary_archive(int32_t shard_id, size_t offset, size_t batch, BinaryArchive& ar) {
+        std::vector<char> rec(batch * record_bytes());
+        size_t got = 0;
+        int32_t st = pshbm_iterate(_shards.at(shard_id), offset, batch, rec.data(), &got);
+        PSHBM_SCHECK(st == PSHBM_OK, "iterate failed");
+        ar.write_raw(rec.data(), got * record_bytes());
+        return got;
+    }
+    uint32_t dim() const { return _dim; }
+    uint32_t value_floats() const { return _vf; }
+    size_t record_bytes() const { return 8 + (size_t)_vf * 4; }
+    const std::string& error() const { return _error; }
+
+private:
+    Configure _config;
+    std::map<int32_t, pshbm_table*> _shards;
+    uint32_t _dim = 0, _vf = 0;
+    std::string _error;
+};
+
+// Marker for the delta storage of the sync path: the queue of blocks (SizeMpscQueueShardStorage,
+// KVShardStorage.h:677-726) lives inside each shard's table.
+class HbmDeltaStorage : public Storage {};
+
+class HbmStorageOperator {
+public:
+    explicit HbmStorageOperator(const Configure& config) : _config(config) {}
+    std::unique_ptr<Storage> create_storage(RuntimeInfo& rt, int32_t /*storage_id*/) {  // StorageOperator.h:106-109
+        return std::make_unique<HbmShardStorage>(rt.local_shards(), _config);
+    }
+    void clear_storage(Storage* st) { static_cast<HbmShardStorage*>(st)->clear(); }  // :111-113
+    void apply_query_info_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp_ret) {  // :123-141
+        std::vector<StorageStatisticInfo> info;
+        auto* st = static_cast<HbmShardStorage*>(storage);
+        for (int32_t shard_id : rt.local_shards())
+            info.push_back({rt.node_id(), shard_id, st->shard_size(shard_id), st->shard_memory_usage(shard_id)});
+        PSResponse resp(req);
+        resp << info;
+        resp_ret = std::move(resp);
+    }
+
+private:
+    Configure _config;
+};
+
+// Server half of the sparse pull. Request: i32 shards_num, i32 merge_num; per shard {i32 shard_id;
+// per merged request {i32 n; if n: one lazy block of n raw uint64 keys}} (SparsePullOperator.h:132-147).
+// Response: i32 shards_num; the shard ids; then merge_num lazy blocks, block i holding the pulled
+// values of merged request i over all shards, in request order (:170-171,183,227,238-244).
+class HbmSparsePullOperator {
+public:
+    explicit HbmSparsePullOperator(const Configure& config)
+        : _read_only(config.number("read_only", 0) != 0),
+          _insert_on_miss(config.number("pull_insert_on_miss", 0) != 0) {}
+
+    void apply_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp) {
+        int32_t shards_num, merge_num;
+        req >> shards_num >> merge_num;
+        std::vector<std::vector<char>> values_ars(merge_num);
+        resp = PSResponse(req);
+        resp << shards_num;
+        bool healthy = true;
+        std::string why;
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        const size_t row_bytes = (size_t)st.dim() * 4;
+        const uint32_t flags = (_insert_on_miss && !_read_only) ? PSHBM_PULL_INSERT_ON_MISS : 0u;  // :219
+        while (shards_num--) {
+            int32_t shard_id;
+            req >> shard_id;
+            resp << shard_id;
+            PSHBM_SCHECK(rt.local_shards().count(shard_id) != 0, "Bad Request: invalid shard_id");  // :185
+            pshbm_table* t = st.get(shard_id);
+            for (int i = 0; i < merge_num; ++i) {
+                int32_t shard_keys_num;
+                req >> shard_keys_num;
+                if (shard_keys_num == 0) continue;  // :203-205: no block follows an empty count
+                std::vector<char> keys_ar;
+                ps_deserialize(req.lazy(), keys_ar);
+                PSHBM_SCHECK(keys_ar.size() == (size_t)shard_keys_num * 8, "key block size mismatch");
+                std::vector<char>& out = values_ars[i];
+                const size_t at = out.size();
+                out.resize(at + (size_t)shard_keys_num * row_bytes);
+                int32_t rc = pshbm_pull(t, reinterpret_cast<const uint64_t*>(keys_ar.data()), shard_keys_num,
+                                        reinterpret_cast<float*>(out.data() + at), nullptr, flags);
+                if (rc != PSHBM_OK) {
+                    healthy = false;
+                    why = pshbm_last_error(t);
+                }
+            }
+        }
+        if (healthy) {
+            for (auto& values_ar : values_ars) ps_serialize(resp.lazy(), std::move(values_ar));
+        } else {  // :245-253: the whole response is replaced
+            resp = PSResponse(req);
+            resp.rpc_response().set_error_code(RpcErrorCodeType::ELOGICERROR);
+            resp << Status::OOM("PServer OOM during pull: " + why);
+        }
+    }
+
+private:
+    bool _read_only, _insert_on_miss;
+};
+
+// Server halves of the sparse push. A push block is n raw std::pair<KEY, PUSH_VALUE> records, here
+// {uint64 key, dim floats} (SparsePushOperator.h:164-179, 245-247).
+class HbmSparsePushOperator {
+public:
+    explicit HbmSparsePushOperator(const Configure&) {}
+
+    // apply_async_push_request, SparsePushOperator.h:197-276. Differences, both documented in
+    // include/pshbm.h: equal keys inside one block are summed (the reference's client never sends
+    // them); a block that does not fit is refused whole and the response carries Status::OOM (the
+    // reference parks the items in the shard's overflow vector and answers OK, :257-259, :274-275).
+    void apply_async_push_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, Storage* /*incr_storage*/,
+                                  PSResponse& resp) {
+        Status status;
+        for_each_block(rt, req, storage, [&](pshbm_table* t, const std::vector<char>& block, int32_t n, size_t stride) {
+            int32_t rc = pshbm_push_pairs(t, block.data(), n, stride, 0);
+            if (rc == PSHBM_OUT_OF_MEMORY) status = Status::OOM(pshbm_last_error(t));
+            else if (rc != PSHBM_OK) status = Status::Error(pshbm_last_error(t));
+        });
+        PSHBM_SCHECK(req.archive().is_exhausted(), "request not exhausted");  // :272
+        resp = PSResponse(req);
+        if (!status.ok()) resp.rpc_response().set_error_code(RpcErrorCodeType::ELOGICERROR);
+        resp << status;
+    }
+
+    // apply_sync_push_request, :278-320: blocks are queued, nothing is merged or applied yet.
+    void apply_sync_push_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp) {
+        Status status;
+        for_each_block(rt, req, storage, [&](pshbm_table* t, const std::vector<char>& block, int32_t n, size_t stride) {
+            if (pshbm_queue_pairs(t, block.data(), n, stride) != PSHBM_OK) status = Status::Error(pshbm_last_error(t));
+        });
+        resp = PSResponse(req);
+        resp << status;
+    }
+
+    // apply_store_request, :322-416: acknowledge first (:370-372), then merge and apply.
+    void apply_store_request(RuntimeInfo& rt, PSRequest& req, Storage* delta_storage, Storage* storage,
+                             Storage* /*incr_storage*/, std::function<void(PSResponse&&)> send_response) {
+        int32_t shard_id;
+        req >> shard_id;
+        PSHBM_SCHECK(req.archive().is_exhausted(), "request not exhausted");
+        PSHBM_SCHECK(rt.local_shards().count(shard_id), "Bad Request: invalid shard_id");
+        PSResponse resp(req);
+        resp << Status();
+        send_response(std::move(resp));
+        if (delta_storage == nullptr) return;  // :336-341
+        pshbm_store(static_cast<HbmShardStorage*>(storage)->get(shard_id), 0);
+    }
+
+    std::unique_ptr<Storage> create_delta_storage(RuntimeInfo&) { return std::make_unique<HbmDeltaStorage>(); }  // :425-427
+
+private:
+    template <class F>
+    static void for_each_block(RuntimeInfo& rt, PSRequest& req, Storage* storage, F&& f) {
+        int32_t shards_num, merge_num;
+        req >> shards_num >> merge_num;
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        const size_t stride = 8 + (size_t)st.dim() * 4;
+        while (shards_num--) {
+            int32_t shard_id;
+            req >> shard_id;
+            PSHBM_SCHECK(rt.local_shards().count(shard_id) != 0, "Bad Request: invalid shard_id");
+            pshbm_table* t = st.get(shard_id);
+            for (int i = 0; i < merge_num; ++i) {
+                int32_t shard_items_num;
+                req >> shard_items_num;
+                if (shard_items_num == 0) continue;
+                std::vector<char> ar;
+                ps_deserialize(req.lazy(), ar);
+                PSHBM_SCHECK(ar.size() == (size_t)shard_items_num * stride, "push block size mismatch");
+                f(t, ar, shard_items_num, stride);
+            }
+        }
+    }
+};
+
+// DirectPushOperator::apply_async_push_request, SparsePushOperator.h:520-574: every item is
+// {key, whole value}; ht[key] = value. OOM -> ELOGICERROR + Status::OOM (:568-573).
+class HbmDirectPushOperator {
+public:
+    explicit HbmDirectPushOperator(const Configure&) {}
+    void apply_async_push_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, Storage*, PSResponse& resp) {
+        resp = PSResponse(req);
+        int32_t shards_num, merge_num;
+        req >> shards_num >> merge_num;
+        bool healthy = true;
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        while (shards_num--) {
+            int32_t shard_id;
+            req >> shard_id;
+            PSHBM_SCHECK(rt.local_shards().count(shard_id) != 0, "Bad Request: invalid shard_id");
+            for (int i = 0; i < merge_num; ++i) {
+                int32_t shard_items_num;
+                req >> shard_items_num;
+                if (shard_items_num == 0) continue;
+                std::vector<char> ar;
+                ps_deserialize(req.lazy(), ar);
+                PSHBM_SCHECK(ar.size() == (size_t)shard_items_num * st.record_bytes(), "block size mismatch");
+                if (pshbm_load(st.get(shard_id), ar.data(), shard_items_num, 0) != PSHBM_OK) healthy = false;
+            }
+        }
+        PSHBM_SCHECK(req.archive().is_exhausted(), "request not exhausted");
+        if (healthy) {
+            resp << Status();
+        } else {
+            resp.rpc_response().set_error_code(RpcErrorCodeType::ELOGICERROR);
+            resp << Status::OOM("PServer OOM during direct push");
+        }
+    }
+};
+
+struct DumpArgs {  // handler/DumpHandler.h: where to write and into how many files per node
+    std::string uri;
+    int32_t file_number = 1;
+    friend BinaryArchive& operator<<(BinaryArchive& ar, const DumpArgs& a) { return ar << a.uri << a.file_number; }
+    friend BinaryArchive& operator>>(BinaryArchive& ar, DumpArgs& a) { return ar >> a.uri >> a.file_number; }
+};
+
+// BaseKVTextFileDumpOperator::apply_request, DumpOperator.h:137-183. Request: DumpArgs, i32 file_id,
+// vector of shard ids (:66-80). DS_WRITER: bool open(const std::string&), bool write(uint64_t key,
+// const float* value, uint32_t value_floats), void close() -- the record encoding stays with the host.
+template <class DS_WRITER>
+class HbmDumpOperator {
+public:
+    explicit HbmDumpOperator(const Configure& config) : _block((size_t)config.number("block_size", 65536)) {}
+    void apply_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp_ret) {
+        DumpArgs args;
+        int32_t file_id;
+        std::vector<int32_t> shard_ids;
+        req.archive() >> args >> file_id >> shard_ids;
+        PSHBM_SCHECK(req.archive().is_exhausted(), "request not exhausted");
+        DS_WRITER writer;
+        const std::string name = args.uri + "/model_" + std::to_string(rt.node_id()) + "_" + std::to_string(file_id);  // :156
+        PSHBM_SCHECK(writer.open(name), "failed to open file for write: " + name);
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        const size_t rec = st.record_bytes();
+        for (int32_t shard_id : shard_ids) {
+            for (size_t off = 0;;) {  // the shard streams out in slab order, block by block
+                BinaryArchive ar;
+                size_t got = st.iterate_batch_as_binary_archive(shard_id, off, _block, ar);
+                for (size_t i = 0; i < got; ++i) {
+                    uint64_t key;
+                    std::memcpy(&key, ar.buffer().data() + i * rec, 8);
+                    PSHBM_SCHECK(writer.write(key, reinterpret_cast<const float*>(ar.buffer().data() + i * rec + 8),
+                                              st.value_floats()),
+                                 "failed to write");
+                }
+                off += got;
+                if (got < _block) break;
+            }
+        }
+        writer.close();
+        PSResponse resp(req);
+        resp << Status();
+        resp_ret = std::move(resp);
+    }
+
+private:
+    size_t _block;
+};
+
+// BaseKVTextFileLoadOperator::restore, LoadOperator.h:164-213: every record of the files whose key
+// belongs to a local shard is inserted, block_size records at a time; a key that is already there
+// aborts (SCHECK(insert.second), :194,210). DS_READER: bool open(const std::string&),
+// bool read(uint64_t& key, float* value). `partition` maps a key to its shard id (one shard: 0).
+template <class DS_READER>
+class HbmLoadOperator {
+public:
+    explicit HbmLoadOperator(const Configure& config) : _block_size((size_t)config.number("block_size", 1000)) {}
+    void restore(const std::vector<std::string>& files, RuntimeInfo& rt, Storage* storage,
+                 const std::function<int32_t(uint64_t)>& partition) {
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        const size_t rec = st.record_bytes();
+        std::map<int32_t, std::vector<char>> pending;
+        auto flush = [&](int32_t shard_id, std::vector<char>& buf) {
+            if (buf.empty()) return;
+            int32_t rc = pshbm_load(st.get(shard_id), buf.data(), buf.size() / rec, PSHBM_LOAD_UNIQUE);
+            PSHBM_SCHECK(rc == PSHBM_OK, std::string("restore: ") + pshbm_last_error(st.get(shard_id)));
+            buf.clear();
+        };
+        std::vector<char> one(rec);
+        for (const std::string& f : files) {
+            DS_READER reader;
+            PSHBM_SCHECK(reader.open(f), "failed to open " + f);
+            uint64_t key;
+            while (reader.read(key, reinterpret_cast<float*>(one.data() + 8))) {
+                const int32_t shard_id = partition(key);
+                if (rt.local_shards().count(shard_id) == 0) continue;  // :185-186
+                std::memcpy(one.data(), &key, 8);
+                auto& buf = pending[shard_id];
+                buf.insert(buf.end(), one.begin(), one.end());
+                if (buf.size() >= _block_size * rec) flush(shard_id, buf);
+            }
+        }
+        for (auto& p : pending) flush(p.first, p.second);
+    }
+
+private:
+    size_t _block_size;
+};
+
+}  // namespace pshbm_host

@@ -1,0 +1,295 @@
+// Drives the host-side operator mirror (parameter-server_amd/host/hbm_ops.h) the way the
+// reference's test_sparse drives its operators (pico-ps/test/ps_service_test.cpp:77-184), but in
+// one process and through hand-built wire requests: every "rank" pushes keys
+// [rank*100, (rank+1)*100) with arg = key once asynchronously and once (even ranks twice)
+// synchronously, the store is applied, the table is dumped to files, restored into a new storage,
+// and pulled. The test operator of the reference (TestValue{sum,count}, TestOps.h:53-118) is the
+// dim-2 SUM table: a push of arg = key is the gradient [key, 1].
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <iostream>
+
+#include "../../parameter-server_amd/host/hbm_ops.h"
+
+using namespace pshbm_host;
+
+static int g_failed = 0;
+#define EXPECT(cond)                                                              \
+    do {                                                                          \
+        if (!(cond)) {                                                            \
+            std::printf("EXPECT failed at line %d: %s\n", __LINE__, #cond);       \
+            ++g_failed;                                                           \
+        }                                                                         \
+    } while (0)
+
+constexpr int TEST_KEY_NUM = 100;  // pico-ps/test/TestOps.h:12
+constexpr int NUM_RANKS = 3;
+constexpr int NUM_SHARDS = 2;
+static int32_t partition(uint64_t key) { return (int32_t)(key % NUM_SHARDS); }
+
+struct Pair {  // std::pair<KEY, PUSH_VALUE> of the wire, SparsePushOperator.h:176-177
+    uint64_t key;
+    float v[2];
+};
+static_assert(sizeof(Pair) == 16, "wire pair is packed");
+
+// Client half of a push for one client batch (generate_push_request, SparsePushOperator.h:156-185).
+static PSRequest make_push_request(const std::vector<uint64_t>& keys, const std::vector<float>& args) {
+    std::vector<std::vector<Pair>> by_shard(NUM_SHARDS);
+    for (size_t i = 0; i < keys.size(); ++i) by_shard[partition(keys[i])].push_back({keys[i], {args[i], 1.0f}});
+    PSRequest req;
+    req << (int32_t)NUM_SHARDS << (int32_t)1;
+    for (int32_t s = 0; s < NUM_SHARDS; ++s) {
+        req << s << (int32_t)by_shard[s].size();
+        if (!by_shard[s].empty()) {
+            const char* p = reinterpret_cast<const char*>(by_shard[s].data());
+            req.lazy().emplace_back(p, p + by_shard[s].size() * sizeof(Pair));
+        }
+    }
+    return req;
+}
+
+// Client half of a pull (generate_request, SparsePullOperator.h:112-154) and of its response
+// (apply_response + fill_pull_items, :256-304), for one unmerged request.
+static std::vector<float> pull(HbmSparsePullOperator& op, RuntimeInfo& rt, Storage* st,
+                               const std::vector<uint64_t>& keys, bool* ok) {
+    std::vector<std::vector<uint64_t>> by_shard(NUM_SHARDS);
+    std::vector<std::vector<size_t>> where(NUM_SHARDS);
+    for (size_t i = 0; i < keys.size(); ++i) {
+        by_shard[partition(keys[i])].push_back(keys[i]);
+        where[partition(keys[i])].push_back(i);
+    }
+    PSRequest req;
+    req << (int32_t)NUM_SHARDS << (int32_t)1;
+    for (int32_t s = 0; s < NUM_SHARDS; ++s) {
+        req << s << (int32_t)by_shard[s].size();
+        if (!by_shard[s].empty()) {
+            const char* p = reinterpret_cast<const char*>(by_shard[s].data());
+            req.lazy().emplace_back(p, p + by_shard[s].size() * 8);
+        }
+    }
+    PSResponse resp;
+    op.apply_request(rt, req, st, resp);
+    std::vector<float> out(keys.size() * 2, -3.0f);
+    *ok = resp.error_code() == RpcErrorCodeType::SUCC;
+    if (!*ok) return out;
+    int32_t shards_num;
+    resp >> shards_num;
+    std::vector<int32_t> ids(shards_num);
+    for (auto& id : ids) resp >> id;
+    std::vector<char> values;
+    ps_deserialize(resp.lazy(), values);
+    const float* v = reinterpret_cast<const float*>(values.data());
+    size_t at = 0;
+    for (int32_t id : ids)
+        for (size_t i : where[id]) {
+            out[i * 2] = v[at * 2];
+            out[i * 2 + 1] = v[at * 2 + 1];
+            ++at;
+        }
+    EXPECT(at * 8 == values.size());
+    return out;
+}
+
+struct FileWriter {  // stands for TestDsWriter (pico-ps/test/TestOpsDs.h:13-45)
+    std::ofstream f;
+    bool open(const std::string& name) {
+        f.open(name, std::ios::binary);
+        return f.good();
+    }
+    bool write(uint64_t key, const float* value, uint32_t vf) {
+        f.write(reinterpret_cast<const char*>(&key), 8);
+        f.write(reinterpret_cast<const char*>(value), vf * 4);
+        return f.good();
+    }
+    void close() { f.close(); }
+};
+struct FileReader {  // stands for TestDsReader (TestOpsDs.h:47-75); dim-2 SUM values
+    std::ifstream f;
+    bool open(const std::string& name) {
+        f.open(name, std::ios::binary);
+        return f.good();
+    }
+    bool read(uint64_t& key, float* value) {
+        f.read(reinterpret_cast<char*>(&key), 8);
+        f.read(reinterpret_cast<char*>(value), 8);
+        return f.good();
+    }
+};
+
+int main(int argc, char** argv) {
+    const std::string dir = argc > 1 ? argv[1] : "/tmp";
+    Configure op_config;
+    op_config.set("dim", 2);
+    op_config.set("optimizer", "sum");
+    op_config.set("hbm_table.expected_max_items", 1000);
+    op_config.set("block_size", 100);  // ps_service_test.cpp:85
+    RuntimeInfo rt(0, {0, 1});
+
+    HbmStorageOperator storage_op(op_config);
+    std::unique_ptr<Storage> storage = storage_op.create_storage(rt, 0);
+    HbmSparsePushOperator push_op(op_config);
+    std::unique_ptr<Storage> delta = push_op.create_delta_storage(rt);
+
+    std::vector<uint64_t> all_keys;
+    for (int rank = 0; rank < NUM_RANKS; ++rank) {
+        std::vector<uint64_t> keys;
+        std::vector<float> args;
+        for (int k = rank * TEST_KEY_NUM; k < (rank + 1) * TEST_KEY_NUM; ++k) {
+            keys.push_back(k);
+            args.push_back((float)k);
+            all_keys.push_back(k);
+        }
+        PSResponse resp;
+        Status status;
+        PSRequest a = make_push_request(keys, args);  // async_push, :104
+        push_op.apply_async_push_request(rt, a, storage.get(), nullptr, resp);
+        resp >> status;
+        EXPECT(status.ok());
+        for (int rep = 0; rep < (rank % 2 == 0 ? 2 : 1); ++rep) {  // sync_push, :106-111
+            PSRequest s = make_push_request(keys, args);
+            push_op.apply_sync_push_request(rt, s, storage.get(), resp);
+            resp >> status;
+            EXPECT(status.ok());
+        }
+    }
+    // before the store only the asynchronous pushes are visible
+    {
+        bool ok;
+        HbmSparsePullOperator pull_op(op_config);
+        auto v = pull(pull_op, rt, storage.get(), all_keys, &ok);
+        EXPECT(ok);
+        for (size_t i = 0; i < all_keys.size(); ++i) EXPECT(v[i * 2] == (float)all_keys[i] && v[i * 2 + 1] == 1.0f);
+    }
+    for (int32_t shard = 0; shard < NUM_SHARDS; ++shard) {  // store, :120: one request per shard
+        PSRequest req;
+        req << shard;
+        bool acked = false;
+        push_op.apply_store_request(rt, req, delta.get(), storage.get(), nullptr, [&](PSResponse&& r) {
+            Status s;
+            r >> s;
+            acked = s.ok();
+        });
+        EXPECT(acked);
+    }
+    auto total_size = [&](Storage* st) {
+        PSRequest req;
+        PSResponse resp;
+        storage_op.apply_query_info_request(rt, req, st, resp);
+        std::vector<StorageStatisticInfo> info;
+        resp.archive() >> info;
+        uint64_t n = 0;
+        for (auto& i : info) {
+            n += i.item_number;
+            EXPECT(i.memory_usage > 0);
+        }
+        return n;
+    };
+    EXPECT(total_size(storage.get()) == (uint64_t)TEST_KEY_NUM * NUM_RANKS);  // :122
+
+    // dump with file_number = 2 (:125-127): shard -> file by shard_id % file_number
+    HbmDumpOperator<FileWriter> dump_op(op_config);
+    std::vector<std::string> files;
+    for (int32_t file_id = 0; file_id < 2; ++file_id) {
+        PSRequest req;
+        DumpArgs args{dir, 2};
+        std::vector<int32_t> shard_ids;
+        for (int32_t s = 0; s < NUM_SHARDS; ++s)
+            if (s % 2 == file_id) shard_ids.push_back(s);
+        req.archive() << args << file_id << shard_ids;
+        PSResponse resp;
+        dump_op.apply_request(rt, req, storage.get(), resp);
+        Status s;
+        resp >> s;
+        EXPECT(s.ok());
+        files.push_back(dir + "/model_0_" + std::to_string(file_id));
+    }
+
+    // a new storage, restore (no rehash, :150-156), clear, restore again
+    std::unique_ptr<Storage> storage2 = storage_op.create_storage(rt, 1);
+    HbmLoadOperator<FileReader> load_op(op_config);
+    load_op.restore(files, rt, storage2.get(), partition);
+    EXPECT(total_size(storage2.get()) == (uint64_t)TEST_KEY_NUM * NUM_RANKS);
+    storage_op.clear_storage(storage2.get());
+    EXPECT(total_size(storage2.get()) == 0);  // :153-154
+    load_op.restore(files, rt, storage2.get(), partition);
+    EXPECT(total_size(storage2.get()) == (uint64_t)TEST_KEY_NUM * NUM_RANKS);
+    bool threw = false;  // restoring keys that are present aborts (LoadOperator.h:194,210)
+    try {
+        load_op.restore(files, rt, storage2.get(), partition);
+    } catch (const std::logic_error&) {
+        threw = true;
+    }
+    EXPECT(threw);
+
+    // pulls, several times (:204-213): key * (2 + (rank even)); a missing key pulls 0 and is not inserted
+    HbmSparsePullOperator pull_op(op_config);
+    std::vector<uint64_t> q = all_keys;
+    for (int i = 0; i < 10; ++i) q.push_back(TEST_KEY_NUM * NUM_RANKS + i);
+    for (int rep = 0; rep < 3; ++rep) {
+        for (Storage* st : {storage.get(), storage2.get()}) {
+            bool ok;
+            auto v = pull(pull_op, rt, st, q, &ok);
+            EXPECT(ok);
+            for (size_t i = 0; i < q.size(); ++i) {
+                const uint64_t key = q[i];
+                const int rank = (int)(key / TEST_KEY_NUM);
+                const float count = key < (uint64_t)TEST_KEY_NUM * NUM_RANKS ? 2.0f + (rank % 2 == 0) : 0.0f;
+                EXPECT(v[i * 2] == (float)key * count && v[i * 2 + 1] == count);
+            }
+        }
+    }
+    EXPECT(total_size(storage.get()) == (uint64_t)TEST_KEY_NUM * NUM_RANKS);
+
+    // direct push overwrites whole values (SparsePushOperator.h:557-562)
+    {
+        HbmDirectPushOperator direct(op_config);
+        std::vector<Pair> items = {{0, {7.0f, 8.0f}}, {1, {9.0f, 10.0f}}, {1000, {1.0f, 2.0f}}};
+        PSRequest req;
+        req << (int32_t)NUM_SHARDS << (int32_t)1;
+        for (int32_t s = 0; s < NUM_SHARDS; ++s) {
+            std::vector<Pair> mine;
+            for (auto& it : items)
+                if (partition(it.key) == s) mine.push_back(it);
+            req << s << (int32_t)mine.size();
+            if (!mine.empty()) {
+                const char* p = reinterpret_cast<const char*>(mine.data());
+                req.lazy().emplace_back(p, p + mine.size() * sizeof(Pair));
+            }
+        }
+        PSResponse resp;
+        direct.apply_async_push_request(rt, req, storage.get(), nullptr, resp);
+        Status s;
+        resp >> s;
+        EXPECT(s.ok());
+        bool ok;
+        auto v = pull(pull_op, rt, storage.get(), {0, 1, 1000, 2}, &ok);
+        EXPECT(v[0] == 7.0f && v[1] == 8.0f && v[2] == 9.0f && v[3] == 10.0f && v[4] == 1.0f && v[5] == 2.0f);
+        EXPECT(v[6] == 6.0f && v[7] == 3.0f);  // key 2, rank 0: 2 * 3
+    }
+
+    // a push that does not fit answers OOM and leaves the table as it was
+    {
+        std::vector<uint64_t> keys;
+        std::vector<float> args;
+        for (int k = 0; k < 2000; ++k) {
+            keys.push_back(100000 + k);
+            args.push_back(1.0f);
+        }
+        PSRequest req = make_push_request(keys, args);
+        PSResponse resp;
+        push_op.apply_async_push_request(rt, req, storage.get(), nullptr, resp);
+        Status s;
+        resp >> s;
+        EXPECT(s.IsOOM() && resp.error_code() == RpcErrorCodeType::ELOGICERROR);
+        EXPECT(total_size(storage.get()) == (uint64_t)TEST_KEY_NUM * NUM_RANKS + 1);
+    }
+
+    if (g_failed) {
+        std::printf("FAILED: %d expectation(s)\n", g_failed);
+        return 1;
+    }
+    std::printf("PASS test_hbm_operators\n");
+    return 0;
+}
