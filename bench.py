@@ -42,7 +42,7 @@ CONFIGS = {
 STATE_BLOCKS = {0: 1, 1: 1, 2: 2, 3: 3}
 KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist": "sort_hist_kernel",
                    "sort_pass": "sort_pass_kernel", "segreduce": "segreduce_kernel",
-                   "fixup": "fixup_kernel", "update_unique": "update_unique_kernel",
+                   "fixup": "fixup_kernel", "fixup_windows": "fixup_windows_kernel", "update_unique": "update_unique_kernel",
                    "gather": "gather_slots_kernel"}
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by the factors a plain
 # copy of known size gave), measured on an MI355X; the summaries are under profiles/.
@@ -68,7 +68,7 @@ def algorithmic_bytes(cfg, phase, k, u):
 
 def build_table(ps, wl, torch, cfg, n_table, seed=0):
     dim = cfg["dim"]
-    cap = n_table + max(n_table // 4, 32 * cfg["batch"])
+    cap = n_table + max(n_table // 16, 8 * cfg["batch"])   # room for keys that pushes insert
     t = ps.Table(dim, capacity=cap, max_batch=cfg["batch"], **cfg["opt"])
     vf = t.value_floats
     stream = torch.cuda.current_stream().cuda_stream

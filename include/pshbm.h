@@ -208,7 +208,8 @@ int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out);
 #define PSHBM_PHASE_UPDATE_UNIQUE 5 /* update of a batch declared duplicate-free */
 #define PSHBM_PHASE_GATHER 6        /* row gather of an inserting pull */
 #define PSHBM_PHASE_SORT_PASS 7     /* radix sort of (slot, index): one 8-bit digit pass */
-#define PSHBM_PHASES 8
+#define PSHBM_PHASE_FIXUP_WINDOWS 8 /* window sums of runs that span many chunks */
+#define PSHBM_PHASES 12
 typedef struct pshbm_profile {
     double ms[PSHBM_PHASES];
     uint64_t launches[PSHBM_PHASES];

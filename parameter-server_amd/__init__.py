@@ -33,7 +33,8 @@ SYMBOLS = [
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
-PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass"]
+PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
+          "fixup_windows"]
 
 
 class Config(C.Structure):
@@ -68,7 +69,7 @@ class Stats(C.Structure):
 
 
 class Profile(C.Structure):
-    _fields_ = [("ms", C.c_double * 8), ("launches", C.c_uint64 * 8)]
+    _fields_ = [("ms", C.c_double * 12), ("launches", C.c_uint64 * 12)]
 
 
 class PshbmError(RuntimeError):

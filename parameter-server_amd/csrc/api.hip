@@ -45,7 +45,7 @@ struct pshbm_table {
     // per-batch workspace of the mutating paths
     size_t ws_cap = 0;
     unsigned sort_parity = 0;  // which half of the sort head the next sort uses
-    DevBuf ws_slot, ws_idx, ws_sslot, ws_sidx, ws_sort, ws_hdr, ws_pval;
+    DevBuf ws_slot, ws_idx, ws_sslot, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wslot, ws_wval;
 
     // staging of the host-pointer entry points
     std::mutex st_mu;
@@ -172,6 +172,8 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     size_t chunks = std::max(g1.n_chunks, g4.n_chunks);
     ST_TRY(ensure(t, t->ws_hdr, chunks * sizeof(uint4)));
     ST_TRY(ensure(t, t->ws_pval, chunks * 2 * (size_t)t->d.dim * 4));
+    ST_TRY(ensure(t, t->ws_wslot, (chunks / 64 + 1) * 4));
+    ST_TRY(ensure(t, t->ws_wval, (chunks / 64 + 1) * (size_t)t->d.dim * 4));
     t->ws_cap = cap;
     return PSHBM_OK;
 }
@@ -278,7 +280,11 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
         float* pval = static_cast<float*>(t->ws_pval.p);
         HIP_TRY_PROF(t, s, PSHBM_PHASE_SEGREDUCE,
                      launch_segreduce(t->d, fs, fi, n, d_grads, hdr, pval, s));
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP, launch_fixup(t->d, n, d_grads, hdr, pval, s));
+        uint32_t* wslot = static_cast<uint32_t*>(t->ws_wslot.p);
+        float* wval = static_cast<float*>(t->ws_wval.p);
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP_WINDOWS,
+                     launch_fixup_windows(t->d, n, d_grads, hdr, pval, wslot, wval, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP, launch_fixup(t->d, n, d_grads, hdr, pval, wslot, wval, s));
     }
     return PSHBM_OK;
 }
@@ -313,7 +319,7 @@ void destroy_impl(pshbm_table* t) {
     DeviceGuard g(t->device);
     (void)hipDeviceSynchronize();
     DevBuf* bufs[] = {&t->ws_slot, &t->ws_idx,  &t->ws_sslot, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
-                      &t->ws_pval, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
+                      &t->ws_pval, &t->ws_wslot, &t->ws_wval, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
         if (b->p) (void)hipFree(b->p);

@@ -438,16 +438,70 @@ __device__ __forceinline__ float4 vshfl_down(float4 v, u32 d) {
                        __shfl_down(v.w, d));
 }
 
+// A key repeated hundreds of thousands of times in a batch spans thousands of chunks. So that the
+// wavefront that joins its partial sums need not visit every one of them, a first pass looks at
+// windows of 64 chunks: if all 64 chunks of a window lie inside one run (each chunk is a single run
+// that is open on both sides), their partial sums are added up into win_val[window] and
+// win_slot[window] names the run's slot; any other window gets SLOT_NONE.
+constexpr u32 WINDOW = 64;
+
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void fixup_windows_kernel(const uint4* __restrict__ part_hdr,
+                                                               const T* __restrict__ part_val,
+                                                               u32* __restrict__ win_slot,
+                                                               T* __restrict__ win_val, u32 units,
+                                                               u32 lp_full, u32 P, u32 n_chunks,
+                                                               u32 n_windows) {
+    const u32 lane = threadIdx.x & 63u;
+    const u32 v = blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
+    if (v >= n_windows) return;
+    const u32 x = v * WINDOW + lane;
+    bool through = false;
+    u32 sl = SLOT_NONE;
+    if (x < n_chunks) {
+        const uint4 h = part_hdr[x];
+        through = (h.y & 1u) && !(h.y & 2u) && !(h.w & 1u);
+        sl = h.x;
+    }
+    const u32 s0 = __shfl(sl, 0);
+    const bool whole = __ballot(through && sl == s0) == ~0ull;
+    if (!whole) {
+        if (lane == 0 && blockIdx.y == 0) win_slot[v] = SLOT_NONE;
+        return;
+    }
+    const u32 col0 = blockIdx.y * 64u;
+    const u32 lp = (units - col0) < 64u ? (units - col0) : 64u;
+    const u32 g = lane / lp_full;
+    const u32 c = lane - g * lp_full;
+    const bool lane_on = g < P && c < lp;
+    const u32 col = col0 + c;
+    T acc = vzero(T());
+    if (lane_on)
+        for (u64 y = (u64)v * WINDOW + g; y < (u64)(v + 1) * WINDOW; y += P)
+            acc = vadd(acc, part_val[(y * 2) * units + col]);
+    u32 top = 1;
+    while (top < P) top <<= 1;
+    for (u32 off = top >> 1; off >= 1; off >>= 1) {
+        T o = vshfl_down(acc, off * lp_full);
+        if (g + off < P) acc = vadd(acc, o);
+    }
+    if (lane_on && g == 0) win_val[(u64)v * units + col] = acc;
+    if (lane == 0 && blockIdx.y == 0) win_slot[v] = s0;
+}
+
 // Joins the partial sums of runs that cross chunk borders. One wavefront per chunk: if a run
 // leaves that chunk to the right, the wavefront finds where the run ends (the first following
-// chunk whose left entry is marked as the run's end), its P lane groups add the left entries of
-// the chunks in between in a strided fashion, a shuffle tree joins the P sums, and group 0
-// applies the step. The order of the additions depends only on the chunk layout, so results
-// repeat from run to run.
+// chunk whose left entry is marked as the run's end; whole windows of the run are skipped through
+// win_slot), its P lane groups add, in a strided fashion, the left entries of the chunks in
+// between -- window sums where a window lies wholly inside the run --, a shuffle tree joins the P
+// sums, and group 0 applies the step. The order of the additions depends only on the chunk
+// layout, so results repeat from run to run.
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* __restrict__ part_hdr,
-                                                       const T* __restrict__ part_val, u32 units,
-                                                       u32 lp_full, u32 P, u32 n_chunks) {
+                                                       const T* __restrict__ part_val,
+                                                       const u32* __restrict__ win_slot,
+                                                       const T* __restrict__ win_val, u32 units,
+                                                       u32 lp_full, u32 P, u32 n_chunks, u32 n_windows) {
     const u32 lane = threadIdx.x & 63u;
     const u32 w = blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
     if (w >= n_chunks) return;
@@ -459,12 +513,16 @@ __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* _
     const u32 c = lane - g * lp_full;
     const bool lane_on = g < P && c < lp;
     const u32 col = col0 + c;
-    // last chunk of the run: 64 headers per step
+    // last chunk of the run
     u32 last = w;
-    for (u32 base = w + 1; base < n_chunks; base += 64) {
-        const u32 x = base + lane;
-        bool ends = false, brk = true;
-        if (x < n_chunks) {
+    u32 x0 = w + 1;
+    bool found = false;
+    while (!found && x0 < n_chunks) {
+        // the rest of x0's window, a header per lane
+        const u32 wend = (x0 / WINDOW + 1) * WINDOW < n_chunks ? (x0 / WINDOW + 1) * WINDOW : n_chunks;
+        const u32 x = x0 + lane;
+        bool ends = false, brk = false;
+        if (x < wend) {
             const uint4 hx = part_hdr[x];
             const bool same = (hx.y & 1u) && hx.x == h.z;
             ends = same && (hx.y & 2u);
@@ -474,15 +532,39 @@ __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* _
         const u64 any = em | bm;
         if (any) {
             const u32 f = (u32)__ffsll((unsigned long long)any) - 1u;
-            last = ((em >> f) & 1ull) ? base + f : base + f - 1u;
+            last = ((em >> f) & 1ull) ? x0 + f : x0 + f - 1u;
+            found = true;
             break;
         }
-        last = base + 63u;
+        last = wend - 1u;
+        x0 = wend;
+        // whole windows of this run, 64 window words per step
+        while (x0 < n_chunks) {
+            const u32 vv = x0 / WINDOW + lane;
+            const bool mine = vv < n_windows && win_slot[vv] == h.z;
+            const u64 nm = ~__ballot(mine);
+            const u32 k = nm ? (u32)__ffsll((unsigned long long)nm) - 1u : 64u;
+            if (k) {
+                x0 += k * WINDOW;
+                last = x0 - 1u;
+            }
+            if (k < 64u) break;
+        }
     }
+    // sum: R entry of w, then the L entries of w+1 .. last
+    const u64 A = (u64)w + 1, B = last;
+    const u64 fs = (A + WINDOW - 1) / WINDOW * WINDOW;  // first window start at or after A
+    const u64 fe = B / WINDOW * WINDOW;                 // start of B's window
     T acc = vzero(T());
     if (lane_on) {
         if (g == 0) acc = part_val[((u64)w * 2 + 1) * units + col];
-        for (u64 x = (u64)w + 1 + g; x <= last; x += P) acc = vadd(acc, part_val[(x * 2) * units + col]);
+        if (fs >= fe) {
+            for (u64 x = A + g; x <= B; x += P) acc = vadd(acc, part_val[(x * 2) * units + col]);
+        } else {
+            for (u64 x = A + g; x < fs; x += P) acc = vadd(acc, part_val[(x * 2) * units + col]);
+            for (u64 v = fs / WINDOW + g; v < fe / WINDOW; v += P) acc = vadd(acc, win_val[v * units + col]);
+            for (u64 x = fe + g; x <= B; x += P) acc = vadd(acc, part_val[(x * 2) * units + col]);
+        }
     }
     u32 top = 1;
     while (top < P) top <<= 1;
@@ -677,19 +759,38 @@ hipError_t launch_segreduce(const TableDev& t, const u32* sorted_slot, const u32
     return hipGetLastError();
 }
 
-hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
-                        const float* part_val, hipStream_t s) {
+hipError_t launch_fixup_windows(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
+                                const float* part_val, u32* win_slot, float* win_val, hipStream_t s) {
     if (n == 0) return hipSuccess;
-    const bool v4 = vec4_ok(t, grads, part_val);  // the layout launch_segreduce chose
+    const bool v4 = vec4_ok(t, grads, part_val) && vec4_ok(t, win_val);  // the layout launch_segreduce chose
     const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
+    const u32 n_windows = (g.n_chunks + WINDOW - 1) / WINDOW;
+    dim3 grid((n_windows + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per window
+    if (v4)
+        fixup_windows_kernel<float4><<<grid, BLOCK, 0, s>>>(
+            part_hdr, reinterpret_cast<const float4*>(part_val), win_slot,
+            reinterpret_cast<float4*>(win_val), g.units, g.lp, g.p, g.n_chunks, n_windows);
+    else
+        fixup_windows_kernel<float><<<grid, BLOCK, 0, s>>>(part_hdr, part_val, win_slot, win_val,
+                                                           g.units, g.lp, g.p, g.n_chunks, n_windows);
+    return hipGetLastError();
+}
+
+hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
+                        const float* part_val, const u32* win_slot, const float* win_val,
+                        hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const bool v4 = vec4_ok(t, grads, part_val) && vec4_ok(t, win_val);
+    const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
+    const u32 n_windows = (g.n_chunks + WINDOW - 1) / WINDOW;
     dim3 grid((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per chunk
     if (v4)
-        fixup_kernel<float4><<<grid, BLOCK, 0, s>>>(t, part_hdr,
-                                                    reinterpret_cast<const float4*>(part_val),
-                                                    g.units, g.lp, g.p, g.n_chunks);
+        fixup_kernel<float4><<<grid, BLOCK, 0, s>>>(
+            t, part_hdr, reinterpret_cast<const float4*>(part_val), win_slot,
+            reinterpret_cast<const float4*>(win_val), g.units, g.lp, g.p, g.n_chunks, n_windows);
     else
-        fixup_kernel<float><<<grid, BLOCK, 0, s>>>(t, part_hdr, part_val, g.units, g.lp, g.p,
-                                                   g.n_chunks);
+        fixup_kernel<float><<<grid, BLOCK, 0, s>>>(t, part_hdr, part_val, win_slot, win_val, g.units,
+                                                   g.lp, g.p, g.n_chunks, n_windows);
     return hipGetLastError();
 }
 

@@ -113,8 +113,15 @@ hipError_t launch_rollback(const TableDev& t, const uint32_t* slot_idx, size_t n
 hipError_t launch_segreduce(const TableDev& t, const uint32_t* sorted_slot, const uint32_t* sorted_idx,
                             size_t n, const float* grads, uint4* part_hdr, float* part_val,
                             hipStream_t s);
+// launch_fixup_windows first adds up every window of 64 chunks that lies wholly inside one run
+// (win_slot: n_chunks/64 + 1 words, win_val: as many rows of dim floats), so that launch_fixup can
+// cross such a run a window at a time.
+hipError_t launch_fixup_windows(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
+                                const float* part_val, uint32_t* win_slot, float* win_val,
+                                hipStream_t s);
 hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
-                        const float* part_val, hipStream_t s);
+                        const float* part_val, const uint32_t* win_slot, const float* win_val,
+                        hipStream_t s);
 
 // One optimizer step per located key, no aggregation (keys distinct).
 hipError_t launch_update_unique(const TableDev& t, const uint32_t* slot_idx, size_t n,

@@ -136,11 +136,15 @@ def test_aggregation_exact_with_integer_gradients(ps, orc, dim):
         g = rng.integers(-3, 4, (n, dim)).astype(np.float32)
         assert t.push(keys, g) == 0 and r.push(keys, g) == 0
     assert_same_table(t, r, exact=True)
-    # one key only: a single run spanning every chunk of the segmented reduction
-    keys = np.full(9000, 77, np.uint64)
-    g = rng.integers(-3, 4, (9000, dim)).astype(np.float32)
-    assert t.push(keys, g) == 0 and r.push(keys, g) == 0
-    assert_same_table(t, r, exact=True)
+    # one key only: a single run spanning every chunk of the segmented reduction; the long one also
+    # spans many 64-chunk windows of the border fix-up, and shares the batch with two more long runs
+    for n in (9000, 150000):
+        keys = np.full(n, 77, np.uint64)
+        keys[n // 2: n // 2 + n // 5] = 78
+        keys[: n // 7] = 1999
+        g = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+        assert t.push(keys, g) == 0 and r.push(keys, g) == 0
+        assert_same_table(t, r, exact=True)
     t.close()
 
 
