@@ -209,6 +209,7 @@ int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out);
 #define PSHBM_PHASE_GATHER 6        /* row gather of an inserting pull */
 #define PSHBM_PHASE_SORT_PASS 7     /* radix sort of (slot, index): one 8-bit digit pass */
 #define PSHBM_PHASE_FIXUP_WINDOWS 8 /* window sums of runs that span many chunks */
+#define PSHBM_PHASE_ASSIGN_ROWS 9   /* rows for the slots an inserting operation claimed */
 #define PSHBM_PHASES 12
 typedef struct pshbm_profile {
     double ms[PSHBM_PHASES];

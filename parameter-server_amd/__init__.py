@@ -34,7 +34,7 @@ SYMBOLS = [
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
-          "fixup_windows"]
+          "fixup_windows", "assign_rows"]
 
 
 class Config(C.Structure):

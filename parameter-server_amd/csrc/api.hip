@@ -45,7 +45,8 @@ struct pshbm_table {
     // per-batch workspace of the mutating paths
     size_t ws_cap = 0;
     unsigned sort_parity = 0;  // which half of the sort head the next sort uses
-    DevBuf ws_slot, ws_idx, ws_sslot, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wslot, ws_wval;
+    DevBuf ws_slot, ws_idx, ws_sslot, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wslot, ws_wval, ws_won;
+    unsigned won_parity = 0;  // which half of ws_won the next inserting operation counts into
 
     // staging of the host-pointer entry points
     std::mutex st_mu;
@@ -174,6 +175,10 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     ST_TRY(ensure(t, t->ws_pval, chunks * 2 * (size_t)t->d.dim * 4));
     ST_TRY(ensure(t, t->ws_wslot, (chunks / 64 + 1) * 4));
     ST_TRY(ensure(t, t->ws_wval, (chunks / 64 + 1) * (size_t)t->d.dim * 4));
+    // winner counts per 1024-key block, two arrays used by alternate operations, zero between uses
+    ST_TRY(ensure(t, t->ws_won, 2 * (assign_blocks(cap) + 1) * 4));
+    HIP_TRY(t, hipMemset(t->ws_won.p, 0, t->ws_won.bytes));
+    t->won_parity = 0;
     t->ws_cap = cap;
     return PSHBM_OK;
 }
@@ -242,6 +247,26 @@ bool has_reserved_key(const uint64_t* keys, size_t n) {
     return bad != 0;
 }
 
+// The probe of a mutating operation: slots of the keys, claiming one for each missing key when
+// `insert`, followed by the launch that gives the claimed slots their rows. The two arrays of
+// per-block winner counts alternate: each operation counts into one and zeroes the other.
+int32_t locate_and_assign(pshbm_table* t, const uint64_t* d_keys, size_t n, uint32_t* slot, uint32_t* idx,
+                          bool insert, bool init_rows, bool count_dups, hipStream_t s) {
+    if (!insert) {
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE,
+                     launch_locate(t->d, d_keys, n, slot, idx, nullptr, count_dups, s));
+        return PSHBM_OK;
+    }
+    const size_t half = t->ws_won.bytes / 8;  // words per array
+    uint32_t* cur = static_cast<uint32_t*>(t->ws_won.p) + (t->won_parity & 1u) * half;
+    uint32_t* next = static_cast<uint32_t*>(t->ws_won.p) + ((t->won_parity & 1u) ^ 1u) * half;
+    ++t->won_parity;
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE, launch_locate(t->d, d_keys, n, slot, idx, cur, count_dups, s));
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_ASSIGN_ROWS,
+                 launch_assign_rows(t->d, d_keys, n, slot, cur, next, half, init_rows, s));
+    return PSHBM_OK;
+}
+
 int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
                     uint32_t flags, hipStream_t s) {
     if (n == 0) return PSHBM_OK;
@@ -254,8 +279,7 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
     if (insert) ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
     uint32_t* idx = static_cast<uint32_t*>(t->ws_idx.p);
-    HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE,
-                 launch_locate(t->d, d_keys, n, slot, unique ? nullptr : idx, insert, true, false, s));
+    ST_TRY(locate_and_assign(t, d_keys, n, slot, unique ? nullptr : idx, insert, true, false, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
     if (unique) {
         HIP_TRY_PROF(t, s, PSHBM_PHASE_UPDATE_UNIQUE, launch_update_unique(t->d, slot, n, d_grads, s));
@@ -298,7 +322,7 @@ int32_t set_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_values
     uint32_t rows_before = 0;
     ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
-    HIP_TRY(t, launch_locate(t->d, d_keys, n, slot, nullptr, true, false, count_dups, s));
+    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, true, false, count_dups, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
     HIP_TRY(t, launch_write_values(t->d, slot, n, d_values, s));
     return PSHBM_OK;
@@ -319,7 +343,7 @@ void destroy_impl(pshbm_table* t) {
     DeviceGuard g(t->device);
     (void)hipDeviceSynchronize();
     DevBuf* bufs[] = {&t->ws_slot, &t->ws_idx,  &t->ws_sslot, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
-                      &t->ws_pval, &t->ws_wslot, &t->ws_wval, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
+                      &t->ws_pval, &t->ws_wslot, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
         if (b->p) (void)hipFree(b->p);
@@ -480,9 +504,7 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     uint32_t rows_before = 0;
     ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
-    HIP_TRY(t, launch_snapshot_entry(t->d, s));
-    HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE,
-                 launch_locate(t->d, d_keys, n, slot, nullptr, true, true, false, s));
+    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, true, true, false, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
     HIP_TRY_PROF(t, s, PSHBM_PHASE_GATHER, launch_gather_slots(t->d, slot, n, d_out_rows, d_hit, s));
     return PSHBM_OK;

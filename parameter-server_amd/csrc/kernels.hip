@@ -16,6 +16,8 @@ namespace {
 
 constexpr int BLOCK = 256;  // 4 wavefronts
 constexpr u32 KEYS_PER_ROUND = 16;
+constexpr u32 WON_BIT = 0x80000000u;  // in a located slot index: this key claimed the slot in this launch
+constexpr u32 ASSIGN_KEYS = 1024;     // keys per workgroup of assign_rows_kernel
 
 // ---- small vector helpers ------------------------------------------------------------------
 __device__ __forceinline__ float vzero(float) { return 0.0f; }
@@ -163,12 +165,15 @@ __global__ __launch_bounds__(BLOCK) void gather_slots_kernel(TableDev t,
 template <bool kInsert>
 __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __restrict__ keys,
                                                         u32 n, u32* __restrict__ slot_out,
-                                                        u32* __restrict__ idx_out, int init_rows,
+                                                        u32* __restrict__ idx_out,
+                                                        u32* __restrict__ won_count,
                                                         int count_dups) {
     const u32 lane = threadIdx.x & 63u;
     const u32 grp = lane >> 2, sub = lane & 3u;
     const u64 wave = ((u64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
     const u64 nwaves = ((u64)gridDim.x * BLOCK) >> 6;
+    // the row count as it is when this operation begins (nothing in this launch changes it)
+    if (kInsert && blockIdx.x == 0 && threadIdx.x == 0) t.counters[CNT_ENTRY] = t.counters[CNT_ROWS];
     for (u64 base = wave * KEYS_PER_ROUND; base < n; base += nwaves * KEYS_PER_ROUND) {
         u64 i = base + grp;
         bool inb = i < n;
@@ -229,32 +234,13 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
                     }
                 }
             }
-            // Rows for the winners: one atomic per wavefront.
-            u64 wm = __ballot(won && sub == 0);
-            if (wm) {
-                u32 first = 0;
-                if (lane == 0) first = atomicAdd(&t.counters[CNT_ROWS], (u32)__popcll(wm));
-                first = __shfl(first, 0);
-                if (won) {
-                    u32 rank = (u32)__popcll(wm & ((1ull << (grp * 4)) - 1ull));
-                    u32 rid = first + rank;
-                    if (rid < t.max_rows) {
-                        if (sub == 0) {
-                            reinterpret_cast<u32*>(&t.slots[slot])[2] = rid;
-                            t.row_keys[rid] = key;
-                        }
-                        if (init_rows) {
-                            float4* r4 = reinterpret_cast<float4*>(t.rows + (u64)rid * t.stride_f);
-                            for (u32 c = sub; c < t.stride_f / 4; c += 4) {
-                                u32 f = c * 4;
-                                r4[c] = make_float4(init_float(t, f), init_float(t, f + 1),
-                                                    init_float(t, f + 2), init_float(t, f + 3));
-                            }
-                        }
-                    } else if (sub == 0) {
-                        t.counters[CNT_OVERFLOW] = 1u;
-                    }
-                }
+            // The group that claimed the slot only marks it and counts itself in its 1024-key
+            // block: rows are handed out afterwards by assign_rows_kernel. (One shared row counter
+            // bumped from here costs a device-scope atomic on one address per wavefront, which
+            // serialises: 1.5 ms for 200,000 inserts.)
+            if (won && sub == 0) {
+                atomicAdd(&won_count[i / ASSIGN_KEYS], 1u);
+                slot |= WON_BIT;
             }
         }
         if (inb && sub == 0) {
@@ -265,7 +251,84 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
     }
 }
 
-__global__ void snapshot_entry_kernel(TableDev t) { t.counters[CNT_ENTRY] = t.counters[CNT_ROWS]; }
+// Dense row ids for the slots that locate_kernel<true> claimed (slot_idx[i] carries WON_BIT).
+// Workgroup b owns keys [b * ASSIGN_KEYS, (b+1) * ASSIGN_KEYS); won_count[b] is how many of them
+// won. Its first row is CNT_ENTRY + the counts of the workgroups before it (summed here: a few
+// thousand words at most), then winners are numbered in (round, thread) order with ballots. The
+// rows are initialised, row_keys and the slot's row word are written, WON_BIT is cleared.
+// Workgroup 0 publishes the new row count; every workgroup zeroes its word of `won_next`, the
+// array the next operation counts into. Rows past the capacity raise CNT_OVERFLOW and stay unset.
+__global__ __launch_bounds__(BLOCK) void assign_rows_kernel(TableDev t, const u64* __restrict__ keys,
+                                                             u32 n, u32* __restrict__ slot_idx,
+                                                             const u32* __restrict__ won_count,
+                                                             u32* __restrict__ won_next, u32 won_words,
+                                                             u32 n_blocks, int init_rows) {
+    __shared__ u32 red[BLOCK / 64];
+    __shared__ u32 wave_cnt[ASSIGN_KEYS / BLOCK][BLOCK / 64];
+    const u32 b = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    for (u32 x = b * BLOCK + tid; x < won_words; x += gridDim.x * BLOCK) won_next[x] = 0;
+    const u32 mine = won_count[b];
+    if (mine == 0 && b != 0) return;  // block-uniform
+    // winners in the workgroups before this one (workgroup 0: in all of them, for the new total)
+    const u32 upto = b == 0 ? n_blocks : b;
+    u32 part = 0;
+    for (u32 x = tid; x < upto; x += BLOCK) part += won_count[x];
+    for (u32 off = 32; off >= 1; off >>= 1) part += __shfl_down(part, off);
+    if (lane == 0) red[w] = part;
+    __syncthreads();
+    u32 sum = 0;
+    for (u32 x = 0; x < BLOCK / 64; ++x) sum += red[x];
+    const u32 entry = t.counters[CNT_ENTRY];
+    if (b == 0) {
+        if (tid == 0) {
+            t.counters[CNT_ROWS] = entry + sum;
+            if (entry + sum > t.max_rows) t.counters[CNT_OVERFLOW] = 1u;
+        }
+        if (mine == 0) return;
+        sum = 0;
+    }
+    const u32 first_row = entry + sum;
+    // number the winners of this workgroup
+    u32 s[ASSIGN_KEYS / BLOCK];
+    u32 before[ASSIGN_KEYS / BLOCK];
+    const u64 lt_mask = (1ull << lane) - 1ull;
+#pragma unroll
+    for (u32 j = 0; j < ASSIGN_KEYS / BLOCK; ++j) {
+        const u64 i = (u64)b * ASSIGN_KEYS + j * BLOCK + tid;
+        s[j] = i < n ? slot_idx[i] : SLOT_NONE;
+        const bool won = s[j] != SLOT_NONE && (s[j] & WON_BIT);
+        const u64 m = __ballot(won);
+        before[j] = (u32)__popcll(m & lt_mask);
+        if (lane == 0) wave_cnt[j][w] = (u32)__popcll(m);
+    }
+    __syncthreads();
+    u32 run = 0;
+#pragma unroll
+    for (u32 j = 0; j < ASSIGN_KEYS / BLOCK; ++j) {
+        u32 my_base = run;
+        for (u32 x = 0; x < BLOCK / 64; ++x) {
+            if (x < w) my_base += wave_cnt[j][x];
+            run += wave_cnt[j][x];
+        }
+        const bool won = s[j] != SLOT_NONE && (s[j] & WON_BIT);
+        if (!won) continue;
+        const u64 i = (u64)b * ASSIGN_KEYS + j * BLOCK + tid;
+        const u32 slot = s[j] & ~WON_BIT;
+        slot_idx[i] = slot;
+        const u32 rid = first_row + my_base + before[j];
+        if (rid >= t.max_rows) continue;  // does not fit: the caller rolls the batch back
+        reinterpret_cast<u32*>(&t.slots[slot])[2] = rid;
+        t.row_keys[rid] = keys[i];
+        if (init_rows) {
+            float4* r4 = reinterpret_cast<float4*>(t.rows + (u64)rid * t.stride_f);
+            for (u32 c = 0; c < t.stride_f / 4; ++c) {
+                const u32 f = c * 4;
+                r4[c] = make_float4(init_float(t, f), init_float(t, f + 1), init_float(t, f + 2),
+                                    init_float(t, f + 3));
+            }
+        }
+    }
+}
 
 __global__ __launch_bounds__(BLOCK) void rollback_kernel(TableDev t, const u32* __restrict__ slot_idx,
                                                           u32 n, u32 first_new_row) {
@@ -686,11 +749,6 @@ hipError_t launch_fill_u32(u32* p, size_t n, u32 v, hipStream_t s) {
     return hipGetLastError();
 }
 
-hipError_t launch_snapshot_entry(const TableDev& t, hipStream_t s) {
-    snapshot_entry_kernel<<<1, 1, 0, s>>>(t);
-    return hipGetLastError();
-}
-
 hipError_t launch_pull(const TableDev& t, const u64* keys, size_t n, float* out, uint8_t* hit,
                        hipStream_t s) {
     if (n == 0) return hipSuccess;
@@ -723,15 +781,27 @@ hipError_t launch_gather_slots(const TableDev& t, const u32* slot_idx, size_t n,
 }
 
 hipError_t launch_locate(const TableDev& t, const u64* keys, size_t n, u32* slot_out, u32* idx_out,
-                         bool insert, bool init_rows, bool count_dups, hipStream_t s) {
+                         u32* won_count, bool count_dups, hipStream_t s) {
     if (n == 0) return hipSuccess;
     const u32 grid = grid_for(n, KEYS_PER_ROUND * (BLOCK / 64), 16384);
-    if (insert)
-        locate_kernel<true><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, init_rows,
+    if (won_count)
+        locate_kernel<true><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, won_count,
                                                    count_dups);
     else
-        locate_kernel<false><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, 0,
+        locate_kernel<false><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, nullptr,
                                                     count_dups);
+    return hipGetLastError();
+}
+
+size_t assign_blocks(size_t n) { return (n + ASSIGN_KEYS - 1) / ASSIGN_KEYS; }
+
+hipError_t launch_assign_rows(const TableDev& t, const u64* keys, size_t n, u32* slot_idx,
+                              const u32* won_count, u32* won_next, size_t won_words, bool init_rows,
+                              hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const u32 n_blocks = (u32)assign_blocks(n);
+    assign_rows_kernel<<<n_blocks, BLOCK, 0, s>>>(t, keys, (u32)n, slot_idx, won_count, won_next,
+                                                  (u32)won_words, n_blocks, init_rows);
     return hipGetLastError();
 }
 

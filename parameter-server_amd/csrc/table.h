@@ -25,7 +25,7 @@ enum {
     CNT_ROWS = 0,      // rows handed out = keys stored
     CNT_OVERFLOW = 1,  // set when an insert found no row or no slot
     CNT_DUP = 2,       // keys that were already present (counted on request)
-    CNT_ENTRY = 3,     // CNT_ROWS as it was when the current pull began
+    CNT_ENTRY = 3,     // CNT_ROWS as it was when the current inserting operation began
     CNT_BADKEY = 4,    // reserved keys met in a batch (skipped)
     CNT_SORT_ERR = 5,  // a sort tile gave up waiting for its predecessor
     CNT_WORDS = 8
@@ -84,18 +84,24 @@ inline SegGeom seg_geometry(uint32_t dim, uint32_t vec, uint64_t n) {
 // All enqueue on `s` and return the hipError_t of the launch.
 
 hipError_t launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t s);
-hipError_t launch_snapshot_entry(const TableDev& t, hipStream_t s);
 
 // Fused probe + gather of pull without insertion. out is n x dim floats; hit may be null.
 hipError_t launch_pull(const TableDev& t, const uint64_t* keys, size_t n, float* out, uint8_t* hit,
                        hipStream_t s);
 
 // slot_out[i] = slot holding keys[i] or SLOT_NONE; idx_out[i] = i when idx_out is not null.
-// insert: claim a slot and a row for each missing key (row initialised when init_rows).
+// won_count != null: claim a slot for each missing key (insert). The claiming occurrence has the
+// top bit set in slot_out and is counted in won_count[i / 1024]; the launch also records the row
+// count at entry (CNT_ENTRY). launch_assign_rows must follow: it gives the claimed slots dense row
+// ids, fills row_keys, initialises the rows if asked, clears the top bits, publishes the new row
+// count, and zeroes won_next (assign_blocks(n) words), the array the next operation counts into.
 // count_dups: count keys that were found present or claimed by another lane into CNT_DUP.
 hipError_t launch_locate(const TableDev& t, const uint64_t* keys, size_t n, uint32_t* slot_out,
-                         uint32_t* idx_out, bool insert, bool init_rows, bool count_dups,
-                         hipStream_t s);
+                         uint32_t* idx_out, uint32_t* won_count, bool count_dups, hipStream_t s);
+size_t assign_blocks(size_t n);
+hipError_t launch_assign_rows(const TableDev& t, const uint64_t* keys, size_t n, uint32_t* slot_idx,
+                              const uint32_t* won_count, uint32_t* won_next, size_t won_words,
+                              bool init_rows, hipStream_t s);
 
 // Gather through located slots (pull with insertion); hit = row existed when the pull began.
 hipError_t launch_gather_slots(const TableDev& t, const uint32_t* slot_idx, size_t n, float* out,
