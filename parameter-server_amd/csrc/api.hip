@@ -36,6 +36,7 @@ struct pshbm_table {
     int device = 0;
     uint64_t nbuckets = 0;
     uint32_t slot_bits = 0;
+    uint32_t row_bits = 0;  // row ids and ROW_NONE differ in their low row_bits bits
     size_t slots_bytes = 0, rows_bytes = 0, keys_bytes = 0;
 
     uint32_t* h_counters = nullptr;  // pinned, CNT_WORDS
@@ -45,7 +46,7 @@ struct pshbm_table {
     // per-batch workspace of the mutating paths
     size_t ws_cap = 0;
     unsigned sort_parity = 0;  // which half of the sort head the next sort uses
-    DevBuf ws_slot, ws_idx, ws_sslot, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wslot, ws_wval, ws_won;
+    DevBuf ws_slot, ws_row, ws_idx, ws_sslot, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wslot, ws_wval, ws_won;
     unsigned won_parity = 0;  // which half of ws_won the next inserting operation counts into
 
     // staging of the host-pointer entry points
@@ -162,6 +163,7 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     size_t cap = std::max<size_t>(n, 1024);
     ST_TRY(ensure(t, t->ws_slot, cap * 4));
     ST_TRY(ensure(t, t->ws_idx, cap * 4));
+    ST_TRY(ensure(t, t->ws_row, cap * 4));
     ST_TRY(ensure(t, t->ws_sslot, cap * 4));
     ST_TRY(ensure(t, t->ws_sidx, cap * 4));
     ST_TRY(ensure(t, t->ws_sort, sort_pairs_temp_bytes(cap)));
@@ -251,19 +253,19 @@ bool has_reserved_key(const uint64_t* keys, size_t n) {
 // `insert`, followed by the launch that gives the claimed slots their rows. The two arrays of
 // per-block winner counts alternate: each operation counts into one and zeroes the other.
 int32_t locate_and_assign(pshbm_table* t, const uint64_t* d_keys, size_t n, uint32_t* slot, uint32_t* idx,
-                          bool insert, bool init_rows, bool count_dups, hipStream_t s) {
+                          uint32_t* row, bool insert, bool init_rows, bool count_dups, hipStream_t s) {
     if (!insert) {
         HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE,
-                     launch_locate(t->d, d_keys, n, slot, idx, nullptr, count_dups, s));
+                     launch_locate(t->d, d_keys, n, slot, idx, row, nullptr, count_dups, s));
         return PSHBM_OK;
     }
     const size_t half = t->ws_won.bytes / 8;  // words per array
     uint32_t* cur = static_cast<uint32_t*>(t->ws_won.p) + (t->won_parity & 1u) * half;
     uint32_t* next = static_cast<uint32_t*>(t->ws_won.p) + ((t->won_parity & 1u) ^ 1u) * half;
     ++t->won_parity;
-    HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE, launch_locate(t->d, d_keys, n, slot, idx, cur, count_dups, s));
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE, launch_locate(t->d, d_keys, n, slot, idx, row, cur, count_dups, s));
     HIP_TRY_PROF(t, s, PSHBM_PHASE_ASSIGN_ROWS,
-                 launch_assign_rows(t->d, d_keys, n, slot, cur, next, half, init_rows, s));
+                 launch_assign_rows(t->d, d_keys, n, slot, row, cur, next, half, init_rows, s));
     return PSHBM_OK;
 }
 
@@ -279,18 +281,24 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
     if (insert) ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
     uint32_t* idx = static_cast<uint32_t*>(t->ws_idx.p);
-    ST_TRY(locate_and_assign(t, d_keys, n, slot, unique ? nullptr : idx, insert, true, false, s));
+    // Everything after the probe works on row ids: they are dense, so the sort needs fewer bits
+    // than for slot indices, the update needs no second look at the hash array, and sorted
+    // positions walk the row slab in ascending address order.
+    uint32_t* row = static_cast<uint32_t*>(t->ws_row.p);
+    ST_TRY(locate_and_assign(t, d_keys, n, slot, unique ? nullptr : idx, row, insert, true, false, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
     if (unique) {
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_UPDATE_UNIQUE, launch_update_unique(t->d, slot, n, d_grads, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_UPDATE_UNIQUE, launch_update_unique(t->d, row, n, d_grads, s));
     } else {
         uint32_t* sslot = static_cast<uint32_t*>(t->ws_sslot.p);
         uint32_t* sidx = static_cast<uint32_t*>(t->ws_sidx.p);
         SortPlan plan;
+        // a key inserted by this batch more than once: only the claiming occurrence got the row
+        const SortLateKeys late{ROW_PENDING, slot, t->d.slots};
         HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_HIST,
-                     sort_begin(t->ws_sort.p, t->ws_sort.bytes, t->sort_parity++, slot, n,
-                                t->slot_bits + 1, &plan, s));
-        uint32_t *kin = slot, *vin = idx, *kout = sslot, *vout = sidx;
+                     sort_begin(t->ws_sort.p, t->ws_sort.bytes, t->sort_parity++, row, n, t->row_bits,
+                                &plan, s, insert ? &late : nullptr));
+        uint32_t *kin = row, *vin = idx, *kout = sslot, *vout = sidx;
         for (uint32_t p = 0; p < plan.passes; ++p) {
             HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_PASS,
                          sort_pass(plan, p, kin, vin, kout, vout, t->d.counters + CNT_SORT_ERR, s));
@@ -298,7 +306,7 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
             std::swap(vin, vout);
         }
         const bool in_b = (plan.passes & 1u) != 0;
-        const uint32_t* fs = in_b ? sslot : slot;
+        const uint32_t* fs = in_b ? sslot : row;
         const uint32_t* fi = in_b ? sidx : idx;
         uint4* hdr = static_cast<uint4*>(t->ws_hdr.p);
         float* pval = static_cast<float*>(t->ws_pval.p);
@@ -322,7 +330,7 @@ int32_t set_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_values
     uint32_t rows_before = 0;
     ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
-    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, true, false, count_dups, s));
+    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, nullptr, true, false, count_dups, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
     HIP_TRY(t, launch_write_values(t->d, slot, n, d_values, s));
     return PSHBM_OK;
@@ -342,7 +350,7 @@ int32_t ensure_bulk(pshbm_table* t) {
 void destroy_impl(pshbm_table* t) {
     DeviceGuard g(t->device);
     (void)hipDeviceSynchronize();
-    DevBuf* bufs[] = {&t->ws_slot, &t->ws_idx,  &t->ws_sslot, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
+    DevBuf* bufs[] = {&t->ws_slot, &t->ws_row, &t->ws_idx,  &t->ws_sslot, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
                       &t->ws_pval, &t->ws_wslot, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
@@ -430,6 +438,8 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     t->nbuckets = nb;
     t->slot_bits = 0;
     while ((1ull << t->slot_bits) < nb * 4) ++t->slot_bits;
+    t->row_bits = 1;
+    while ((1ull << t->row_bits) <= max_rows) ++t->row_bits;
 
     TableDev& d = t->d;
     d.bucket_mask = (uint32_t)(nb - 1);
@@ -504,7 +514,7 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     uint32_t rows_before = 0;
     ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
-    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, true, true, false, s));
+    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, nullptr, true, true, false, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
     HIP_TRY_PROF(t, s, PSHBM_PHASE_GATHER, launch_gather_slots(t->d, slot, n, d_out_rows, d_hit, s));
     return PSHBM_OK;

@@ -166,6 +166,7 @@ template <bool kInsert>
 __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __restrict__ keys,
                                                         u32 n, u32* __restrict__ slot_out,
                                                         u32* __restrict__ idx_out,
+                                                        u32* __restrict__ row_out,
                                                         u32* __restrict__ won_count,
                                                         int count_dups) {
     const u32 lane = threadIdx.x & 63u;
@@ -181,10 +182,12 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
         bool active = inb && key < KEY_DELETED;
         if (inb && !active && sub == 0) atomicAdd(&t.counters[CNT_BADKEY], 1u);
         u32 slot = SLOT_NONE;
+        u32 row = ROW_NONE;
         bool dup = false;
         if constexpr (!kInsert) {
             Found f = probe_find(t, key, active, grp, sub);
             slot = f.slot;
+            row = f.row;
             dup = f.slot != SLOT_NONE;
         } else {
             bool won = false;
@@ -193,11 +196,17 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
             u32 steps = 0;
             while (__ballot(!done)) {
                 u64 skey = 0;
+                u32 srow = ROW_NONE;
                 // Coherent at the device level: a slot claimed by another compute unit during
-                // this launch must be seen, so the load bypasses the per-CU cache.
-                if (!done)
-                    skey = __hip_atomic_load(reinterpret_cast<u64*>(&t.slots[(u64)b * 4 + sub]),
-                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // this launch must be seen, so the loads bypass the per-CU cache.
+                if (!done) {
+                    uint4* sp = &t.slots[(u64)b * 4 + sub];
+                    skey = __hip_atomic_load(reinterpret_cast<u64*>(sp), __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+                    if (row_out)
+                        srow = __hip_atomic_load(reinterpret_cast<u32*>(sp) + 2, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+                }
                 bool match = !done && skey == key;
                 bool empty = !done && skey == KEY_EMPTY;
                 u32 m4 = (u32)(__ballot(match) >> (grp * 4)) & 0xFu;
@@ -209,18 +218,24 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
                     old = atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[(u64)b * 4 + tgt]),
                                     (unsigned long long)KEY_EMPTY, (unsigned long long)key);
                 u64 oldb = shfl64(old, grp * 4 + tgt);
+                const u32 msub = m4 ? (u32)__ffs((int)m4) - 1u : 0u;
+                const u32 mrow = __shfl(srow, (int)(grp * 4 + msub));
                 if (!done) {
                     if (m4) {
-                        slot = b * 4 + (u32)__ffs((int)m4) - 1u;
+                        slot = b * 4 + msub;
+                        // a key that another group claimed in this launch has no row yet
+                        row = mrow < t.max_rows ? mrow : ROW_PENDING;
                         dup = true;
                         done = true;
                     } else if (e4) {
                         if (oldb == KEY_EMPTY) {
                             slot = b * 4 + tgt;
+                            row = ROW_PENDING;
                             won = true;
                             done = true;
                         } else if (oldb == key) {  // the same key, claimed by another group
                             slot = b * 4 + tgt;
+                            row = ROW_PENDING;
                             dup = true;
                             done = true;
                         }
@@ -246,6 +261,7 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
         if (inb && sub == 0) {
             slot_out[i] = slot;
             if (idx_out) idx_out[i] = (u32)i;
+            if (row_out) row_out[i] = row;
             if (count_dups && dup) atomicAdd(&t.counters[CNT_DUP], 1u);
         }
     }
@@ -260,6 +276,7 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
 // array the next operation counts into. Rows past the capacity raise CNT_OVERFLOW and stay unset.
 __global__ __launch_bounds__(BLOCK) void assign_rows_kernel(TableDev t, const u64* __restrict__ keys,
                                                              u32 n, u32* __restrict__ slot_idx,
+                                                             u32* __restrict__ row_out,
                                                              const u32* __restrict__ won_count,
                                                              u32* __restrict__ won_next, u32 won_words,
                                                              u32 n_blocks, int init_rows) {
@@ -316,7 +333,11 @@ __global__ __launch_bounds__(BLOCK) void assign_rows_kernel(TableDev t, const u6
         const u32 slot = s[j] & ~WON_BIT;
         slot_idx[i] = slot;
         const u32 rid = first_row + my_base + before[j];
-        if (rid >= t.max_rows) continue;  // does not fit: the caller rolls the batch back
+        if (rid >= t.max_rows) {  // does not fit: the caller rolls the batch back
+            if (row_out) row_out[i] = ROW_NONE;
+            continue;
+        }
+        if (row_out) row_out[i] = rid;
         reinterpret_cast<u32*>(&t.slots[slot])[2] = rid;
         t.row_keys[rid] = keys[i];
         if (init_rows) {
@@ -392,11 +413,10 @@ __device__ __forceinline__ void opt_step(const OptParams& o, float g, float& w, 
     }
 }
 
-// Applies the aggregated gradient `g` (columns [col, col+1) in units of T) to the row in `slot`.
+// Applies the aggregated gradient `g` (columns [col, col+1) in units of T) to row `row`.
 template <typename T>
-__device__ __forceinline__ void finalize(const TableDev& t, u32 slot, u32 col, u32 units, T g) {
+__device__ __forceinline__ void finalize(const TableDev& t, u32 row, u32 col, u32 units, T g) {
     constexpr int N = sizeof(T) / 4;
-    u32 row = reinterpret_cast<const u32*>(&t.slots[slot])[2];
     if (row >= t.max_rows) return;
     T* r = reinterpret_cast<T*>(t.rows + (u64)row * t.stride_f);
     const int kind = t.opt.kind;
@@ -416,89 +436,241 @@ __device__ __forceinline__ void finalize(const TableDev& t, u32 slot, u32 col, u
 }
 
 // ---- duplicate aggregation + update over slot-sorted pairs -------------------------------------
-// Each wavefront owns `wch` consecutive sorted positions (a chunk) and walks them in rounds of P
-// positions, `lp` lanes per position. Within a round equal slots are summed by a segmented
-// inclusive scan across lane groups; the running sum of the round's last position is carried into
-// the next round. A run that ends inside the chunk and began inside it is complete: its lanes
-// apply the optimizer step to the row at once. A run that crosses a chunk border leaves a partial
-// sum in part_val (entry 0: the run that entered from the left, entry 1: the run that leaves to
-// the right) for fixup_kernel to join.
+// Each wavefront owns `wch` consecutive sorted positions (a chunk). It copies the chunk's slots
+// and the gradient rows they point to into LDS (16 independent row loads per lane in flight),
+// lists the starts of the runs of equal slots with ballots, and then gives each run to one group
+// of `lp` lanes, which adds the run's rows in sorted order, one LDS read per row. A run longer
+// than 2 P rows is added by all P groups together (strided, then a shuffle tree). A run that
+// begins and ends inside the chunk is complete: its sum is applied to the table row, four runs
+// per lane group at a time so that the row loads of different runs overlap. A run that crosses a
+// chunk border leaves a partial sum in part_val (entry 0: the run that entered from the left,
+// entry 1: the run that leaves to the right) for fixup_kernel to join.
 // part_hdr[w] = {slot of entry 0, flags of entry 0 (1 present, 2 run ends in this chunk),
 //               slot of entry 1, flags of entry 1 (1 present)}.
-template <typename T>
-__global__ __launch_bounds__(BLOCK) void segreduce_kernel(
-    TableDev t, const u32* __restrict__ sslot, const u32* __restrict__ sidx, u32 n,
-    const T* __restrict__ grads, uint4* __restrict__ part_hdr, T* __restrict__ part_val, u32 units,
-    u32 lp_full, u32 P, u32 wch, u32 n_chunks) {
-    const u32 lane = threadIdx.x & 63u;
-    const u32 w = blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
-    if (w >= n_chunks) return;
-    const u32 col0 = blockIdx.y * 64u;
-    const u32 lp = (units - col0) < 64u ? (units - col0) : 64u;
-    const u32 g = lane / lp_full;
-    const u32 c = lane - g * lp_full;
-    const bool lane_on = g < P && c < lp;
-    const u32 cs = w * wch;
-    const u32 ce = (n - cs) < wch ? n : cs + wch;
-    const u32 pe = ce - 1;
-    const u32 first_slot = sslot[cs];
-    const bool open_left = cs > 0 && sslot[cs - 1] == first_slot;
+// LDS per wavefront: wch * lp_full elements of T, then three arrays of wch + 1 words (slots;
+// batch indices, later one action word per run; run starts).
+constexpr int SEG_BLOCK = 128;  // 2 wavefronts
 
-    u32 carry_slot = SLOT_NONE;
-    T carry_v = vzero(T());
-    bool l_present = false, l_ends = false, r_present = false;
-
-    for (u32 r0 = cs; r0 < ce; r0 += P) {
-        const u32 p = r0 + g;
-        const bool valid = lane_on && p < ce;
-        u32 slot = SLOT_NONE, nslot = SLOT_NONE;
-        T v = vzero(T());
-        if (valid) {
-            slot = sslot[p];
-            if (p + 1 < n) nslot = sslot[p + 1];
-            if (slot != SLOT_NONE) {
-                u32 i = sidx[p];
-                v = grads[(u64)i * units + col0 + c];
-            }
-        }
-        if (g == 0 && slot == carry_slot) v = vadd(v, carry_v);
-        // segmented inclusive scan over the P positions of the round (slots are sorted, so equal
-        // end points mean one run)
-        u32 prev = __shfl_up(slot, lp_full);
-        bool cont = valid && g > 0 && prev == slot;
-        if (__any(cont)) {
-            for (u32 off = 1; off < P; off <<= 1) {
-                u32 us = __shfl_up(slot, off * lp_full);
-                T uv = vshfl_up(v, off * lp_full);
-                if (g >= off && us == slot) v = vadd(v, uv);
-            }
-        }
-        const bool real = valid && slot != SLOT_NONE;
-        const bool is_tail = nslot != slot;
-        const bool first_run = open_left && slot == first_slot;
-        const bool do_l = real && first_run && (is_tail || p == pe);
-        const bool do_r = real && !first_run && !is_tail && p == pe;
-        if (real && !first_run && is_tail) finalize<T>(t, slot, col0 + c, units, v);
-        if (do_l) part_val[((u64)w * 2 + 0) * units + col0 + c] = v;
-        if (do_r) part_val[((u64)w * 2 + 1) * units + col0 + c] = v;
-        l_present |= __any(do_l) != 0;
-        l_ends |= __any(do_l && is_tail) != 0;
-        r_present |= __any(do_r) != 0;
-        // the running sum at the round's last position feeds the next round
-        const u32 left = ce - r0;
-        const u32 last_g = (left < P ? left : P) - 1u;
-        carry_slot = __shfl(slot, (int)(last_g * lp_full));
-        carry_v = vshfl(v, last_g * lp_full + c);
-    }
-    if (lane == 0 && blockIdx.y == 0)
-        part_hdr[w] = make_uint4(first_slot, (l_present ? 1u : 0u) | (l_ends ? 2u : 0u), sslot[pe],
-                                 r_present ? 1u : 0u);
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 __device__ __forceinline__ float vshfl_down(float v, u32 d) { return __shfl_down(v, d); }
 __device__ __forceinline__ float4 vshfl_down(float4 v, u32 d) {
     return make_float4(__shfl_down(v.x, d), __shfl_down(v.y, d), __shfl_down(v.z, d),
                        __shfl_down(v.w, d));
+}
+
+// Applies the sums that segreduce_kernel left in LDS (first row of each run whose action word is
+// set) to the table rows, FB runs per lane group at a time. STATES = optimizer state blocks.
+template <typename T, int STATES, u32 FB>
+__device__ __forceinline__ void apply_runs(const TableDev& t, const T* s_val, const u32* s_row,
+                                           const u32* s_act, const u32* s_start, u32 nruns, u32 P,
+                                           u32 g, u32 c, bool lane_on, u32 lp_full, u32 units,
+                                           u32 col) {
+    constexpr int N = sizeof(T) / 4;
+    T* rows = reinterpret_cast<T*>(t.rows);
+    const u32 stride_units = t.stride_f / N;
+    for (u32 j0 = 0; j0 < nruns; j0 += FB * P) {
+        u32 row[FB], st[FB];
+        T wv[FB], av[STATES >= 1 ? FB : 1], bv[STATES >= 2 ? FB : 1];
+#pragma unroll
+        for (u32 k = 0; k < FB; ++k) {
+            const u32 j = j0 + k * P + g;
+            row[k] = ROW_NONE;
+            st[k] = 0;
+            if (lane_on && j < nruns && s_act[j]) {
+                st[k] = s_start[j];
+                const u32 r = s_row[st[k]];
+                if (r < t.max_rows) row[k] = r;
+            }
+        }
+#pragma unroll
+        for (u32 k = 0; k < FB; ++k) {
+            if (row[k] == ROW_NONE) continue;
+            const T* r = rows + (u64)row[k] * stride_units + col;
+            wv[k] = r[0];
+            if constexpr (STATES >= 1) av[k] = r[units];
+            if constexpr (STATES >= 2) bv[k] = r[2 * units];
+        }
+#pragma unroll
+        for (u32 k = 0; k < FB; ++k) {
+            if (row[k] == ROW_NONE) continue;
+            T gs = s_val[st[k] * lp_full + c];
+            T a0 = vzero(T()), b0 = vzero(T());
+            if constexpr (STATES >= 1) a0 = av[k];
+            if constexpr (STATES >= 2) b0 = bv[k];
+            float* gp = reinterpret_cast<float*>(&gs);
+            float* wp = reinterpret_cast<float*>(&wv[k]);
+            float* ap = reinterpret_cast<float*>(&a0);
+            float* bp = reinterpret_cast<float*>(&b0);
+#pragma unroll
+            for (int e = 0; e < N; ++e) opt_step(t.opt, gp[e], wp[e], ap[e], bp[e]);
+            T* r = rows + (u64)row[k] * stride_units + col;
+            r[0] = wv[k];
+            if constexpr (STATES >= 1) r[units] = a0;
+            if constexpr (STATES >= 2) r[2 * units] = b0;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
+    TableDev t, const u32* __restrict__ sslot, const u32* __restrict__ sidx, u32 n,
+    const T* __restrict__ grads, uint4* __restrict__ part_hdr, T* __restrict__ part_val, u32 units,
+    u32 lp_full, u32 P, u32 wch, u32 n_chunks, u32 val_bytes, u32 arr_bytes) {
+    extern __shared__ uint4 seg_lds[];
+    const u32 lane = threadIdx.x & 63u;
+    const u32 wv = threadIdx.x >> 6;
+    const u32 w = blockIdx.x * (SEG_BLOCK / 64) + wv;
+    if (w >= n_chunks) return;  // no workgroup barriers below
+    char* base = reinterpret_cast<char*>(seg_lds) + (size_t)wv * (val_bytes + 3 * arr_bytes);
+    T* s_val = reinterpret_cast<T*>(base);
+    u32* s_slot = reinterpret_cast<u32*>(base + val_bytes);
+    u32* s_aux = reinterpret_cast<u32*>(base + val_bytes + arr_bytes);
+    u32* s_start = reinterpret_cast<u32*>(base + val_bytes + 2 * arr_bytes);
+
+    const u32 col0 = blockIdx.y * 64u;
+    const u32 lp = (units - col0) < 64u ? (units - col0) : 64u;
+    const u32 g = lane / lp_full;
+    const u32 c = lane - g * lp_full;
+    const bool lane_on = g < P && c < lp;
+    const u32 cs = w * wch;
+    const u32 cnt = (n - cs) < wch ? (n - cs) : wch;
+
+    // slots and batch indices of the chunk
+    for (u32 pl = lane; pl < wch; pl += 64) {
+        u32 sl = SLOT_NONE, ix = 0;
+        if (pl < cnt) {
+            sl = sslot[cs + pl];
+            ix = sidx[cs + pl];
+        }
+        s_slot[pl] = sl;
+        s_aux[pl] = ix;
+    }
+    const u32 first_slot = sslot[cs];
+    const u32 last_slot = sslot[cs + cnt - 1];
+    const bool open_left = cs > 0 && sslot[cs - 1] == first_slot;
+    const u32 after = cs + cnt < n ? sslot[cs + cnt] : SLOT_NONE;
+    wave_sync();
+
+    // gradient rows into LDS: position r * P + g in round r
+    {
+        T v[SEG_ROUNDS];
+#pragma unroll
+        for (u32 r = 0; r < SEG_ROUNDS; ++r) {
+            const u32 pl = r * P + g;
+            v[r] = vzero(T());
+            if (lane_on && pl < cnt && s_slot[pl] != SLOT_NONE)
+                v[r] = grads[(u64)s_aux[pl] * units + col0 + c];
+        }
+#pragma unroll
+        for (u32 r = 0; r < SEG_ROUNDS; ++r) {
+            const u32 pl = r * P + g;
+            if (lane_on) s_val[pl * lp_full + c] = v[r];
+        }
+    }
+    wave_sync();
+
+    // run starts; unfound keys (SLOT_NONE) sort last and form no run
+    u32 nruns = 0, nreal = 0;
+    for (u32 k0 = 0; k0 < wch; k0 += 64) {
+        const u32 pl = k0 + lane;
+        u32 sl = SLOT_NONE, pv = SLOT_NONE;
+        if (pl < wch) {
+            sl = s_slot[pl];
+            if (pl > 0) pv = s_slot[pl - 1];
+        }
+        const bool real = sl != SLOT_NONE;
+        const bool head = real && (pl == 0 || pv != sl);
+        const u64 hm = __ballot(head);
+        if (head) s_start[nruns + (u32)__popcll(hm & ((1ull << lane) - 1ull))] = pl;
+        nruns += (u32)__popcll(hm);
+        nreal += (u32)__popcll(__ballot(real));
+    }
+    if (lane == 0) s_start[nruns] = nreal;
+    wave_sync();
+
+    // sums of the runs. A sum that can be applied goes back to LDS in the run's first row and the
+    // run's action word becomes 1; a sum that crosses a border goes to part_val.
+    bool my_l = false, my_le = false, my_r = false;
+    auto classify = [&](u32 j, u32 st, u32 en, T acc) {
+        const u32 sl = s_slot[st];
+        const bool first_run = open_left && j == 0;
+        const bool last_open = en == cnt && after == sl;
+        u32 act = 0;
+        if (first_run) {
+            part_val[((u64)w * 2 + 0) * units + col0 + c] = acc;
+            my_l = true;
+            my_le = !last_open;
+        } else if (last_open) {
+            part_val[((u64)w * 2 + 1) * units + col0 + c] = acc;
+            my_r = true;
+        } else {
+            s_val[st * lp_full + c] = acc;
+            act = 1;
+        }
+        if (c == 0) s_aux[j] = act;
+    };
+    u32 top = 1;
+    while (top < P) top <<= 1;
+    const u32 long_run = 2 * P;
+    for (u32 j0 = 0; j0 < nruns; j0 += P) {
+        const u32 j = j0 + g;
+        const bool have = lane_on && j < nruns;
+        u32 st = 0, en = 0;
+        if (have) {
+            st = s_start[j];
+            en = s_start[j + 1];
+        }
+        const bool is_long = P > 1 && en - st > long_run;
+        if (have && !is_long) {
+            T acc = vzero(T());
+            for (u32 q = st; q < en; ++q) acc = vadd(acc, s_val[q * lp_full + c]);
+            classify(j, st, en, acc);
+        }
+        u64 lm = __ballot(have && is_long && c == 0);
+        while (lm) {
+            const u32 src = (u32)__ffsll((unsigned long long)lm) - 1u;
+            lm &= lm - 1;
+            const u32 jj = __shfl(j, (int)src), s2 = __shfl(st, (int)src), e2 = __shfl(en, (int)src);
+            T a = vzero(T());
+            if (lane_on)
+                for (u32 q = s2 + g; q < e2; q += P) a = vadd(a, s_val[q * lp_full + c]);
+            for (u32 off = top >> 1; off >= 1; off >>= 1) {
+                T o = vshfl_down(a, off * lp_full);
+                if (g + off < P) a = vadd(a, o);
+            }
+            if (lane_on && g == 0) classify(jj, s2, e2, a);
+        }
+    }
+    wave_sync();
+
+    // optimizer step on the rows of the complete runs; a lane group holds as many runs at once
+    // as registers allow, so that their row loads overlap
+    const u32 col = col0 + c;
+    switch (t.opt.kind) {
+        case 0:
+        case 1:
+            apply_runs<T, 0, SEG_ROUNDS>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+                                         lp_full, units, col);
+            break;
+        case 2:
+            apply_runs<T, 1, SEG_ROUNDS / 2>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+                                             lp_full, units, col);
+            break;
+        default:
+            apply_runs<T, 2, SEG_ROUNDS / 4>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+                                             lp_full, units, col);
+            break;
+    }
+
+    const bool l_present = __any(my_l) != 0, l_ends = __any(my_le) != 0, r_present = __any(my_r) != 0;
+    if (lane == 0 && blockIdx.y == 0)
+        part_hdr[w] = make_uint4(first_slot, (l_present ? 1u : 0u) | (l_ends ? 2u : 0u), last_slot,
+                                 r_present ? 1u : 0u);
 }
 
 // A key repeated hundreds of thousands of times in a batch spans thousands of chunks. So that the
@@ -781,26 +953,26 @@ hipError_t launch_gather_slots(const TableDev& t, const u32* slot_idx, size_t n,
 }
 
 hipError_t launch_locate(const TableDev& t, const u64* keys, size_t n, u32* slot_out, u32* idx_out,
-                         u32* won_count, bool count_dups, hipStream_t s) {
+                         u32* row_out, u32* won_count, bool count_dups, hipStream_t s) {
     if (n == 0) return hipSuccess;
     const u32 grid = grid_for(n, KEYS_PER_ROUND * (BLOCK / 64), 16384);
     if (won_count)
-        locate_kernel<true><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, won_count,
-                                                   count_dups);
+        locate_kernel<true><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, row_out,
+                                                   won_count, count_dups);
     else
-        locate_kernel<false><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, nullptr,
-                                                    count_dups);
+        locate_kernel<false><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, slot_out, idx_out, row_out,
+                                                    nullptr, count_dups);
     return hipGetLastError();
 }
 
 size_t assign_blocks(size_t n) { return (n + ASSIGN_KEYS - 1) / ASSIGN_KEYS; }
 
 hipError_t launch_assign_rows(const TableDev& t, const u64* keys, size_t n, u32* slot_idx,
-                              const u32* won_count, u32* won_next, size_t won_words, bool init_rows,
-                              hipStream_t s) {
+                              u32* row_out, const u32* won_count, u32* won_next, size_t won_words,
+                              bool init_rows, hipStream_t s) {
     if (n == 0) return hipSuccess;
     const u32 n_blocks = (u32)assign_blocks(n);
-    assign_rows_kernel<<<n_blocks, BLOCK, 0, s>>>(t, keys, (u32)n, slot_idx, won_count, won_next,
+    assign_rows_kernel<<<n_blocks, BLOCK, 0, s>>>(t, keys, (u32)n, slot_idx, row_out, won_count, won_next,
                                                   (u32)won_words, n_blocks, init_rows);
     return hipGetLastError();
 }
@@ -817,15 +989,19 @@ hipError_t launch_segreduce(const TableDev& t, const u32* sorted_slot, const u32
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads, part_val);
     const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
-    dim3 grid((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);
+    const u32 val_bytes = g.wch * g.lp * (v4 ? 16u : 4u);  // a multiple of 64
+    const u32 arr_bytes = ((g.wch + 1) * 4u + 15u) & ~15u;
+    const size_t lds = (size_t)(SEG_BLOCK / 64) * (val_bytes + 3 * arr_bytes);  // at most 57 KiB
+    dim3 grid((g.n_chunks + SEG_BLOCK / 64 - 1) / (SEG_BLOCK / 64), g.col_blocks);
     if (v4)
-        segreduce_kernel<float4><<<grid, BLOCK, 0, s>>>(
+        segreduce_kernel<float4><<<grid, SEG_BLOCK, lds, s>>>(
             t, sorted_slot, sorted_idx, (u32)n, reinterpret_cast<const float4*>(grads), part_hdr,
-            reinterpret_cast<float4*>(part_val), g.units, g.lp, g.p, g.wch, g.n_chunks);
+            reinterpret_cast<float4*>(part_val), g.units, g.lp, g.p, g.wch, g.n_chunks, val_bytes,
+            arr_bytes);
     else
-        segreduce_kernel<float><<<grid, BLOCK, 0, s>>>(t, sorted_slot, sorted_idx, (u32)n, grads,
-                                                       part_hdr, part_val, g.units, g.lp, g.p,
-                                                       g.wch, g.n_chunks);
+        segreduce_kernel<float><<<grid, SEG_BLOCK, lds, s>>>(t, sorted_slot, sorted_idx, (u32)n, grads,
+                                                             part_hdr, part_val, g.units, g.lp, g.p,
+                                                             g.wch, g.n_chunks, val_bytes, arr_bytes);
     return hipGetLastError();
 }
 

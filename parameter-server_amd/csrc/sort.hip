@@ -44,8 +44,9 @@ constexpr size_t HEAD_COUNTERS = MAX_PASSES * RADIX;
 constexpr size_t HEAD_WORDS = HEAD_COUNTERS + 16;
 constexpr size_t OFF_STATUS = 2 * HEAD_WORDS;
 
-__global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(const u32* __restrict__ keys, u32 n,
-                                                                u32 n_tiles, u32 passes,
+__global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(u32* __restrict__ keys, u32 n,
+                                                                SortLateKeys late, u32 n_tiles,
+                                                                u32 passes,
                                                                 u32* __restrict__ totals,
                                                                 u32* __restrict__ status,
                                                                 u32* __restrict__ next_head) {
@@ -60,6 +61,16 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(const u32* __rest
     for (u32 j = 0; j < SORT_ITEMS; ++j) {  // all loads in flight before the first LDS atomic
         const u64 i = base + (u64)j * SORT_BLOCK + tid;
         k[j] = i < n ? keys[i] : 0u;
+    }
+    if (late.table) {  // keys that became known only after the caller's previous launch
+#pragma unroll
+        for (u32 j = 0; j < SORT_ITEMS; ++j) {
+            const u64 i = base + (u64)j * SORT_BLOCK + tid;
+            if (i < n && k[j] == late.marker) {
+                k[j] = late.table[late.index[i] & 0x7FFFFFFFu].z;
+                keys[i] = k[j];
+            }
+        }
     }
     __syncthreads();
 #pragma unroll
@@ -251,8 +262,8 @@ size_t sort_pairs_temp_bytes(size_t n) {
 
 size_t sort_pairs_head_bytes() { return OFF_STATUS * 4; }
 
-hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, const uint32_t* keys, size_t n,
-                      unsigned end_bit, SortPlan* plan, hipStream_t s) {
+hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys, size_t n,
+                      unsigned end_bit, SortPlan* plan, hipStream_t s, const SortLateKeys* late) {
     plan->n = 0;
     plan->passes = 0;
     if (n == 0) return hipSuccess;
@@ -269,7 +280,9 @@ hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, const uint
     plan->totals = head + HEAD_TOTALS;
     plan->status = words + OFF_STATUS;
     plan->rows = n_tiles + (n_tiles + GROUP - 1) / GROUP;  // per pass: tile words, group words
-    sort_hist_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys, (u32)n, n_tiles, passes, plan->totals,
+    SortLateKeys lk{0u, nullptr, nullptr};
+    if (late) lk = *late;
+    sort_hist_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys, (u32)n, lk, n_tiles, passes, plan->totals,
                                                     plan->status, next_head);
     return hipGetLastError();
 }

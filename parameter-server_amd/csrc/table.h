@@ -19,6 +19,8 @@ constexpr uint64_t KEY_EMPTY = 0xFFFFFFFFFFFFFFFFull;
 constexpr uint64_t KEY_DELETED = 0xFFFFFFFFFFFFFFFEull;
 constexpr uint32_t ROW_NONE = 0xFFFFFFFFu;
 constexpr uint32_t SLOT_NONE = 0xFFFFFFFFu;
+// row of a key whose slot was claimed in the running operation, before rows are handed out
+constexpr uint32_t ROW_PENDING = 0xFFFFFFFEu;
 
 // indices into TableDev::counters
 enum {
@@ -67,7 +69,7 @@ struct SegGeom {
     uint32_t wch;         // positions per wave chunk
     uint32_t n_chunks;    // for a batch of n positions
 };
-constexpr uint32_t SEG_ROUNDS = 16;
+constexpr uint32_t SEG_ROUNDS = 8;
 
 inline SegGeom seg_geometry(uint32_t dim, uint32_t vec, uint64_t n) {
     SegGeom g;
@@ -96,12 +98,17 @@ hipError_t launch_pull(const TableDev& t, const uint64_t* keys, size_t n, float*
 // ids, fills row_keys, initialises the rows if asked, clears the top bits, publishes the new row
 // count, and zeroes won_next (assign_blocks(n) words), the array the next operation counts into.
 // count_dups: count keys that were found present or claimed by another lane into CNT_DUP.
+// row_out (may be null): row_out[i] = row of keys[i], ROW_NONE if the key is not stored, or
+// ROW_PENDING if its slot was claimed in this launch; launch_assign_rows fills in the rows of the
+// claiming occurrences, and a later occurrence of such a key stays ROW_PENDING: its row is
+// slots[slot_out[i]].z once launch_assign_rows has run (SortLateKeys does that lookup).
 hipError_t launch_locate(const TableDev& t, const uint64_t* keys, size_t n, uint32_t* slot_out,
-                         uint32_t* idx_out, uint32_t* won_count, bool count_dups, hipStream_t s);
+                         uint32_t* idx_out, uint32_t* row_out, uint32_t* won_count, bool count_dups,
+                         hipStream_t s);
 size_t assign_blocks(size_t n);
 hipError_t launch_assign_rows(const TableDev& t, const uint64_t* keys, size_t n, uint32_t* slot_idx,
-                              const uint32_t* won_count, uint32_t* won_next, size_t won_words,
-                              bool init_rows, hipStream_t s);
+                              uint32_t* row_out, const uint32_t* won_count, uint32_t* won_next,
+                              size_t won_words, bool init_rows, hipStream_t s);
 
 // Gather through located slots (pull with insertion); hit = row existed when the pull began.
 hipError_t launch_gather_slots(const TableDev& t, const uint32_t* slot_idx, size_t n, float* out,
@@ -112,11 +119,12 @@ hipError_t launch_gather_slots(const TableDev& t, const uint32_t* slot_idx, size
 hipError_t launch_rollback(const TableDev& t, const uint32_t* slot_idx, size_t n,
                            uint32_t first_new_row, hipStream_t s);
 
-// Duplicate aggregation + update over pairs sorted by slot, in two launches: launch_segreduce
-// sums runs of equal slots inside each wavefront's chunk and applies the complete ones;
+// Duplicate aggregation + update over (row, batch index) pairs sorted by row (ROW_NONE = key not
+// stored, sorted last and skipped), in three launches: launch_segreduce
+// sums runs of equal rows inside each wavefront's chunk and applies the complete ones;
 // launch_fixup joins the runs that cross chunk borders. part_hdr: n_chunks uint4;
 // part_val: n_chunks * 2 * dim floats.
-hipError_t launch_segreduce(const TableDev& t, const uint32_t* sorted_slot, const uint32_t* sorted_idx,
+hipError_t launch_segreduce(const TableDev& t, const uint32_t* sorted_row, const uint32_t* sorted_idx,
                             size_t n, const float* grads, uint4* part_hdr, float* part_val,
                             hipStream_t s);
 // launch_fixup_windows first adds up every window of 64 chunks that lies wholly inside one run
@@ -129,8 +137,8 @@ hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const u
                         const float* part_val, const uint32_t* win_slot, const float* win_val,
                         hipStream_t s);
 
-// One optimizer step per located key, no aggregation (keys distinct).
-hipError_t launch_update_unique(const TableDev& t, const uint32_t* slot_idx, size_t n,
+// One optimizer step per located key, no aggregation (keys distinct); rows[i] = row of key i.
+hipError_t launch_update_unique(const TableDev& t, const uint32_t* rows, size_t n,
                                 const float* grads, hipStream_t s);
 
 // rows[slot->row] = values[i] (whole value, vf floats).
@@ -167,8 +175,16 @@ struct SortPlan {
     uint32_t* status;
     size_t rows;
 };
-hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, const uint32_t* keys, size_t n,
-                      unsigned end_bit, SortPlan* plan, hipStream_t s);
+// late (may be null): every keys[i] equal to late->marker is first replaced, in `keys` too, by
+// late->table[late->index[i]].z.
+struct SortLateKeys {
+    uint32_t marker;
+    const uint32_t* index;
+    const uint4* table;
+};
+hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys, size_t n,
+                      unsigned end_bit, SortPlan* plan, hipStream_t s,
+                      const SortLateKeys* late = nullptr);
 hipError_t sort_pass(const SortPlan& plan, unsigned p, const uint32_t* kin, const uint32_t* vin,
                      uint32_t* kout, uint32_t* vout, uint32_t* err_flag, hipStream_t s);
 hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys_a,
