@@ -190,8 +190,18 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
             row = f.row;
             dup = f.slot != SLOT_NONE;
         } else {
+            // Most keys of a batch are stored already: look for them with ordinary cached loads
+            // first. What those loads show may be older than this launch, never wrong: a key that
+            // is seen is stored (slots only go from empty to a key), and a key that is not seen
+            // is looked for again below, with loads that bypass the caches.
+            Found f = probe_find(t, key, active, grp, sub);
+            if (f.slot != SLOT_NONE) {
+                slot = f.slot;
+                row = f.row < t.max_rows ? f.row : ROW_PENDING;
+                dup = true;
+            }
             bool won = false;
-            bool done = !active;
+            bool done = !active || f.slot != SLOT_NONE;
             u32 b = (u32)hash64(key) & t.bucket_mask;
             u32 steps = 0;
             while (__ballot(!done)) {
