@@ -159,7 +159,8 @@ hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long l
                              hipStream_t s);
 
 // ---- sort (sort.hip) -----------------------------------------------------------------------
-// Stable radix sort of (key, value) pairs on the low `end_bit` bits (rounded up to whole bytes).
+// Stable radix sort of (key, value) pairs on the low `end_bit` bits (rounded up to whole digits of
+// 8 to 10 bits: as few digit passes as 10-bit digits allow).
 // Both buffer pairs are scratch: the sorted pairs end in (keys_b, vals_b) when *result_in_b, else
 // in (keys_a, vals_a). *err_flag (device) is raised if a tile's bounded wait for its predecessor
 // ran out, in which case the output is not sorted.
@@ -167,10 +168,10 @@ hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long l
 // and is kept zeroed by the sorts themselves as long as `parity` alternates 0,1,0,1,...
 size_t sort_pairs_temp_bytes(size_t n);
 size_t sort_pairs_head_bytes();
-// The same sort launch by launch (the histogram, then one launch per 8-bit digit p = 0 .. passes-1,
+// The same sort launch by launch (the histogram, then one launch per digit p = 0 .. passes-1,
 // alternating between the two buffer pairs), for callers that time or interleave the launches.
 struct SortPlan {
-    uint32_t n, n_tiles, passes;
+    uint32_t n, n_tiles, passes, bits;
     uint32_t* totals;
     uint32_t* status;
     size_t rows;
