@@ -383,43 +383,63 @@ __global__ __launch_bounds__(BLOCK) void fill_u32_kernel(u32* p, u64 n, u32 v) {
 // ---- optimizer step ------------------------------------------------------------------------
 // One fp32 element; each operation rounds on its own (the file is compiled with
 // -ffp-contract=off and correctly rounded divide / sqrt).
+template <int KIND>
 __device__ __forceinline__ void opt_step(const OptParams& o, float g, float& w, float& s1,
                                          float& s2) {
+    if constexpr (KIND == 0) {  // SUM
+        w = w + g;
+    } else if constexpr (KIND == 1) {  // SGD
+        float step = o.lr * g;
+        w = w - step;
+    } else if constexpr (KIND == 2) {  // ADAGRAD: s1 = accumulator
+        float gg = g * g;
+        float nn = s1 + gg;
+        float num = o.lr * g;
+        float step = num / sqrtf(nn);
+        s1 = nn;
+        w = w - step;
+    } else {  // FTRL: s1 = z, s2 = n
+        float gg = g * g;
+        float n_new = s2 + gg;
+        float sq_new = sqrtf(n_new);
+        float sigma = (sq_new - sqrtf(s2)) / o.alpha;
+        float sw = sigma * w;
+        float z = (s1 + g) - sw;
+        float w_new;
+        if (fabsf(z) <= o.l1) {
+            w_new = 0.0f;
+        } else {
+            float shrunk = z > 0.0f ? z - o.l1 : z + o.l1;
+            float denom = (o.beta + sq_new) / o.alpha + o.l2;
+            w_new = -shrunk / denom;
+        }
+        w = w_new;
+        s1 = z;
+        s2 = n_new;
+    }
+}
+
+// N consecutive elements; the optimizer is chosen once, outside the element loop.
+template <int N>
+__device__ __forceinline__ void opt_step_n(const OptParams& o, const float* g, float* w, float* s1,
+                                           float* s2) {
     switch (o.kind) {
-        case 0:  // SUM
-            w = w + g;
+        case 0:
+#pragma unroll
+            for (int e = 0; e < N; ++e) opt_step<0>(o, g[e], w[e], s1[e], s2[e]);
             break;
-        case 1: {  // SGD
-            float step = o.lr * g;
-            w = w - step;
-        } break;
-        case 2: {  // ADAGRAD
-            float gg = g * g;
-            float nn = s1 + gg;
-            float num = o.lr * g;
-            float step = num / sqrtf(nn);
-            s1 = nn;
-            w = w - step;
-        } break;
-        default: {  // FTRL: s1 = z, s2 = n
-            float gg = g * g;
-            float n_new = s2 + gg;
-            float sq_new = sqrtf(n_new);
-            float sigma = (sq_new - sqrtf(s2)) / o.alpha;
-            float sw = sigma * w;
-            float z = (s1 + g) - sw;
-            float w_new;
-            if (fabsf(z) <= o.l1) {
-                w_new = 0.0f;
-            } else {
-                float shrunk = z > 0.0f ? z - o.l1 : z + o.l1;
-                float denom = (o.beta + sq_new) / o.alpha + o.l2;
-                w_new = -shrunk / denom;
-            }
-            w = w_new;
-            s1 = z;
-            s2 = n_new;
-        } break;
+        case 1:
+#pragma unroll
+            for (int e = 0; e < N; ++e) opt_step<1>(o, g[e], w[e], s1[e], s2[e]);
+            break;
+        case 2:
+#pragma unroll
+            for (int e = 0; e < N; ++e) opt_step<2>(o, g[e], w[e], s1[e], s2[e]);
+            break;
+        default:
+#pragma unroll
+            for (int e = 0; e < N; ++e) opt_step<3>(o, g[e], w[e], s1[e], s2[e]);
+            break;
     }
 }
 
@@ -438,8 +458,7 @@ __device__ __forceinline__ void finalize(const TableDev& t, u32 row, u32 col, u3
     float* wp = reinterpret_cast<float*>(&wv);
     float* ap = reinterpret_cast<float*>(&av);
     float* bp = reinterpret_cast<float*>(&bv);
-#pragma unroll
-    for (int e = 0; e < N; ++e) opt_step(t.opt, gp[e], wp[e], ap[e], bp[e]);
+    opt_step_n<N>(t.opt, gp, wp, ap, bp);
     r[col] = wv;
     if (kind >= 2) r[units + col] = av;
     if (kind == 3) r[2 * units + col] = bv;
@@ -475,12 +494,13 @@ __device__ __forceinline__ float4 vshfl_down(float4 v, u32 d) {
 
 // Applies the sums that segreduce_kernel left in LDS (first row of each run whose action word is
 // set) to the table rows, FB runs per lane group at a time. STATES = optimizer state blocks.
-template <typename T, int STATES, u32 FB>
+template <typename T, int KIND, u32 FB>
 __device__ __forceinline__ void apply_runs(const TableDev& t, const T* s_val, const u32* s_row,
                                            const u32* s_act, const u32* s_start, u32 nruns, u32 P,
                                            u32 g, u32 c, bool lane_on, u32 lp_full, u32 units,
                                            u32 col) {
     constexpr int N = sizeof(T) / 4;
+    constexpr int STATES = KIND <= 1 ? 0 : KIND - 1;
     T* rows = reinterpret_cast<T*>(t.rows);
     const u32 stride_units = t.stride_f / N;
     for (u32 j0 = 0; j0 < nruns; j0 += FB * P) {
@@ -517,7 +537,7 @@ __device__ __forceinline__ void apply_runs(const TableDev& t, const T* s_val, co
             float* ap = reinterpret_cast<float*>(&a0);
             float* bp = reinterpret_cast<float*>(&b0);
 #pragma unroll
-            for (int e = 0; e < N; ++e) opt_step(t.opt, gp[e], wp[e], ap[e], bp[e]);
+            for (int e = 0; e < N; ++e) opt_step<KIND>(t.opt, gp[e], wp[e], ap[e], bp[e]);
             T* r = rows + (u64)row[k] * stride_units + col;
             r[0] = wv[k];
             if constexpr (STATES >= 1) r[units] = a0;
@@ -663,16 +683,19 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
     const u32 col = col0 + c;
     switch (t.opt.kind) {
         case 0:
-        case 1:
             apply_runs<T, 0, SEG_ROUNDS>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
                                          lp_full, units, col);
             break;
+        case 1:
+            apply_runs<T, 1, SEG_ROUNDS>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+                                         lp_full, units, col);
+            break;
         case 2:
-            apply_runs<T, 1, SEG_ROUNDS / 2>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+            apply_runs<T, 2, SEG_ROUNDS / 2>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
                                              lp_full, units, col);
             break;
         default:
-            apply_runs<T, 2, SEG_ROUNDS / 4>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+            apply_runs<T, 3, SEG_ROUNDS / 4>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
                                              lp_full, units, col);
             break;
     }
