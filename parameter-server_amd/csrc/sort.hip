@@ -1,21 +1,28 @@
 // Stable LSD radix sort of (row, batch index) pairs by row: the grouping step of duplicate-key
-// aggregation. Written for batches of 10^5..10^7 pairs, where launch count and latency matter more
-// than bandwidth: one histogram launch, then ONE launch per digit. The digit width is chosen per
-// sort, 8 to 10 bits, so that keys of up to 30 bits take three digit passes.
-//
-// A digit pass cuts the input into tiles of 4096 pairs, one per 1024-thread workgroup:
+// aggregation. The digit width is chosen per sort, 8 to 10 bits, so that keys of up to 30 bits
+// take three digit passes. Every pass cuts the input into tiles of 4096 pairs, one per
+// 1024-thread workgroup, and places a tile's pairs in three steps:
 //   1. each of the 16 wavefronts ranks its 256 pairs, 64 at a time: one ballot per digit bit gives
 //      every lane the set of lanes holding the same digit; its rank is the wave's running count for
 //      that digit plus the number of lower lanes in that set (equal digits keep their input order);
-//   2. thread b owns digit b: it chains the 16 wave counts into the tile count and publishes
-//      it; the last tile of every group of 16 tiles also publishes the group's count. The number
-//      of pairs with digit b in earlier tiles is then the sum of at most 15 tile words and of the
-//      group words before -- two or three batches of loads that wait only for published counts,
-//      never for another tile's finished prefix, so no chain forms across the tiles;
+//   2. thread b owns digit b: it chains the 16 wave counts into the tile's count and learns how
+//      many pairs with digit b lie in earlier tiles (below);
 //   3. the pairs are first put in digit order in LDS, then written out by consecutive lanes, so
 //      that each run of equal digits is a contiguous, coalesced store.
-// The wait is bounded: if a word is not published within SPIN_LIMIT polls the tile raises
-// *err_flag and goes on with what it has, so the grid always drains.
+// How a tile learns what lies before it depends on the size of the input.
+//   * Up to 256 tiles (2^20 pairs; one tile per compute unit, all resident at once) a pass is ONE
+//     launch: every tile publishes its counts, the last tile of every group of 16 tiles also
+//     publishes the group's count, and a tile adds up at most 15 tile words and 15 group words --
+//     two batches of loads that wait only for published counts, never for another tile's finished
+//     prefix, so no chain forms across the tiles. Latency matters most at this size, and one launch
+//     per digit is the shortest path. The wait is bounded: if a word is not published within
+//     SPIN_LIMIT polls the tile raises *err_flag and goes on with what it has, so the grid always
+//     drains. The published words are read with loads that bypass the L2 (tiles run on different
+//     XCDs): about 30 rows of counts per tile, more data than the tile's own pairs -- which is why
+//     this scheme stops paying once tiles queue up.
+//   * Above that a pass is three launches without any waiting: per-tile digit counts, a scan of
+//     the counts over the tiles (which leaves in each tile's row the global position of its first
+//     pair of every digit), and the placement.
 #include "table.h"
 
 namespace pshbm {
@@ -36,35 +43,27 @@ constexpr u32 RADIX_MAX = 1u << MAX_BITS;  // = SORT_BLOCK: a thread per digit
 constexpr u32 MAX_PASSES = 4;
 constexpr u32 FLAG_READY = 1u << 30, COUNT_MASK = (1u << 30) - 1u;
 constexpr u32 SPIN_LIMIT = 1u << 24;
-constexpr u32 GROUP = 16;  // tiles per group of the two-level tile prefix
+constexpr u32 GROUP = 16;                      // tiles per group of the two-level tile prefix
+constexpr u32 LOOKBACK_TILES = GROUP * GROUP;  // largest input of the one-launch passes, in tiles
 
 // temp layout in 32-bit words: two heads {digit totals [MAX_PASSES][RADIX_MAX], pad} used by
 // alternate sorts -- each sort zeroes the other one for its successor, which saves a fill launch --
-// then, per pass, [n_tiles][RADIX_MAX] tile words and [n_groups][RADIX_MAX] group words.
+// then rows of RADIX_MAX words: one-launch passes use, per pass, [n_tiles] tile rows and
+// [n_groups] group rows; three-launch passes use [n_tiles] rows of counts, reused by every pass.
 constexpr size_t HEAD_TOTALS = 0;
 constexpr size_t HEAD_WORDS = MAX_PASSES * RADIX_MAX + 16;
-constexpr size_t OFF_STATUS = 2 * HEAD_WORDS;
+constexpr size_t OFF_ROWS = 2 * HEAD_WORDS;
 
-__global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(u32* __restrict__ keys, u32 n,
-                                                                SortLateKeys late, u32 n_tiles,
-                                                                u32 passes, u32 bits,
-                                                                u32* __restrict__ totals,
-                                                                u32* __restrict__ status,
-                                                                u32* __restrict__ next_head) {
-    // Counts the lowest digit only; every digit pass counts the next digit of the pairs it holds.
-    __shared__ u32 h[RADIX_MAX];
-    const u32 tid = threadIdx.x;
-    const u32 radix = 1u << bits;
-    h[tid] = 0;
-    const u32 tile = blockIdx.x;
-    const u64 base = (u64)tile * SORT_TILE;
-    u32 k[SORT_ITEMS];
+// The tile's four keys per thread, with the keys that became known only after the caller's
+// previous launch filled in (and written back).
+__device__ __forceinline__ void load_keys_late(u32* __restrict__ keys, u32 n, const SortLateKeys& late,
+                                               u64 base, u32 tid, u32 (&k)[SORT_ITEMS]) {
 #pragma unroll
-    for (u32 j = 0; j < SORT_ITEMS; ++j) {  // all loads in flight before the first LDS atomic
+    for (u32 j = 0; j < SORT_ITEMS; ++j) {  // all loads in flight before the first use
         const u64 i = base + (u64)j * SORT_BLOCK + tid;
         k[j] = i < n ? keys[i] : 0u;
     }
-    if (late.table) {  // keys that became known only after the caller's previous launch
+    if (late.table) {
 #pragma unroll
         for (u32 j = 0; j < SORT_ITEMS; ++j) {
             const u64 i = base + (u64)j * SORT_BLOCK + tid;
@@ -74,6 +73,24 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(u32* __restrict__
             }
         }
     }
+}
+
+// One-launch passes: counts of the lowest digit over the whole input (every digit pass counts the
+// next digit of the pairs it holds), and the words the passes publish start at zero.
+__global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(u32* __restrict__ keys, u32 n,
+                                                                SortLateKeys late, u32 n_tiles,
+                                                                u32 passes, u32 bits,
+                                                                u32* __restrict__ totals,
+                                                                u32* __restrict__ status,
+                                                                u32* __restrict__ next_head) {
+    __shared__ u32 h[RADIX_MAX];
+    const u32 tid = threadIdx.x;
+    const u32 radix = 1u << bits;
+    h[tid] = 0;
+    const u32 tile = blockIdx.x;
+    const u64 base = (u64)tile * SORT_TILE;
+    u32 k[SORT_ITEMS];
+    load_keys_late(keys, n, late, base, tid, k);
     __syncthreads();
 #pragma unroll
     for (u32 j = 0; j < SORT_ITEMS; ++j)
@@ -93,6 +110,36 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(u32* __restrict__
         for (u32 x = tid; x < HEAD_WORDS; x += SORT_BLOCK) next_head[x] = 0;
 }
 
+// Three-launch passes, first launch: counts[tile][d] = pairs of the tile whose digit is d, and the
+// digit totals over the whole input.
+__global__ __launch_bounds__(SORT_BLOCK) void sort_tile_count_kernel(u32* __restrict__ keys, u32 n,
+                                                                      SortLateKeys late, u32 shift,
+                                                                      u32 bits,
+                                                                      u32* __restrict__ totals,
+                                                                      u32* __restrict__ counts,
+                                                                      u32* __restrict__ next_head) {
+    __shared__ u32 h[RADIX_MAX];
+    const u32 tid = threadIdx.x;
+    const u32 radix = 1u << bits;
+    h[tid] = 0;
+    const u32 tile = blockIdx.x;
+    const u64 base = (u64)tile * SORT_TILE;
+    u32 k[SORT_ITEMS];
+    load_keys_late(keys, n, late, base, tid, k);
+    __syncthreads();
+#pragma unroll
+    for (u32 j = 0; j < SORT_ITEMS; ++j)
+        if (base + (u64)j * SORT_BLOCK + tid < n) atomicAdd(&h[(k[j] >> shift) & (radix - 1u)], 1u);
+    __syncthreads();
+    if (tid < radix) {
+        const u32 c = h[tid];
+        counts[(size_t)tile * RADIX_MAX + tid] = c;
+        if (c) atomicAdd(&totals[tid], c);
+    }
+    if (next_head && tile == 0)
+        for (u32 x = tid; x < HEAD_WORDS; x += SORT_BLOCK) next_head[x] = 0;
+}
+
 // exclusive scan over the values held by the 1024 threads of the block; all threads must call it
 // (it contains a barrier). `sums` is LDS scratch of SORT_WAVES words.
 __device__ __forceinline__ u32 scan_block_exclusive(u32 v, u32 tid, u32* sums) {
@@ -109,9 +156,52 @@ __device__ __forceinline__ u32 scan_block_exclusive(u32 v, u32 tid, u32* sums) {
     return r;
 }
 
+// Three-launch passes, second launch: counts[tile][d] becomes the position of the tile's first
+// pair with digit d in the sorted output = (pairs with a smaller digit) + (pairs with digit d in
+// earlier tiles). A workgroup owns 64 digits (lane = digit, so rows are read 256 bytes at a time);
+// its 16 wavefronts split the tiles into 16 consecutive ranges.
+__global__ __launch_bounds__(SORT_BLOCK) void sort_scan_kernel(u32* __restrict__ counts,
+                                                                const u32* __restrict__ totals,
+                                                                u32 n_tiles, u32 radix) {
+    __shared__ u32 sums[SORT_WAVES];
+    __shared__ u32 dbase[64];
+    __shared__ u32 part[SORT_WAVES][64];
+    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const u32 d0 = blockIdx.x * 64u;
+    // pairs with a smaller digit: exclusive scan of the totals (every workgroup repeats it)
+    const u32 base = scan_block_exclusive(tid < radix ? totals[tid] : 0u, tid, sums);
+    if (tid >= d0 && tid < d0 + 64u) dbase[tid - d0] = base;
+    const u32 per = (n_tiles + SORT_WAVES - 1) / SORT_WAVES;
+    const u32 t0 = w * per < n_tiles ? w * per : n_tiles;
+    const u32 t1 = t0 + per < n_tiles ? t0 + per : n_tiles;
+    u32* col = counts + d0 + lane;
+    u32 s = 0;
+    for (u32 t = t0; t < t1; t += 8) {
+        u32 v[8];
+#pragma unroll
+        for (u32 x = 0; x < 8; ++x) v[x] = t + x < t1 ? col[(size_t)(t + x) * RADIX_MAX] : 0u;
+#pragma unroll
+        for (u32 x = 0; x < 8; ++x) s += v[x];
+    }
+    part[w][lane] = s;
+    __syncthreads();
+    u32 run = dbase[lane];
+    for (u32 x = 0; x < w; ++x) run += part[x][lane];
+    for (u32 t = t0; t < t1; t += 8) {
+        u32 v[8];
+#pragma unroll
+        for (u32 x = 0; x < 8; ++x) v[x] = t + x < t1 ? col[(size_t)(t + x) * RADIX_MAX] : 0u;
+#pragma unroll
+        for (u32 x = 0; x < 8; ++x) {
+            if (t + x < t1) col[(size_t)(t + x) * RADIX_MAX] = run;
+            run += v[x];
+        }
+    }
+}
+
 // Sum of `count` (<= GROUP) published words spaced RADIX_MAX apart, starting at `words`. The loads
-// of a batch are issued together; the batch is fetched again until every word carries FLAG_READY.
-// The wait is bounded: past SPIN_LIMIT polls the caller gets what is there and *err_flag is raised.
+// are issued together; the batch is fetched again until every word carries FLAG_READY. The wait is
+// bounded: past SPIN_LIMIT polls the caller gets what is there and *err_flag is raised.
 __device__ __forceinline__ u32 wait_sum(const u32* words, u32 count, u32* err_flag) {
     if (count == 0) return 0;
     u32 spins = 0;
@@ -133,20 +223,24 @@ __device__ __forceinline__ u32 wait_sum(const u32* words, u32 count, u32* err_fl
             *err_flag = 1u;
             return sum;
         }
-        __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_s_sleep(2);
     }
 }
 
-template <u32 BITS>
+// One digit pass. LOOKBACK: the one-launch scheme (totals, status, group_status, err_flag are
+// used, and the counts of the next digit go to totals_next); otherwise `first_pos` is the tile's
+// row of positions left by sort_scan_kernel.
+template <u32 BITS, bool LOOKBACK>
 __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
     const u32* __restrict__ kin, const u32* __restrict__ vin, u32* __restrict__ kout,
     u32* __restrict__ vout, u32 n, u32 shift, const u32* __restrict__ totals,
-    u32* __restrict__ totals_next, u32* status, u32* group_status, u32 n_tiles, u32* err_flag) {
+    u32* __restrict__ totals_next, u32* status, u32* group_status, const u32* __restrict__ first_pos,
+    u32 n_tiles, u32* err_flag) {
     constexpr u32 RADIX = 1u << BITS;
     // 32 KiB used twice: the per-wave digit counts (16 bits each: a wave holds 256 pairs, a tile
     // 4096) while ranking, then the tile's pairs in digit order
     __shared__ u32 pool[2 * SORT_TILE];
-    __shared__ u32 hnext[RADIX];       // this tile's counts of the next digit
+    __shared__ u32 hnext[LOOKBACK ? RADIX : 1];  // this tile's counts of the next digit
     __shared__ u32 binpos[RADIX];      // global position of a digit's run - its place in the tile
     __shared__ u32 tile_start[RADIX];  // place of a digit's run in the tile
     __shared__ u32 sums_a[SORT_WAVES], sums_b[SORT_WAVES];
@@ -155,18 +249,26 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
     u32* skey = pool;
     u32* sval = pool + SORT_TILE;
     const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
-    // Tiles are taken in workgroup order. The hardware starts workgroups in that order, so a
-    // tile's predecessors are running (or done) when it looks back; should that ever not hold,
-    // the bounded spin below turns a would-be hang into an error flag.
+    // Tiles are taken in workgroup order. With the one-launch scheme every tile is resident at
+    // once (at most one per compute unit), so the tiles a tile waits for are running or done;
+    // should that ever not hold, the bounded spin turns a would-be hang into an error flag.
     const u32 tile = blockIdx.x;
-    const u32 tot = tid < RADIX ? totals[tid] : 0u;  // needed late; fetched with the pairs
+    u32 tot = 0, gpos = 0;  // needed late; fetched with the pairs
+    if (tid < RADIX) {
+        if constexpr (LOOKBACK)
+            tot = totals[tid];
+        else
+            gpos = first_pos[(size_t)tile * RADIX_MAX + tid];
+    }
 #pragma unroll
     for (u32 x = 0; x < SORT_WAVES * RADIX / 2 / SORT_BLOCK; ++x) pool[x * SORT_BLOCK + tid] = 0;
-    if (tid < RADIX) hnext[tid] = 0;
+    if constexpr (LOOKBACK)
+        if (tid < RADIX) hnext[tid] = 0;
     __syncthreads();
     const u64 tile_base = (u64)tile * SORT_TILE;
     const u64 base = tile_base + (u64)w * SORT_WAVE_SPAN;
     const u64 lt_mask = (1ull << lane) - 1ull;
+    const u32 lt_lo = (u32)lt_mask, lt_hi = (u32)(lt_mask >> 32);
 
     u32 key[SORT_ITEMS], val[SORT_ITEMS], rnk[SORT_ITEMS];
 #pragma unroll
@@ -181,24 +283,31 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
     for (u32 j = 0; j < SORT_ITEMS; ++j) {
         const bool valid = base + (u64)j * 64 + lane < n;
         const u32 d = (key[j] >> shift) & (RADIX - 1u);
-        u64 peers = __ballot(valid);
+        // peers = the valid lanes that hold the same digit. Lanes past the end of the input never
+        // enter the set, so the per-bit ballots need not exclude them.
+        const u64 vm = __builtin_amdgcn_ballot_w64(valid);
+        u32 plo = (u32)vm, phi = (u32)(vm >> 32);
 #pragma unroll
         for (u32 b = 0; b < BITS; ++b) {
-            const bool bit = (d >> b) & 1u;
-            const u64 m = __ballot(valid && bit);
-            peers &= bit ? m : ~m;
+            const u32 bit = (d >> b) & 1u;
+            const u64 m = __builtin_amdgcn_ballot_w64(bit != 0u);
+            const u32 flip = bit - 1u;  // 0 where the bit is set, all ones where it is clear
+            plo &= (u32)m ^ flip;
+            phi &= (u32)(m >> 32) ^ flip;
         }
-        const u32 before = (u32)__popcll(peers & lt_mask);
+        const u32 before = (u32)__popc(plo & lt_lo) + (u32)__popc(phi & lt_hi);
+        const u32 npeers = (u32)__popc(plo) + (u32)__popc(phi);
         u32 running = 0;
         if (valid) {
             running = wcnt[w * RADIX + d];
-            if (before == 0) wcnt[w * RADIX + d] = (u16)(running + (u32)__popcll(peers));
+            if (before == 0) wcnt[w * RADIX + d] = (u16)(running + npeers);
         }
         rnk[j] = running + before;
-        if (valid && totals_next) atomicAdd(&hnext[(key[j] >> (shift + BITS)) & (RADIX - 1u)], 1u);
+        if constexpr (LOOKBACK)
+            if (valid && totals_next) atomicAdd(&hnext[(key[j] >> (shift + BITS)) & (RADIX - 1u)], 1u);
     }
     __syncthreads();
-    // 2. thread b < RADIX owns digit b: wave offsets, tile count, digit base, look-back
+    // 2. thread b < RADIX owns digit b: wave offsets, tile count, what lies before the tile
     u32 tile_count = 0;
     if (tid < RADIX) {
         u32 run = 0;
@@ -209,30 +318,33 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
             run += c;
         }
         tile_count = run;
-        if (totals_next && hnext[tid]) atomicAdd(&totals_next[tid], hnext[tid]);
-        // publish early: successors only ever wait for these per-tile counts
-        __hip_atomic_store(status + (size_t)tile * RADIX_MAX + tid, FLAG_READY | tile_count,
-                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if constexpr (LOOKBACK) {
+            if (totals_next && hnext[tid]) atomicAdd(&totals_next[tid], hnext[tid]);
+            // publish early: successors only ever wait for these per-tile counts
+            __hip_atomic_store(status + (size_t)tile * RADIX_MAX + tid, FLAG_READY | tile_count,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
-    const u32 digit_base = scan_block_exclusive(tot, tid, sums_a);          // over the whole input
     const u32 local_start = scan_block_exclusive(tile_count, tid, sums_b);  // inside this tile
+    if constexpr (LOOKBACK) {
+        const u32 digit_base = scan_block_exclusive(tot, tid, sums_a);  // over the whole input
+        if (tid < RADIX) {
+            const u32 b = tid;
+            const u32 grp = tile / GROUP, first = grp * GROUP;
+            // (a) the tiles before this one in its group of GROUP: one batch of loads
+            const u32 in_group = wait_sum(status + (size_t)first * RADIX_MAX + b, tile - first, err_flag);
+            // the last tile of a group (or of the input) publishes the group's total
+            if (tile + 1 == first + GROUP || tile + 1 == n_tiles)
+                __hip_atomic_store(group_status + (size_t)grp * RADIX_MAX + b,
+                                   FLAG_READY | ((in_group + tile_count) & COUNT_MASK), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            // (b) the groups before this one (at most GROUP - 1): one more batch
+            gpos = digit_base + in_group + wait_sum(group_status + b, grp, err_flag);
+        }
+    }
     if (tid < RADIX) {
-        const u32 b = tid;
-        const u32 grp = tile / GROUP, first = grp * GROUP;
-        // (a) the tiles before this one in its group of GROUP: one batch of loads
-        const u32 in_group = wait_sum(status + (size_t)first * RADIX_MAX + b, tile - first, err_flag);
-        // the last tile of a group (or of the input) publishes the group's total
-        if (tile + 1 == first + GROUP || tile + 1 == n_tiles)
-            __hip_atomic_store(group_status + (size_t)grp * RADIX_MAX + b,
-                               FLAG_READY | ((in_group + tile_count) & COUNT_MASK), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-        // (b) the groups before this one, GROUP words per round trip
-        u32 excl = in_group;
-        for (u32 g0 = 0; g0 < grp; g0 += GROUP)
-            excl += wait_sum(group_status + (size_t)g0 * RADIX_MAX + b,
-                             (grp - g0) < GROUP ? grp - g0 : GROUP, err_flag);
-        tile_start[b] = local_start;
-        binpos[b] = digit_base + excl - local_start;  // wraps; undone by adding the place in the tile
+        tile_start[tid] = local_start;
+        binpos[tid] = gpos - local_start;  // wraps; undone by adding the place in the tile
     }
     __syncthreads();
     // 3. digit order in LDS (over the wave counts, once every place is known), then coalesced stores
@@ -265,15 +377,46 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
     }
 }
 
+size_t tiles_of(size_t n) { return (n + SORT_TILE - 1) / SORT_TILE; }
+
+template <bool LOOKBACK>
+hipError_t launch_pass(u32 bits, u32 n_tiles, hipStream_t s, const u32* kin, const u32* vin, u32* kout,
+                       u32* vout, u32 n, u32 shift, const u32* totals, u32* totals_next, u32* status,
+                       u32* group_status, const u32* first_pos, u32* err_flag) {
+    switch (bits) {
+        case 8:
+            sort_pass_kernel<8, LOOKBACK><<<n_tiles, SORT_BLOCK, 0, s>>>(
+                kin, vin, kout, vout, n, shift, totals, totals_next, status, group_status, first_pos,
+                n_tiles, err_flag);
+            break;
+        case 9:
+            sort_pass_kernel<9, LOOKBACK><<<n_tiles, SORT_BLOCK, 0, s>>>(
+                kin, vin, kout, vout, n, shift, totals, totals_next, status, group_status, first_pos,
+                n_tiles, err_flag);
+            break;
+        case 10:
+            sort_pass_kernel<10, LOOKBACK><<<n_tiles, SORT_BLOCK, 0, s>>>(
+                kin, vin, kout, vout, n, shift, totals, totals_next, status, group_status, first_pos,
+                n_tiles, err_flag);
+            break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 }  // namespace
 
 size_t sort_pairs_temp_bytes(size_t n) {
-    const size_t n_tiles = (n + SORT_TILE - 1) / SORT_TILE;
-    const size_t rows = (n_tiles ? n_tiles : 1) + (n_tiles + GROUP - 1) / GROUP + 1;
-    return (OFF_STATUS + (size_t)MAX_PASSES * rows * RADIX_MAX) * 4;
+    const size_t n_tiles = tiles_of(n);
+    size_t rows;
+    if (n_tiles <= LOOKBACK_TILES)
+        rows = MAX_PASSES * ((n_tiles ? n_tiles : 1) + (n_tiles + GROUP - 1) / GROUP + 1);
+    else
+        rows = n_tiles;
+    return (OFF_ROWS + rows * RADIX_MAX) * 4;
 }
 
-size_t sort_pairs_head_bytes() { return OFF_STATUS * 4; }
+size_t sort_pairs_head_bytes() { return OFF_ROWS * 4; }
 
 hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys, size_t n,
                       unsigned end_bit, SortPlan* plan, hipStream_t s, const SortLateKeys* late) {
@@ -287,7 +430,7 @@ hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, uint32_t* 
     u32 bits = (end_bit + passes - 1) / passes;
     if (bits < MIN_BITS) bits = MIN_BITS;
     if (passes > MAX_PASSES) return hipErrorInvalidValue;
-    const u32 n_tiles = (u32)((n + SORT_TILE - 1) / SORT_TILE);
+    const u32 n_tiles = (u32)tiles_of(n);
     u32* words = static_cast<u32*>(temp);
     u32* head = words + (parity & 1u) * HEAD_WORDS;
     u32* next_head = words + ((parity & 1u) ^ 1u) * HEAD_WORDS;
@@ -295,13 +438,18 @@ hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, uint32_t* 
     plan->n_tiles = n_tiles;
     plan->passes = passes;
     plan->bits = bits;
+    plan->lookback = n_tiles <= LOOKBACK_TILES;
     plan->totals = head + HEAD_TOTALS;
-    plan->status = words + OFF_STATUS;
-    plan->rows = n_tiles + (n_tiles + GROUP - 1) / GROUP;  // per pass: tile words, group words
+    plan->status = words + OFF_ROWS;
+    plan->rows = n_tiles + (n_tiles + GROUP - 1) / GROUP;  // one-launch passes: tile and group rows
     SortLateKeys lk{0u, nullptr, nullptr};
     if (late) lk = *late;
-    sort_hist_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys, (u32)n, lk, n_tiles, passes, bits,
-                                                    plan->totals, plan->status, next_head);
+    if (plan->lookback)
+        sort_hist_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys, (u32)n, lk, n_tiles, passes, bits,
+                                                        plan->totals, plan->status, next_head);
+    else
+        sort_tile_count_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys, (u32)n, lk, 0u, bits, plan->totals,
+                                                              plan->status, next_head);
     return hipGetLastError();
 }
 
@@ -310,29 +458,27 @@ hipError_t sort_pass(const SortPlan& plan, unsigned p, const uint32_t* kin, cons
     if (plan.n == 0) return hipSuccess;
     if (p >= plan.passes) return hipErrorInvalidValue;
     const u32 shift = plan.bits * p;
-    const u32* totals = plan.totals + p * RADIX_MAX;
-    u32* totals_next = p + 1 < plan.passes ? plan.totals + (p + 1) * RADIX_MAX : nullptr;
-    u32* status = plan.status + (size_t)p * plan.rows * RADIX_MAX;
-    u32* group_status = plan.status + ((size_t)p * plan.rows + plan.n_tiles) * RADIX_MAX;
-    switch (plan.bits) {
-        case 8:
-            sort_pass_kernel<8><<<plan.n_tiles, SORT_BLOCK, 0, s>>>(kin, vin, kout, vout, plan.n, shift,
-                                                                    totals, totals_next, status,
-                                                                    group_status, plan.n_tiles, err_flag);
-            break;
-        case 9:
-            sort_pass_kernel<9><<<plan.n_tiles, SORT_BLOCK, 0, s>>>(kin, vin, kout, vout, plan.n, shift,
-                                                                    totals, totals_next, status,
-                                                                    group_status, plan.n_tiles, err_flag);
-            break;
-        case 10:
-            sort_pass_kernel<10><<<plan.n_tiles, SORT_BLOCK, 0, s>>>(kin, vin, kout, vout, plan.n, shift,
-                                                                     totals, totals_next, status,
-                                                                     group_status, plan.n_tiles, err_flag);
-            break;
-        default: return hipErrorInvalidValue;
+    u32* totals = plan.totals + p * RADIX_MAX;
+    if (plan.lookback) {
+        u32* totals_next = p + 1 < plan.passes ? plan.totals + (p + 1) * RADIX_MAX : nullptr;
+        u32* status = plan.status + (size_t)p * plan.rows * RADIX_MAX;
+        u32* group_status = plan.status + ((size_t)p * plan.rows + plan.n_tiles) * RADIX_MAX;
+        return launch_pass<true>(plan.bits, plan.n_tiles, s, kin, vin, kout, vout, plan.n, shift, totals,
+                                 totals_next, status, group_status, nullptr, err_flag);
     }
-    return hipGetLastError();
+    const SortLateKeys none{0u, nullptr, nullptr};
+    if (p > 0) {  // pass 0 was counted by sort_begin
+        sort_tile_count_kernel<<<plan.n_tiles, SORT_BLOCK, 0, s>>>(
+            const_cast<u32*>(kin), plan.n, none, shift, plan.bits, totals, plan.status, nullptr);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    const u32 radix = 1u << plan.bits;
+    sort_scan_kernel<<<radix / 64, SORT_BLOCK, 0, s>>>(plan.status, totals, plan.n_tiles, radix);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return launch_pass<false>(plan.bits, plan.n_tiles, s, kin, vin, kout, vout, plan.n, shift, nullptr,
+                              nullptr, nullptr, nullptr, plan.status, err_flag);
 }
 
 hipError_t sort_pairs(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys_a,

@@ -168,10 +168,11 @@ hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long l
 // and is kept zeroed by the sorts themselves as long as `parity` alternates 0,1,0,1,...
 size_t sort_pairs_temp_bytes(size_t n);
 size_t sort_pairs_head_bytes();
-// The same sort launch by launch (the histogram, then one launch per digit p = 0 .. passes-1,
+// The same sort step by step (sort_begin counts, then sort_pass places digit p = 0 .. passes-1,
 // alternating between the two buffer pairs), for callers that time or interleave the launches.
 struct SortPlan {
     uint32_t n, n_tiles, passes, bits;
+    bool lookback;  // one launch per pass (inputs of up to 2^20 pairs) or three
     uint32_t* totals;
     uint32_t* status;
     size_t rows;
