@@ -148,6 +148,31 @@ def test_aggregation_exact_with_integer_gradients(ps, orc, dim):
     t.close()
 
 
+@pytest.mark.parametrize("n", [(1 << 20) + 1, 1_300_000, 2_500_000])
+def test_aggregation_exact_large_batch(ps, orc, n):
+    """Batches beyond 2^20 pairs take the sort's three-launch passes; the batch mixes one key that
+    fills a tenth of it, skewed repeats, keys pushed for the first time more than once, and keys
+    that are not stored and must be dropped (second push, no insertion)."""
+    rng = np.random.default_rng(n)
+    dim = 4
+    t = ps.Table(dim, capacity=700_000, max_batch=n, **OPTS["sum"])
+    r = orc.Oracle(dim, capacity=700_000, **OPTS["sum"])
+    keys = (rng.zipf(1.1, n).astype(np.uint64) * np.uint64(2654435761)) % np.uint64(400_000)
+    keys[rng.integers(0, n, n // 10)] = 123456789
+    fresh = rng.integers(1 << 40, 1 << 41, 50_000).astype(np.uint64)
+    keys[rng.integers(0, n, 120_000)] = fresh[rng.integers(0, fresh.size, 120_000)]
+    g = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+    assert t.push(keys, g) == 0 and r.push(keys, g) == 0
+    assert_same_table(t, r, exact=True)
+    keys2 = keys.copy()
+    keys2[::3] += np.uint64(1 << 50)                   # not stored
+    g2 = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+    assert t.push(keys2, g2, ps.PUSH_NO_INSERT) == 0
+    assert r.push(keys2, g2, orc.PUSH_NO_INSERT) == 0
+    assert_same_table(t, r, exact=True)
+    t.close()
+
+
 LOW_MULTIPLICITY = 32
 
 
