@@ -48,8 +48,9 @@ KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist"
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by the factors a plain
 # copy of known size gave), measured on an MI355X; the summaries are under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", "pull"): 191_700_000, ("c2", "locate"): 71_500_000, ("c2", "sort_hist"): 5_400_000,
-    ("c2", "sort_pass"): 21_200_000, ("c2", "segreduce"): 235_500_000, ("c2", "fixup"): 1_400_000,
+    ("c2", "pull"): 191_800_000, ("c2", "locate"): 75_700_000, ("c2", "assign_rows"): 100_000,
+    ("c2", "sort_hist"): 6_200_000, ("c2", "sort_pass"): 26_100_000, ("c2", "segreduce"): 194_800_000,
+    ("c2", "fixup_windows"): 300_000, ("c2", "fixup"): 1_900_000,
 }
 
 
