@@ -165,7 +165,60 @@ def cpu_baseline(cfg, wl, budget_keys):
         "value": keys_per_step / per_step, "unit": "keys/s", "cores": 1, "kind": "port",
         "sample": f"{n}-key table (of {cfg['n']}), median of {steps - 1} steps of {k}-key batches, "
                   f"oracle/ps_oracle.cpp single thread",
+        "sharded": cpu_baseline_sharded(cfg, wl, n, oracle, np),
     }
+
+
+def cpu_baseline_sharded(cfg, wl, n, oracle, np):
+    """The same sample on S shards, one applying thread per shard (a push takes its shard
+    exclusively, pico-ps/operator/SparsePushOperator.h:220, so a shard never has more): the table
+    and every batch are split by key, as the reference's client does before it sends
+    (SparsePushOperator.h:161-184); the split is not timed, the shards run concurrently."""
+    from concurrent.futures import ThreadPoolExecutor
+    S = max(1, min(16, os.cpu_count() or 1))
+    dim, k = cfg["dim"], cfg["batch"]
+    shards = [oracle.Oracle(dim, capacity=2 * n // S + 8 * k, **cfg["opt"]) for _ in range(S)]
+    vf = shards[0].value_floats
+    rng = np.random.default_rng(1)
+    chunk = 1_000_000
+    for start in range(0, n, chunk):
+        cnt = min(chunk, n - start)
+        keys = wl.table_keys_np(start, cnt, seed=0)
+        vals = (rng.standard_normal((cnt, vf), dtype=np.float32) * np.float32(0.01))
+        if cfg["opt"]["optimizer"] == 2:
+            vals[:, dim:] = cfg["opt"]["init_acc"]
+        if cfg["opt"]["optimizer"] == 3:
+            vals[:, 2 * dim:] = vals[:, dim:2 * dim] ** 2
+        which = keys % np.uint64(S)
+        for s in range(S):
+            m = which == s
+            assert shards[s].set(keys[m], vals[m]) == 0
+
+    def apply(job):
+        o, keys, grads = job
+        o.pull(keys)
+        if not cfg["pull_only"]:
+            assert o.push(keys, grads) == 0
+
+    steps, times = 4, []
+    with ThreadPoolExecutor(S) as pool:
+        for _ in range(steps):
+            if cfg["s"] is None:
+                keys = wl.keys_of_index_np(rng.integers(0, n, k), 0)
+            else:
+                keys = wl.zipf_batch_np(rng, n, cfg["s"], k, seed=0)
+            grads = rng.standard_normal((k, dim), dtype=np.float32) * np.float32(cfg["sigma"])
+            which = keys % np.uint64(S)
+            jobs = [(shards[s], np.ascontiguousarray(keys[which == s]),
+                     np.ascontiguousarray(grads[which == s])) for s in range(S)]
+            t0 = time.perf_counter()
+            list(pool.map(apply, jobs))
+            times.append(time.perf_counter() - t0)
+    for o in shards:
+        o.close()
+    per_step = sorted(times[1:])[len(times[1:]) // 2]
+    return {"value": k * (1 if cfg["pull_only"] else 2) / per_step, "unit": "keys/s", "cores": S,
+            "sample": f"the same table and batches split over {S} shards by key, one thread per shard"}
 
 
 def main():
