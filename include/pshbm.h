@@ -184,6 +184,64 @@ int32_t pshbm_dump(pshbm_table* t, void* records, size_t capacity_records, size_
  * *n_out < batch marks the end. */
 int32_t pshbm_iterate(pshbm_table* t, size_t offset, size_t batch, void* records, size_t* n_out);
 
+/* ---- for-each and erase-if ------------------------------------------------------------------
+ * The reference's hooks for_each(key, value) and erase_if(key, value) are C++ virtuals
+ * (pico-ps/operator/ForEachOperator.h:180-190, pico-ps/operator/EraseIfOperator.h:38-47). A hook
+ * that has to run on the host is served by pshbm_iterate (visit every record) and pshbm_erase
+ * (erase the keys the hook chose). The common hooks -- a comparison on the key or on a few value
+ * columns, counting and summing -- run on the device from a description: up to four terms, all of
+ * which must hold; no term = every record. */
+#define PSHBM_COL_KEY (-1) /* term on the key (operands u, u2) instead of a value column (operand f) */
+enum {
+    PSHBM_CMP_LT = 0,
+    PSHBM_CMP_LE = 1,
+    PSHBM_CMP_GT = 2,
+    PSHBM_CMP_GE = 3,
+    PSHBM_CMP_EQ = 4,
+    PSHBM_CMP_NE = 5,
+    PSHBM_CMP_MOD_EQ = 6 /* key % u == u2 (keys only; u > 0) */
+};
+typedef struct pshbm_term {
+    int32_t column; /* 0 .. value_floats-1, or PSHBM_COL_KEY */
+    int32_t cmp;    /* PSHBM_CMP_* */
+    float f;        /* right-hand side for a value column */
+    uint32_t reserved;
+    uint64_t u;  /* right-hand side for the key (modulus for MOD_EQ) */
+    uint64_t u2; /* remainder for MOD_EQ */
+} pshbm_term;
+#define PSHBM_MAX_TERMS 4
+typedef struct pshbm_predicate {
+    uint32_t struct_size; /* = sizeof(pshbm_predicate) */
+    uint32_t n_terms;     /* 0 .. PSHBM_MAX_TERMS */
+    pshbm_term term[PSHBM_MAX_TERMS];
+} pshbm_predicate;
+
+/* Read-only for-each with the reduction "count the records and add up their values": replaces
+ * SparseTableForEachReadOperator::apply_request (ForEachOperator.h:166-199) for hooks of that
+ * shape, e.g. the reference's TestForEachOperator {num, sum, count} (pico-ps/test/TestOps.h:159-185).
+ * where == NULL visits every record. *count = records that satisfy `where`; column_sums (may be
+ * NULL) receives value_floats doubles, the sums of each value column over those records. The sums
+ * are added in a fixed order: two calls on the same table give the same bits. */
+int32_t pshbm_for_each(pshbm_table* t, const pshbm_predicate* where, uint64_t* count,
+                       double* column_sums);
+
+/* Erases every record that satisfies `where` (NULL = all, like pshbm_clear): replaces
+ * SparseTableEraseIfOperator::apply_request (EraseIfOperator.h:27-55). *erased (may be NULL) =
+ * records removed. The rows that remain are packed to the front of the slab, so dump / iterate
+ * stay a dense walk; their relative order changes, like the reference's after safe_erase
+ * (KVShardStorage.h:827-834). */
+int32_t pshbm_erase_if(pshbm_table* t, const pshbm_predicate* where, uint64_t* erased);
+
+/* Erases the given keys (absent keys and repeats are ignored); *erased (may be NULL) = records
+ * removed. The building block for an erase_if hook evaluated on the host. */
+int32_t pshbm_erase(pshbm_table* t, const uint64_t* keys, size_t n, uint64_t* erased);
+int32_t pshbm_erase_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, uint64_t* erased, void* stream);
+
+/* Rebuilds the hash array from the stored keys, dropping the markers that erased keys leave in
+ * their slots: the counterpart of safe_shrink (KVShardStorage.h:816-825). Erase calls do this by
+ * themselves once the markers fill an eighth of the slots. */
+int32_t pshbm_compact(pshbm_table* t);
+
 /* Empties the table and keeps its memory: KVShardStorage.h:902-908. */
 int32_t pshbm_clear(pshbm_table* t);
 

@@ -35,6 +35,36 @@ class _Config(C.Structure):
     ]
 
 
+COL_KEY = -1
+CMP_LT, CMP_LE, CMP_GT, CMP_GE, CMP_EQ, CMP_NE, CMP_MOD_EQ = range(7)
+
+
+class _Term(C.Structure):
+    _fields_ = [("column", C.c_int32), ("cmp", C.c_int32), ("f", C.c_float), ("reserved", C.c_uint32),
+                ("u", C.c_uint64), ("u2", C.c_uint64)]
+
+
+class Predicate(C.Structure):
+    _fields_ = [("struct_size", C.c_uint32), ("n_terms", C.c_uint32), ("term", _Term * 4)]
+
+
+def predicate(*terms):
+    """The same constructor as the product binding's: (column, cmp, operand) terms."""
+    p = Predicate()
+    p.struct_size = C.sizeof(Predicate)
+    p.n_terms = len(terms)
+    for i, (col, cmp_, operand) in enumerate(terms):
+        p.term[i].column, p.term[i].cmp = col, cmp_
+        if col == COL_KEY:
+            if cmp_ == CMP_MOD_EQ:
+                p.term[i].u, p.term[i].u2 = operand
+            else:
+                p.term[i].u = operand
+        else:
+            p.term[i].f = operand
+    return p
+
+
 def build():
     """Compiles the oracle with g++ (a few seconds)."""
     subprocess.run(["make", "-C", _HERE, "-B", "libps_oracle.so"], check=True, capture_output=True)
@@ -65,6 +95,9 @@ def lib():
         L.pso_load.argtypes = [vp, vp, C.c_size_t, C.c_uint32]
         L.pso_iterate.argtypes = [vp, C.c_size_t, C.c_size_t, vp, C.POINTER(C.c_size_t)]
         L.pso_dump.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_size_t)]
+        L.pso_for_each.argtypes = [vp, vp, C.POINTER(C.c_uint64), vp]
+        L.pso_erase_if.argtypes = [vp, vp, C.POINTER(C.c_uint64)]
+        L.pso_erase.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_uint64)]
         L.pso_clear.argtypes = [vp]
         L.pso_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         _lib = L
@@ -160,6 +193,27 @@ class Oracle:
         got = C.c_size_t()
         st = lib().pso_iterate(self._h, offset, batch, rec.ctypes.data, C.byref(got))
         return st, rec[: got.value]
+
+    def for_each(self, where=None):
+        n = C.c_uint64()
+        sums = np.zeros(self.value_floats, dtype=np.float64)
+        st = lib().pso_for_each(self._h, C.byref(where) if where is not None else None, C.byref(n),
+                                sums.ctypes.data)
+        return st, n.value, sums
+
+    def erase_if(self, where=None):
+        n = C.c_uint64()
+        st = lib().pso_erase_if(self._h, C.byref(where) if where is not None else None, C.byref(n))
+        return st, n.value
+
+    def erase(self, keys):
+        k, kp = _keys(keys)
+        n = C.c_uint64()
+        st = lib().pso_erase(self._h, kp, k.size, C.byref(n))
+        return st, n.value
+
+    def compact(self):
+        return OK
 
     def clear(self):
         return lib().pso_clear(self._h)

@@ -19,6 +19,10 @@
 //       pinned by the reference's integer test operator: pushing arg=key c times gives
 //       sum = key*c, count = c (pico-ps/test/TestOps.h:98-117,171-172;
 //       pico-ps/test/ps_pmem_test.cpp:401-439).
+//   pso_for_each, pso_erase_if, pso_erase
+//       pinned by the reference's test operators (pico-ps/test/TestOps.h:138-185: erase the odd
+//       keys; count and sum every record) and the counts its service test asserts
+//       (pico-ps/test/ps_service_test.cpp:158-166,176-184), and by a brute-force dict model.
 //   SGD / ADAGRAD / FTRL arithmetic (apply_update below)
 //       PARITY UNPINNED BY THE REFERENCE: pico-ps ships no optimizer (the update is the user
 //       hook SparsePushOperator.h:448). The formulas are this repository's definition; they are
@@ -384,6 +388,120 @@ int32_t pso_dump(void* h, void* records, size_t capacity_records, size_t* n_out)
     Oracle& o = *static_cast<Oracle*>(h);
     if (capacity_records < o.row_keys.size()) return ST_ERROR;
     return pso_iterate(h, 0, o.row_keys.size(), records, n_out);
+}
+
+// ---- for-each / erase-if -------------------------------------------------------------------
+// The hooks the reference leaves to the application (for_each, erase_if) in the declarative form
+// the device library evaluates: up to four comparisons on the key or on value columns, all of
+// which must hold. Layout identical to pshbm_term / pshbm_predicate.
+struct pso_term {
+    int32_t column;  // -1 = the key
+    int32_t cmp;     // 0 LT, 1 LE, 2 GT, 3 GE, 4 EQ, 5 NE, 6 MOD_EQ (key % u == u2)
+    float f;
+    uint32_t reserved;
+    uint64_t u, u2;
+};
+struct pso_predicate {
+    uint32_t struct_size;
+    uint32_t n_terms;
+    pso_term term[4];
+};
+
+static bool holds(const pso_predicate* p, uint64_t key, const float* v) {
+    if (!p) return true;
+    for (uint32_t i = 0; i < p->n_terms; ++i) {
+        const pso_term& t = p->term[i];
+        bool r = false;
+        if (t.column < 0) {
+            switch (t.cmp) {
+                case 0: r = key < t.u; break;
+                case 1: r = key <= t.u; break;
+                case 2: r = key > t.u; break;
+                case 3: r = key >= t.u; break;
+                case 4: r = key == t.u; break;
+                case 5: r = key != t.u; break;
+                case 6: r = t.u != 0 && key % t.u == t.u2; break;
+            }
+        } else {
+            const float x = v[t.column];
+            switch (t.cmp) {
+                case 0: r = x < t.f; break;
+                case 1: r = x <= t.f; break;
+                case 2: r = x > t.f; break;
+                case 3: r = x >= t.f; break;
+                case 4: r = x == t.f; break;
+                case 5: r = x != t.f; break;
+            }
+        }
+        if (!r) return false;
+    }
+    return true;
+}
+
+// safe_erase (KVShardStorage.h:827-834) on the slab model: the last row takes the erased row's
+// place, so the slab stays dense; iteration order after an erase is unspecified, as in the reference.
+static void erase_row(Oracle& o, uint32_t r) {
+    const uint32_t last = (uint32_t)o.row_keys.size() - 1;
+    o.map.erase(o.row_keys[r]);
+    if (r != last) {
+        o.row_keys[r] = o.row_keys[last];
+        std::memcpy(&o.rows[(size_t)r * o.vf], &o.rows[(size_t)last * o.vf], (size_t)o.vf * 4);
+        o.map[o.row_keys[r]] = r;
+    }
+    o.row_keys.pop_back();
+    o.rows.resize((size_t)last * o.vf);
+}
+
+// SparseTableForEachReadOperator::apply_request, ForEachOperator.h:180-190, with the hook
+// "result = {1, value}" and merge_result = add (the shape of TestForEachOperator, TestOps.h:159-185):
+// *count = records that satisfy the predicate, sums[c] = sum of value column c over them.
+int32_t pso_for_each(void* h, const pso_predicate* where, uint64_t* count, double* sums) {
+    Oracle& o = *static_cast<Oracle*>(h);
+    uint64_t n = 0;
+    if (sums)
+        for (uint32_t c = 0; c < o.vf; ++c) sums[c] = 0.0;
+    for (size_t r = 0; r < o.row_keys.size(); ++r) {
+        const float* v = &o.rows[r * o.vf];
+        if (!holds(where, o.row_keys[r], v)) continue;
+        ++n;
+        if (sums)
+            for (uint32_t c = 0; c < o.vf; ++c) sums[c] += (double)v[c];
+    }
+    *count = n;
+    return ST_OK;
+}
+
+// SparseTableEraseIfOperator::apply_request, EraseIfOperator.h:38-47.
+int32_t pso_erase_if(void* h, const pso_predicate* where, uint64_t* erased) {
+    Oracle& o = *static_cast<Oracle*>(h);
+    if (o.c.read_only) return ST_ERROR;
+    uint64_t n = 0;
+    for (size_t r = 0; r < o.row_keys.size();) {
+        if (holds(where, o.row_keys[r], &o.rows[r * o.vf])) {
+            erase_row(o, (uint32_t)r);  // the row that moved in is examined next
+            ++n;
+        } else {
+            ++r;
+        }
+    }
+    if (erased) *erased = n;
+    return ST_OK;
+}
+
+// erase of chosen keys: what an erase_if hook evaluated outside the storage comes down to.
+int32_t pso_erase(void* h, const uint64_t* keys, size_t n, uint64_t* erased) {
+    Oracle& o = *static_cast<Oracle*>(h);
+    if (o.c.read_only) return ST_ERROR;
+    uint64_t gone = 0;
+    for (size_t i = 0; i < n; ++i) {
+        if (reserved(keys[i])) return ST_ERROR;
+        auto it = o.map.find(keys[i]);
+        if (it == o.map.end()) continue;
+        erase_row(o, it->second);
+        ++gone;
+    }
+    if (erased) *erased = gone;
+    return ST_OK;
 }
 
 // KVShardStorage::clear, KVShardStorage.h:902-908

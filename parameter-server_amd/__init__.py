@@ -30,6 +30,7 @@ SYMBOLS = [
     "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
     "pshbm_queue", "pshbm_queue_dev", "pshbm_queue_pairs", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
     "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
+    "pshbm_for_each", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
@@ -66,6 +67,39 @@ class Stats(C.Structure):
         ("probe_hist", C.c_uint64 * 16),
         ("max_probe", C.c_uint64),
     ]
+
+
+COL_KEY = -1
+CMP_LT, CMP_LE, CMP_GT, CMP_GE, CMP_EQ, CMP_NE, CMP_MOD_EQ = range(7)
+
+
+class Term(C.Structure):
+    _fields_ = [("column", C.c_int32), ("cmp", C.c_int32), ("f", C.c_float), ("reserved", C.c_uint32),
+                ("u", C.c_uint64), ("u2", C.c_uint64)]
+
+
+class Predicate(C.Structure):
+    """pshbm_predicate: up to four terms that must all hold."""
+    _fields_ = [("struct_size", C.c_uint32), ("n_terms", C.c_uint32), ("term", Term * 4)]
+
+
+def predicate(*terms):
+    """predicate((column, cmp, operand), ...): column COL_KEY compares the key with an integer
+    operand -- (COL_KEY, CMP_MOD_EQ, (modulus, remainder)) for key % modulus == remainder --,
+    any other column compares that value column with a float."""
+    p = Predicate()
+    p.struct_size = C.sizeof(Predicate)
+    p.n_terms = len(terms)
+    for i, (col, cmp_, operand) in enumerate(terms):
+        p.term[i].column, p.term[i].cmp = col, cmp_
+        if col == COL_KEY:
+            if cmp_ == CMP_MOD_EQ:
+                p.term[i].u, p.term[i].u2 = operand
+            else:
+                p.term[i].u = operand
+        else:
+            p.term[i].f = operand
+    return p
 
 
 class Profile(C.Structure):
@@ -130,6 +164,11 @@ def lib():
         L.pshbm_load.argtypes = [vp, vp, sz, u32]
         L.pshbm_dump.argtypes = [vp, vp, sz, C.POINTER(sz)]
         L.pshbm_iterate.argtypes = [vp, sz, sz, vp, C.POINTER(sz)]
+        L.pshbm_for_each.argtypes = [vp, vp, C.POINTER(C.c_uint64), vp]
+        L.pshbm_erase_if.argtypes = [vp, vp, C.POINTER(C.c_uint64)]
+        L.pshbm_erase.argtypes = [vp, vp, sz, C.POINTER(C.c_uint64)]
+        L.pshbm_erase_dev.argtypes = [vp, vp, sz, C.POINTER(C.c_uint64), vp]
+        L.pshbm_compact.argtypes = [vp]
         L.pshbm_clear.argtypes = [vp]
         L.pshbm_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pshbm_memory_usage.argtypes = [vp, C.POINTER(C.c_uint64)]
@@ -251,6 +290,33 @@ class Table:
         got = C.c_size_t()
         st = lib().pshbm_iterate(self._h, offset, batch, rec.ctypes.data, C.byref(got))
         return st, rec[: got.value]
+
+    def for_each(self, where=None):
+        """(status, count, column sums) over the records that satisfy `where` (a Predicate)."""
+        n = C.c_uint64()
+        sums = np.zeros(self.value_floats, dtype=np.float64)
+        st = lib().pshbm_for_each(self._h, C.byref(where) if where is not None else None, C.byref(n),
+                                  sums.ctypes.data)
+        return st, n.value, sums
+
+    def erase_if(self, where=None):
+        n = C.c_uint64()
+        st = lib().pshbm_erase_if(self._h, C.byref(where) if where is not None else None, C.byref(n))
+        return st, n.value
+
+    def erase(self, keys):
+        k = _u64(keys)
+        n = C.c_uint64()
+        st = lib().pshbm_erase(self._h, k.ctypes.data, k.size, C.byref(n))
+        return st, n.value
+
+    def erase_dev(self, d_keys, n, stream=0):
+        got = C.c_uint64()
+        st = lib().pshbm_erase_dev(self._h, d_keys, n, C.byref(got), stream)
+        return st, got.value
+
+    def compact(self):
+        return lib().pshbm_compact(self._h)
 
     def clear(self):
         return lib().pshbm_clear(self._h)

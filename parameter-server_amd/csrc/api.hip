@@ -53,6 +53,14 @@ struct pshbm_table {
     std::mutex st_mu;
     DevBuf st_keys, st_vals, st_out, st_hit, st_raw;
 
+    // for-each / erase scratch: per-row flags, per-tile counts, row lists, reduction partials;
+    // device and pinned copies of {erased, rows left, holes} and of the for-each result
+    DevBuf ms_dead, ms_tiles, ms_lists, ms_fe;
+    uint32_t* d_info = nullptr;
+    uint32_t* h_info = nullptr;
+    double* h_fe = nullptr;
+    uint64_t tombstones = 0;  // slots holding the marker of an erased key
+
     // sync-push queue
     DevBuf q_keys, q_grads;
     size_t q_n = 0;
@@ -352,6 +360,7 @@ void destroy_impl(pshbm_table* t) {
     (void)hipDeviceSynchronize();
     DevBuf* bufs[] = {&t->ws_slot, &t->ws_row, &t->ws_idx,  &t->ws_sslot, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
                       &t->ws_pval, &t->ws_wslot, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
+                      &t->ms_dead, &t->ms_tiles, &t->ms_lists, &t->ms_fe,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
         if (b->p) (void)hipFree(b->p);
@@ -368,6 +377,9 @@ void destroy_impl(pshbm_table* t) {
     if (t->d_hist) (void)hipFree(t->d_hist);
     if (t->h_counters) (void)hipHostFree(t->h_counters);
     if (t->h_hist) (void)hipHostFree(t->h_hist);
+    if (t->d_info) (void)hipFree(t->d_info);
+    if (t->h_info) (void)hipHostFree(t->h_info);
+    if (t->h_fe) (void)hipHostFree(t->h_fe);
     if (t->order_ev) (void)hipEventDestroy(t->order_ev);
     for (hipEvent_t e : t->prof_ev) (void)hipEventDestroy(e);
     if (t->stream) (void)hipStreamDestroy(t->stream);
@@ -376,6 +388,68 @@ void destroy_impl(pshbm_table* t) {
 }
 
 thread_local std::string g_create_error;
+
+// ---- for-each / erase ----------------------------------------------------------------------
+int32_t check_predicate(pshbm_table* t, const pshbm_predicate* w, pshbm_predicate* out) {
+    std::memset(out, 0, sizeof *out);
+    out->struct_size = sizeof *out;
+    if (!w) return PSHBM_OK;
+    if (w->struct_size != sizeof(pshbm_predicate)) return fail(t, PSHBM_INVALID_CONFIG, "predicate: struct_size");
+    if (w->n_terms > PSHBM_MAX_TERMS) return fail(t, PSHBM_INVALID_CONFIG, "predicate: more than %d terms", PSHBM_MAX_TERMS);
+    for (uint32_t i = 0; i < w->n_terms; ++i) {
+        const pshbm_term& m = w->term[i];
+        if (m.column != PSHBM_COL_KEY && (m.column < 0 || (uint32_t)m.column >= t->d.vf))
+            return fail(t, PSHBM_INVALID_CONFIG, "predicate: term %u names column %d of %u", i, m.column, t->d.vf);
+        if (m.cmp < PSHBM_CMP_LT || m.cmp > PSHBM_CMP_MOD_EQ)
+            return fail(t, PSHBM_INVALID_CONFIG, "predicate: term %u has no such comparison", i);
+        if (m.cmp == PSHBM_CMP_MOD_EQ && (m.column != PSHBM_COL_KEY || m.u == 0))
+            return fail(t, PSHBM_INVALID_CONFIG, "predicate: term %u: MOD_EQ needs the key and a modulus", i);
+    }
+    *out = *w;
+    return PSHBM_OK;
+}
+
+int32_t ensure_maint(pshbm_table* t) {
+    if (!t->d_info) HIP_TRY(t, hipMalloc(reinterpret_cast<void**>(&t->d_info), 4 * sizeof(uint32_t)));
+    if (!t->h_info) HIP_TRY(t, hipHostMalloc(reinterpret_cast<void**>(&t->h_info), 4 * sizeof(uint32_t), hipHostMallocDefault));
+    if (!t->h_fe)
+        HIP_TRY(t, hipHostMalloc(reinterpret_cast<void**>(&t->h_fe), ((size_t)t->d.vf + 1) * sizeof(double), hipHostMallocDefault));
+    return PSHBM_OK;
+}
+
+// Hash array rebuilt from the stored keys (the table lock is held).
+int32_t compact_locked(pshbm_table* t, hipStream_t s) {
+    ST_TRY(read_counters(t, s));
+    const uint32_t rows = t->h_counters[CNT_ROWS];
+    HIP_TRY(t, hipMemsetAsync(t->d.slots, 0xFF, t->slots_bytes, s));
+    HIP_TRY(t, launch_reinsert(t->d, rows, s));
+    ST_TRY(read_counters(t, s));
+    if (t->h_counters[CNT_OVERFLOW]) return fail(t, PSHBM_FATAL, "compact: the hash array overflowed");
+    t->tombstones = 0;
+    return PSHBM_OK;
+}
+
+// Removes the rows flagged in ms_dead (one byte per row of the `rows` stored). The lock is held.
+int32_t erase_flagged(pshbm_table* t, uint32_t rows, hipStream_t s, uint64_t* erased) {
+    uint8_t* dead = static_cast<uint8_t*>(t->ms_dead.p);
+    ST_TRY(ensure(t, t->ms_tiles, (erase_tiles(rows) + 1) * 4));
+    uint32_t* tiles = static_cast<uint32_t*>(t->ms_tiles.p);
+    HIP_TRY(t, launch_erase_count(t->d, rows, dead, tiles, t->d_info, s));
+    HIP_TRY(t, hipMemcpyAsync(t->h_info, t->d_info, 4 * sizeof(uint32_t), hipMemcpyDeviceToHost, s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    const uint32_t gone = t->h_info[0];
+    if (erased) *erased = gone;
+    t->size_bound = rows - gone;
+    if (gone == 0) return PSHBM_OK;
+    ST_TRY(ensure(t, t->ms_lists, 3 * (size_t)gone * 4));
+    HIP_TRY(t, launch_erase_apply(t->d, rows, gone, dead, tiles, t->d_info,
+                                  static_cast<uint32_t*>(t->ms_lists.p), s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    t->tombstones += gone;
+    if (t->tombstones > t->nbuckets * 4 / 8) ST_TRY(compact_locked(t, s));
+    return PSHBM_OK;
+}
+
 
 }  // namespace
 
@@ -871,6 +945,101 @@ int32_t pshbm_dump(pshbm_table* t, void* records, size_t capacity_records, size_
 }
 
 // ---- clear / size / stats ----------------------------------------------------------------------
+// ---- for-each / erase ------------------------------------------------------------------------
+int32_t pshbm_for_each(pshbm_table* t, const pshbm_predicate* where, uint64_t* count, double* column_sums) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (!count) return fail(t, PSHBM_ERROR, "for_each: null count");
+    pshbm_predicate pred;
+    ST_TRY(check_predicate(t, where, &pred));
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    hipStream_t s = t->stream;
+    ST_TRY(begin_op(t, s));
+    ST_TRY(ensure_maint(t));
+    ST_TRY(read_counters(t, s));
+    const uint32_t rows = t->h_counters[CNT_ROWS];
+    const uint32_t vf = t->d.vf;
+    *count = 0;
+    if (column_sums) std::fill(column_sums, column_sums + vf, 0.0);
+    if (rows == 0) return PSHBM_OK;
+    ST_TRY(ensure(t, t->ms_fe, for_each_scratch_bytes(t->d)));
+    double* scratch = static_cast<double*>(t->ms_fe.p);
+    HIP_TRY(t, launch_for_each(t->d, rows, pred, scratch, s));
+    HIP_TRY(t, hipMemcpyAsync(t->h_fe, scratch, ((size_t)vf + 1) * sizeof(double), hipMemcpyDeviceToHost, s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    *count = (uint64_t)t->h_fe[vf];
+    if (column_sums) std::copy(t->h_fe, t->h_fe + vf, column_sums);
+    return PSHBM_OK;
+}
+
+int32_t pshbm_erase_if(pshbm_table* t, const pshbm_predicate* where, uint64_t* erased) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (t->cfg.read_only) return fail(t, PSHBM_ERROR, "erase_if: the table is read-only");
+    pshbm_predicate pred;
+    ST_TRY(check_predicate(t, where, &pred));
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    hipStream_t s = t->stream;
+    ST_TRY(begin_op(t, s));
+    ST_TRY(ensure_maint(t));
+    ST_TRY(read_counters(t, s));
+    const uint32_t rows = t->h_counters[CNT_ROWS];
+    if (erased) *erased = 0;
+    if (rows == 0) return PSHBM_OK;
+    ST_TRY(ensure(t, t->ms_dead, round_up(rows, 4)));
+    HIP_TRY(t, launch_mark_pred(t->d, rows, pred, static_cast<uint8_t*>(t->ms_dead.p), s));
+    return erase_flagged(t, rows, s, erased);
+}
+
+int32_t pshbm_erase_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, uint64_t* erased, void* stream) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (erased) *erased = 0;
+    if (n == 0) return PSHBM_OK;
+    if (!d_keys) return fail(t, PSHBM_ERROR, "erase: null buffer");
+    if (n > 0x7FFFFFFFull) return fail(t, PSHBM_ERROR, "erase: batch larger than 2^31-1 keys");
+    if (t->cfg.read_only) return fail(t, PSHBM_ERROR, "erase: the table is read-only");
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    ST_TRY(begin_op(t, s));
+    ST_TRY(ensure_maint(t));
+    ST_TRY(ensure_workspace(t, n));
+    ST_TRY(read_counters(t, s));
+    const uint32_t rows = t->h_counters[CNT_ROWS];
+    if (rows == 0) return PSHBM_OK;
+    ST_TRY(ensure(t, t->ms_dead, round_up(rows, 4)));
+    uint8_t* dead = static_cast<uint8_t*>(t->ms_dead.p);
+    HIP_TRY(t, hipMemsetAsync(dead, 0, round_up(rows, 4), s));
+    uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
+    uint32_t* row = static_cast<uint32_t*>(t->ws_row.p);
+    HIP_TRY(t, launch_locate(t->d, d_keys, n, slot, nullptr, row, nullptr, false, s));
+    HIP_TRY(t, launch_mark_rows(row, n, rows, dead, s));
+    return erase_flagged(t, rows, s, erased);
+}
+
+int32_t pshbm_erase(pshbm_table* t, const uint64_t* keys, size_t n, uint64_t* erased) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (erased) *erased = 0;
+    if (n == 0) return PSHBM_OK;
+    if (!keys) return fail(t, PSHBM_ERROR, "erase: null buffer");
+    if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "erase: reserved key in batch");
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    ST_TRY(ensure(t, t->st_keys, n * 8));
+    hipStream_t s = t->stream;
+    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, n * 8, hipMemcpyHostToDevice, s));
+    return pshbm_erase_dev(t, static_cast<const uint64_t*>(t->st_keys.p), n, erased, s);
+}
+
+int32_t pshbm_compact(pshbm_table* t) {
+    if (!t) return PSHBM_INVALID_ID;
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    hipStream_t s = t->stream;
+    ST_TRY(begin_op(t, s));
+    return compact_locked(t, s);
+}
+
 int32_t pshbm_clear(pshbm_table* t) {
     if (!t) return PSHBM_INVALID_ID;
     DeviceGuard g(t->device);
@@ -881,6 +1050,7 @@ int32_t pshbm_clear(pshbm_table* t) {
     HIP_TRY(t, hipMemsetAsync(t->d.counters, 0, CNT_WORDS * 4, s));
     HIP_TRY(t, hipStreamSynchronize(s));
     t->size_bound = 0;
+    t->tombstones = 0;
     return PSHBM_OK;
 }
 

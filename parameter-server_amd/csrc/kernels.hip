@@ -6,16 +6,12 @@
 // to a key, so that consecutive lanes touch consecutive 16 bytes of a row or of the packed
 // response.
 #include "table.h"
+#include "probe.h"
 
 namespace pshbm {
 
-using u32 = uint32_t;
-using u64 = uint64_t;
-
 namespace {
 
-constexpr int BLOCK = 256;  // 4 wavefronts
-constexpr u32 KEYS_PER_ROUND = 16;
 constexpr u32 WON_BIT = 0x80000000u;  // in a located slot index: this key claimed the slot in this launch
 constexpr u32 ASSIGN_KEYS = 1024;     // keys per workgroup of assign_rows_kernel
 
@@ -35,12 +31,6 @@ __device__ __forceinline__ float vshfl_up(float v, u32 d) { return __shfl_up(v, 
 __device__ __forceinline__ float4 vshfl_up(float4 v, u32 d) {
     return make_float4(__shfl_up(v.x, d), __shfl_up(v.y, d), __shfl_up(v.z, d), __shfl_up(v.w, d));
 }
-__device__ __forceinline__ u64 shfl64(u64 v, u32 src) {
-    u32 lo = __shfl((u32)v, (int)src);
-    u32 hi = __shfl((u32)(v >> 32), (int)src);
-    return ((u64)hi << 32) | lo;
-}
-
 // n / d for n*d < 2^32 by one multiply: m = ceil(2^32 / d) (d == 1 handled by m = 2^32).
 __device__ __forceinline__ u32 div_small(u32 n, u64 m) { return (u32)(((u64)n * m) >> 32); }
 // n / d for any 64-bit n by one multiply-high: m = ceil(2^64 / d), d >= 2.
@@ -48,46 +38,6 @@ __device__ __forceinline__ u64 div_big(u64 n, u64 m, u32 d) { return d == 1 ? n 
 
 inline u64 magic32(u32 d) { return ((1ull << 32) + d - 1) / d; }
 inline u64 magic64(u32 d) { return d <= 1 ? 0 : (~0ull / d) + 1; }
-
-// ---- probing -------------------------------------------------------------------------------
-struct Found {
-    u32 slot;
-    u32 row;
-};
-
-// Four lanes (sub = 0..3 of group grp) look for `key`. Every lane of the wavefront must call
-// this; lanes whose `active` is false only take part in the ballots.
-__device__ __forceinline__ Found probe_find(const TableDev& t, u64 key, bool active, u32 grp,
-                                            u32 sub) {
-    Found f{SLOT_NONE, ROW_NONE};
-    u32 b = (u32)hash64(key) & t.bucket_mask;
-    bool done = !active;
-    u32 steps = 0;
-    while (__ballot(!done)) {
-        uint4 s = make_uint4(0u, 0u, 0u, 0u);
-        if (!done) s = t.slots[(u64)b * 4 + sub];
-        u64 skey = ((u64)s.y << 32) | s.x;
-        bool match = !done && skey == key;
-        bool empty = !done && skey == KEY_EMPTY;
-        u32 m4 = (u32)(__ballot(match) >> (grp * 4)) & 0xFu;
-        u32 e4 = (u32)(__ballot(empty) >> (grp * 4)) & 0xFu;
-        u32 src = grp * 4 + (m4 ? (u32)__ffs((int)m4) - 1u : 0u);
-        u32 row = __shfl(s.z, (int)src);
-        if (!done) {
-            if (m4) {
-                f.slot = b * 4 + (src & 3u);
-                f.row = row;
-                done = true;
-            } else if (e4) {
-                done = true;
-            } else {
-                b = (b + 1) & t.bucket_mask;
-                if (++steps > t.bucket_mask) done = true;
-            }
-        }
-    }
-    return f;
-}
 
 __device__ __forceinline__ float init_float(const TableDev& t, u32 f) {
     return (t.opt.kind == 2 /*ADAGRAD*/ && f >= t.dim) ? t.opt.init_acc : 0.0f;

@@ -13,6 +13,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../../include/pshbm.h"
+
 namespace pshbm {
 
 constexpr uint64_t KEY_EMPTY = 0xFFFFFFFFFFFFFFFFull;
@@ -157,6 +159,30 @@ hipError_t launch_unpack_records(const uint32_t* records, size_t n, uint32_t str
 // probe-distance histogram over the stored keys: hist[0..15], hist[16] = max distance.
 hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long long* hist,
                              hipStream_t s);
+
+// ---- for-each / erase / rebuild (maint.hip) -------------------------------------------------
+// Count and column sums of the rows that satisfy `pred`. scratch: for_each_scratch_bytes();
+// the result is left in its first vf + 1 doubles (column sums, then the count).
+size_t for_each_scratch_bytes(const TableDev& t);
+hipError_t launch_for_each(const TableDev& t, uint32_t n_rows, const ::pshbm_predicate& pred,
+                           double* scratch, hipStream_t s);
+// dead[r] = 1 where row r satisfies `pred`, else 0 / dead[rows[i]] = 1 for every rows[i] < n_rows.
+hipError_t launch_mark_pred(const TableDev& t, uint32_t n_rows, const ::pshbm_predicate& pred,
+                            uint8_t* dead, hipStream_t s);
+hipError_t launch_mark_rows(const uint32_t* rows, size_t n, uint32_t n_rows, uint8_t* dead,
+                            hipStream_t s);
+// Erase of the flagged rows in two steps. launch_erase_count: tile_cnt (erase_tiles(n_rows) + 1
+// words) becomes the prefix of the dead rows per tile of 4096 rows, info = {erased, rows left, -}
+// and the table's row count becomes the rows left. launch_erase_apply (erased = info[0], read back
+// by the host; lists: 3 * erased words): the erased keys' slots become markers, the surviving rows
+// are packed into [0, rows left) and their slots follow them.
+size_t erase_tiles(uint32_t n_rows);
+hipError_t launch_erase_count(const TableDev& t, uint32_t n_rows, const uint8_t* dead, uint32_t* tile_cnt,
+                              uint32_t* info, hipStream_t s);
+hipError_t launch_erase_apply(const TableDev& t, uint32_t n_rows, uint32_t erased, const uint8_t* dead,
+                              const uint32_t* tile_off, uint32_t* info, uint32_t* lists, hipStream_t s);
+// Every row < n_rows claims a slot for its key in a hash array that the caller has emptied.
+hipError_t launch_reinsert(const TableDev& t, uint32_t n_rows, hipStream_t s);
 
 // ---- sort (sort.hip) -----------------------------------------------------------------------
 // Stable radix sort of (key, value) pairs on the low `end_bit` bits (rounded up to whole digits of

@@ -319,6 +319,75 @@ public:
     }
 };
 
+// Result of the device for-each: what TestForEachResult {num, sum, count} generalises to
+// (pico-ps/test/TestOps.h:152-157): the records visited and the sum of every value column.
+struct HbmForEachResult {
+    int64_t num = 0;
+    std::vector<double> sums;
+    void merge(const HbmForEachResult& in) {  // merge_result, TestOps.h:180-184
+        num += in.num;
+        if (sums.size() < in.sums.size()) sums.resize(in.sums.size(), 0.0);
+        for (size_t i = 0; i < in.sums.size(); ++i) sums[i] += in.sums[i];
+    }
+    friend BinaryArchive& operator<<(BinaryArchive& ar, const HbmForEachResult& r) { return ar << r.num << r.sums; }
+    friend BinaryArchive& operator>>(BinaryArchive& ar, HbmForEachResult& r) { return ar >> r.num >> r.sums; }
+};
+
+// Server half of the read-only for-each (SparseTableForEachReadOperator::apply_request,
+// ForEachOperator.h:166-199). Request: i32 shard_id (a carried item would follow; this hook has
+// none). Response: Status, then the result of that shard. The hook is the count / column-sum
+// reduction over the records that satisfy `where` (none = all), evaluated on the device.
+class HbmForEachOperator {
+public:
+    explicit HbmForEachOperator(const Configure&) { _where.struct_size = sizeof _where; }
+    void set_where(const pshbm_predicate& w) { _where = w; }
+    void apply_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp_ret) {
+        int32_t shard_id;
+        req >> shard_id;
+        PSHBM_SCHECK(req.archive().is_exhausted(), "Bad Request: trailing bytes");           // :176
+        PSHBM_SCHECK(rt.local_shards().count(shard_id) != 0, "Bad Request: invalid shard_id");  // :177-178
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        HbmForEachResult res;
+        res.sums.assign(st.value_floats(), 0.0);
+        uint64_t count = 0;
+        int32_t rc = pshbm_for_each(st.get(shard_id), _where.n_terms ? &_where : nullptr, &count, res.sums.data());
+        PSHBM_SCHECK(rc == PSHBM_OK, std::string("for_each failed: ") + pshbm_last_error(st.get(shard_id)));
+        res.num = (int64_t)count;
+        PSResponse resp(req);
+        resp << Status();
+        resp.archive() << res;
+        resp_ret = std::move(resp);
+    }
+
+private:
+    pshbm_predicate _where{};
+};
+
+// Server half of erase-if (SparseTableEraseIfOperator::apply_request, EraseIfOperator.h:27-55).
+// Request: i32 shard_id. Response: Status and an empty archive. The erase_if hook is `where`.
+class HbmEraseIfOperator {
+public:
+    explicit HbmEraseIfOperator(const Configure&) { _where.struct_size = sizeof _where; }
+    void set_where(const pshbm_predicate& w) { _where = w; }
+    void apply_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp_ret) {
+        int32_t shard_id;
+        req >> shard_id;
+        PSHBM_SCHECK(req.archive().is_exhausted(), "Bad Request: trailing bytes");           // :34
+        PSHBM_SCHECK(rt.local_shards().count(shard_id) != 0, "Bad Request: invalid shard_id");  // :35-36
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        int32_t rc = pshbm_erase_if(st.get(shard_id), _where.n_terms ? &_where : nullptr, nullptr);
+        PSHBM_SCHECK(rc == PSHBM_OK, std::string("erase_if failed: ") + pshbm_last_error(st.get(shard_id)));
+        PSResponse resp(req);
+        BinaryArchive empty_ar;
+        resp << Status();
+        resp.archive() << empty_ar.size();
+        resp_ret = std::move(resp);
+    }
+
+private:
+    pshbm_predicate _where{};
+};
+
 struct DumpArgs {  // handler/DumpHandler.h: where to write and into how many files per node
     std::string uri;
     int32_t file_number = 1;

@@ -242,6 +242,73 @@ int main(int argc, char** argv) {
     }
     EXPECT(total_size(storage.get()) == (uint64_t)TEST_KEY_NUM * NUM_RANKS);
 
+    // for-each over the restored storage: num = every record, and the merged columns
+    // (ps_service_test.cpp:158-161; TestForEachOperator, TestOps.h:159-185); then erase_if(key % 2)
+    // (TestEraseIfOperator, TestOps.h:138-150): half the records are left (:163-166) and an erased
+    // key pulls 0 (:176-184)
+    {
+        HbmForEachOperator for_each_op(op_config);
+        HbmEraseIfOperator erase_if_op(op_config);
+        pshbm_predicate odd{};
+        odd.struct_size = sizeof odd;
+        odd.n_terms = 1;
+        odd.term[0].column = PSHBM_COL_KEY;
+        odd.term[0].cmp = PSHBM_CMP_MOD_EQ;
+        odd.term[0].u = 2;
+        odd.term[0].u2 = 1;
+        erase_if_op.set_where(odd);
+        auto sync_for_each = [&](Storage* st) {
+            HbmForEachResult total;
+            for (int32_t sh = 0; sh < NUM_SHARDS; ++sh) {
+                PSRequest req;
+                req << sh;
+                PSResponse resp;
+                for_each_op.apply_request(rt, req, st, resp);
+                Status s;
+                resp >> s;
+                EXPECT(s.ok());
+                HbmForEachResult one;
+                resp.archive() >> one;
+                total.merge(one);
+            }
+            return total;
+        };
+        double want_sum = 0, want_count = 0, even_sum = 0, even_count = 0;
+        for (uint64_t key : all_keys) {
+            const double count = 2.0 + ((key / TEST_KEY_NUM) % 2 == 0);
+            want_sum += (double)key * count;
+            want_count += count;
+            if (key % 2 == 0) {
+                even_sum += (double)key * count;
+                even_count += count;
+            }
+        }
+        HbmForEachResult all = sync_for_each(storage2.get());
+        EXPECT(all.num == (int64_t)TEST_KEY_NUM * NUM_RANKS);
+        EXPECT(all.sums.size() == 2 && all.sums[0] == want_sum && all.sums[1] == want_count);
+        for (int32_t sh = 0; sh < NUM_SHARDS; ++sh) {
+            PSRequest req;
+            req << sh;
+            PSResponse resp;
+            erase_if_op.apply_request(rt, req, storage2.get(), resp);
+            Status s;
+            resp >> s;
+            EXPECT(s.ok());
+        }
+        HbmForEachResult left = sync_for_each(storage2.get());
+        EXPECT(left.num == (int64_t)TEST_KEY_NUM * NUM_RANKS / 2);
+        EXPECT(left.sums[0] == even_sum && left.sums[1] == even_count);
+        EXPECT(total_size(storage2.get()) == (uint64_t)TEST_KEY_NUM * NUM_RANKS / 2);
+        bool ok;
+        auto v = pull(pull_op, rt, storage2.get(), all_keys, &ok);
+        EXPECT(ok);
+        for (size_t i = 0; i < all_keys.size(); ++i) {
+            const uint64_t key = all_keys[i];
+            const float count = key % 2 ? 0.0f : 2.0f + ((key / TEST_KEY_NUM) % 2 == 0);
+            EXPECT(v[i * 2] == (float)key * count && v[i * 2 + 1] == count);
+        }
+    }
+
     // direct push overwrites whole values (SparsePushOperator.h:557-562)
     {
         HbmDirectPushOperator direct(op_config);

@@ -46,6 +46,21 @@ def test_sparse(num_process):
     ops.append({"op": "expect_pull", "keys": missing, "rows": [[0, 0]] * len(missing),
                 "hit": [0] * len(missing)})
     ops.append({"op": "expect_size", "value": TEST_KEY_NUM * num_process})
+    # for-each over every record: num = records, and the merged sum / count columns
+    # (TestForEachOperator, TestOps.h:159-185; ps_service_test.cpp:158-161)
+    ops.append({"op": "expect_for_each", "where": [], "count": len(all_keys),
+                "sums": [sum(row(k)[0] for k in all_keys), sum(row(k)[1] for k in all_keys)]})
+    # erase_if(key % 2) (TestEraseIfOperator, TestOps.h:138-150), then half the records are left
+    # (ps_service_test.cpp:163-166) and an erased key pulls 0 (:176-184)
+    odd = [[-1, 6, [2, 1]]]   # key % 2 == 1
+    even_keys = [k for k in all_keys if k % 2 == 0]
+    ops.append({"op": "erase_if", "where": odd, "erased": len(all_keys) - len(even_keys)})
+    ops.append({"op": "expect_for_each", "where": [], "count": len(even_keys),
+                "sums": [sum(row(k)[0] for k in even_keys), sum(row(k)[1] for k in even_keys)]})
+    ops.append({"op": "expect_size", "value": len(even_keys)})
+    ops.append({"op": "expect_pull", "keys": all_keys,
+                "rows": [row(k) if k % 2 == 0 else [0, 0] for k in all_keys],
+                "hit": [1 if k % 2 == 0 else 0 for k in all_keys]})
     ops.append({"op": "clear"})                                           # :153
     ops.append({"op": "expect_size", "value": 0})                         # :154
     return {"name": f"test_sparse_{num_process}", "dim": 2, "optimizer": "SUM",

@@ -1,7 +1,7 @@
 """Runs a golden scenario (tests/golden/reference_known_answers.json) against a backend.
 
 A backend is anything with the method set shared by oracle.Oracle and the product's Table:
-pull / push / queue / store / dump / load / clear / size. `make` builds a fresh backend of the
+pull / push / queue / store / dump / load / for_each / erase_if / clear / size. `make` builds a fresh backend of the
 scenario's shape (used for the dump -> load round trip into a new storage).
 """
 import json
@@ -19,8 +19,16 @@ def load_scenarios():
         return json.load(f)["scenarios"]
 
 
-def run(scn, make):
-    """make(dim, optimizer) -> backend. Asserts every expectation of the scenario."""
+def _where(predicate, terms):
+    """[[column, cmp, operand], ...] of the fixture -> predicate object (None = every record)"""
+    if not terms:
+        return None
+    return predicate(*[(c, m, tuple(o) if isinstance(o, list) else o) for c, m, o in terms])
+
+
+def run(scn, make, predicate):
+    """make(dim, optimizer) -> backend; predicate(*terms) -> the backend's predicate object.
+    Asserts every expectation of the scenario."""
     dim, opt = scn["dim"], OPT[scn["optimizer"]]
     b = make(dim, opt)
     for step, op in enumerate(scn["ops"]):
@@ -44,6 +52,13 @@ def run(scn, make):
             assert st == 0, where
             np.testing.assert_array_equal(rows, np.array(op["rows"], dtype=np.float32), err_msg=where)
             np.testing.assert_array_equal(hit, np.array(op["hit"], dtype=np.uint8), err_msg=where)
+        elif kind == "expect_for_each":
+            st, count, sums = b.for_each(_where(predicate, op["where"]))
+            assert st == 0 and count == op["count"], where
+            np.testing.assert_array_equal(sums, np.array(op["sums"], dtype=np.float64), err_msg=where)
+        elif kind == "erase_if":
+            st, erased = b.erase_if(_where(predicate, op["where"]))
+            assert st == 0 and erased == op["erased"], where
         elif kind == "dump_load_roundtrip":
             # dump, load into a new storage; then clear that one and restore it (unique load)
             st, rec = b.dump()

@@ -45,7 +45,7 @@ def assert_same_table(t, r, exact):
 
 @pytest.mark.parametrize("scn", scenario.load_scenarios(), ids=lambda s: s["name"])
 def test_reference_known_answers(ps, scn):
-    scenario.run(scn, lambda dim, opt: ps.Table(dim, opt, capacity=1 << 12))
+    scenario.run(scn, lambda dim, opt: ps.Table(dim, opt, capacity=1 << 12), ps.predicate)
 
 
 @pytest.mark.parametrize("dim", [1, 3, 4, 8, 16, 64, 128, 260])
@@ -382,4 +382,119 @@ def test_device_pointer_entry_points(ps, orc, wl):
     assert r.queue(q, g) == 0 and r.store() == 0
     np.testing.assert_allclose(out.cpu().numpy(), r.pull(q)[1], rtol=RTOL, atol=ATOL)
     assert_same_table(t, r, exact=False)
+    t.close()
+
+
+def _random_predicates(mod, rng, vf):
+    """a few predicates on the key and on value columns, built for module `mod`"""
+    col = int(rng.integers(0, vf))
+    return [
+        None,
+        mod.predicate((mod.COL_KEY, mod.CMP_MOD_EQ, (3, 1))),
+        mod.predicate((col, mod.CMP_LT, -0.002)),
+        mod.predicate((mod.COL_KEY, mod.CMP_GE, 1 << 62), (col, mod.CMP_GT, 0.0)),
+        mod.predicate((0, mod.CMP_LE, 0.004), (vf - 1, mod.CMP_NE, 0.0), (mod.COL_KEY, mod.CMP_MOD_EQ, (2, 0))),
+        mod.predicate((mod.COL_KEY, mod.CMP_EQ, 12345)),          # nothing matches
+    ]
+
+
+@pytest.mark.parametrize("opt,dim", [("sum", 2), ("sgd", 16), ("adagrad", 8), ("ftrl", 100), ("sgd", 300)])
+def test_for_each_counts_and_sums(ps, orc, wl, opt, dim):
+    """Read-only for-each (pico-ps/operator/ForEachOperator.h:180-190) with the count / sum
+    reduction: counts are exact; the column sums are float64 sums of fp32 values added in another
+    order than the oracle's, so they agree to 1e-12 relative."""
+    rng = np.random.default_rng(dim)
+    t, r = pair(ps, orc, dim, opt, capacity=40000)
+    n = 30011
+    keys = wl.table_keys_np(0, n, seed=4)
+    vals = rng.normal(0, 0.01, (n, t.value_floats)).astype(np.float32)
+    assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+    for pg, po in zip(_random_predicates(ps, np.random.default_rng(1), t.value_floats),
+                      _random_predicates(orc, np.random.default_rng(1), t.value_floats)):
+        st, cnt, sums = t.for_each(pg)
+        st2, cnt2, sums2 = r.for_each(po)
+        assert st == st2 == 0 and cnt == cnt2
+        np.testing.assert_allclose(sums, sums2, rtol=1e-12, atol=1e-15)
+        again = t.for_each(pg)
+        assert again[1] == cnt and np.array_equal(again[2], sums)     # fixed order of additions
+    # an empty table, and a predicate that the library must refuse
+    t.clear()
+    assert t.for_each()[1:2] == (0,)
+    assert t.for_each(ps.predicate((t.value_floats, ps.CMP_LT, 0.0)))[0] == 1     # no such column
+    assert t.for_each(ps.predicate((0, ps.CMP_MOD_EQ, 1.0)))[0] == 1              # MOD_EQ needs the key
+    t.close()
+
+
+@pytest.mark.parametrize("opt,dim", [("sum", 2), ("sgd", 16), ("adagrad", 64), ("ftrl", 5)])
+def test_erase_if_and_erase_keep_the_table_consistent(ps, orc, wl, opt, dim):
+    """erase_if (pico-ps/operator/EraseIfOperator.h:38-47) by predicate and erase of chosen keys:
+    after every step the stored set equals the oracle's, the rows are dense (dump, iterate, size
+    agree), erased keys miss, survivors keep their values bit for bit, pushes and inserts after
+    the erase behave as on a table that never held the erased keys."""
+    rng = np.random.default_rng(dim + 100)
+    t, r = pair(ps, orc, dim, opt, capacity=60000)
+    n = 40000
+    keys = wl.table_keys_np(0, n, seed=6)
+    vals = rng.normal(0, 0.01, (n, t.value_floats)).astype(np.float32)
+    if opt == "adagrad":
+        vals[:, dim:] = 0.1
+    if opt == "ftrl":
+        vals[:, 2 * dim:] = vals[:, dim:2 * dim] ** 2
+    assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+
+    def check():
+        assert t.size() == r.size()
+        assert_same_table(t, r, exact=True)
+        st, rec = t.iterate(0, t.size() + 10)
+        assert st == 0 and rec.size == t.size() and np.unique(rec["key"]).size == rec.size
+        q = np.concatenate([keys[:3000], keys[-3000:]])
+        a, b = t.pull(q), r.pull(q)
+        np.testing.assert_array_equal(a[2], b[2])
+        np.testing.assert_array_equal(a[1], b[1])
+
+    # by predicate: a third of the keys, then a value column
+    for pg, po in ((ps.predicate((ps.COL_KEY, ps.CMP_MOD_EQ, (3, 0))), orc.predicate((orc.COL_KEY, orc.CMP_MOD_EQ, (3, 0)))),
+                   (ps.predicate((0, ps.CMP_GT, 0.005)), orc.predicate((0, orc.CMP_GT, 0.005)))):
+        a, b = t.erase_if(pg), r.erase_if(po)
+        assert a == b and a[0] == 0 and a[1] > 0
+        check()
+    # chosen keys, with repeats and keys that are not stored
+    victims = np.concatenate([keys[rng.integers(0, n, 5000)], wl.fresh_keys_np(rng, 300), keys[:10], keys[:10]])
+    a, b = t.erase(victims), r.erase(victims)
+    assert a == b and a[0] == 0
+    check()
+    # the table keeps working: push with duplicates re-inserts some erased keys, then more erases
+    q = np.concatenate([keys[rng.integers(0, n, 20000)], wl.fresh_keys_np(rng, 500)])
+    g = rng.integers(-3, 4, (q.size, dim)).astype(np.float32) if opt == "sum" else rng.normal(0, 1e-3, (q.size, dim)).astype(np.float32)
+    uq, first = np.unique(q, return_index=True)              # distinct keys: bit-exact for every optimizer
+    assert t.push(uq, g[first]) == 0 and r.push(uq, g[first]) == 0
+    check()
+    assert t.compact() == 0
+    check()
+    a, b = t.erase_if(ps.predicate((ps.COL_KEY, ps.CMP_MOD_EQ, (2, 1)))), r.erase_if(orc.predicate((orc.COL_KEY, orc.CMP_MOD_EQ, (2, 1))))
+    assert a == b
+    check()
+    # erase everything, in two ways
+    a, b = t.erase_if(None), r.erase_if(None)
+    assert a == b and t.size() == 0
+    assert t.set(keys[:100], vals[:100]) == 0 and t.erase(keys[:100]) == (0, 100) and t.size() == 0
+    st, cnt, sums = t.for_each()
+    assert cnt == 0 and not sums.any()
+    t.close()
+
+
+def test_erase_many_rounds_triggers_rebuild(ps, orc, wl):
+    """Markers of erased keys pile up in the slots until the hash array is rebuilt by itself (an
+    eighth of the slots); lookups, inserts and erases must not notice."""
+    rng = np.random.default_rng(9)
+    t, r = pair(ps, orc, 4, "sum", capacity=4000)
+    for it in range(12):
+        keys = wl.table_keys_np(it * 2500, 2500, seed=8)
+        vals = rng.integers(-5, 6, (2500, 4)).astype(np.float32)
+        assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+        assert t.erase(keys[:2400]) == r.erase(keys[:2400]) == (0, 2400)
+        assert t.erase_if(ps.predicate((ps.COL_KEY, ps.CMP_EQ, int(keys[2400])))) == (0, 1)
+        assert r.erase_if(orc.predicate((orc.COL_KEY, orc.CMP_EQ, int(keys[2400])))) == (0, 1)
+        assert_same_table(t, r, exact=True)
+    assert t.size() == r.size() == 12 * 99
     t.close()

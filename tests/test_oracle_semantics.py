@@ -8,7 +8,7 @@ import scenario
 
 @pytest.mark.parametrize("scn", scenario.load_scenarios(), ids=lambda s: s["name"])
 def test_reference_known_answers(orc, scn):
-    scenario.run(scn, lambda dim, opt: orc.Oracle(dim, opt, capacity=1 << 16))
+    scenario.run(scn, lambda dim, opt: orc.Oracle(dim, opt, capacity=1 << 16), orc.predicate)
 
 
 class DictModel:
@@ -159,3 +159,58 @@ def test_reserved_keys_are_rejected(orc):
     assert o.push(bad, np.ones((2, 1), np.float32)) == orc.ERROR
     assert o.pull(bad)[0] == orc.ERROR
     assert o.size() == 0
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_for_each_and_erase_against_dict_model(orc, seed):
+    """for_each / erase_if / erase against a plain dict; the hooks are the reference's test
+    operators generalised: count + column sums (pico-ps/test/TestOps.h:159-185), erase by a
+    comparison on the key or a value column (TestOps.h:138-150 erases the odd keys)."""
+    rng = np.random.default_rng(seed)
+    dim = 3
+    o = orc.Oracle(dim, orc.OPT_SUM, capacity=5000)
+    model = {}
+    keys = rng.integers(0, 3000, 2000).astype(np.uint64)
+    vals = rng.integers(-9, 10, (2000, dim)).astype(np.float32)
+    assert o.set(keys, vals) == 0
+    for k, v in zip(keys, vals):
+        model[int(k)] = v.copy()
+
+    def check(where, fn):
+        st, cnt, sums = o.for_each(where)
+        sel = [v for k, v in model.items() if fn(k, v)]
+        assert st == 0 and cnt == len(sel)
+        np.testing.assert_array_equal(sums, np.sum(np.array(sel, dtype=np.float64).reshape(-1, dim), axis=0))
+
+    check(None, lambda k, v: True)
+    check(orc.predicate((orc.COL_KEY, orc.CMP_MOD_EQ, (2, 1))), lambda k, v: k % 2 == 1)
+    check(orc.predicate((1, orc.CMP_GE, 3.0), (orc.COL_KEY, orc.CMP_LT, 1500)), lambda k, v: v[1] >= 3 and k < 1500)
+    check(orc.predicate((0, orc.CMP_NE, 0.0), (2, orc.CMP_LE, -1.0), (1, orc.CMP_EQ, 2.0)),
+          lambda k, v: v[0] != 0 and v[2] <= -1 and v[1] == 2)
+    # erase_if: the odd keys (the reference's own hook), then a value column
+    st, gone = o.erase_if(orc.predicate((orc.COL_KEY, orc.CMP_MOD_EQ, (2, 1))))
+    odd = [k for k in model if k % 2 == 1]
+    assert st == 0 and gone == len(odd)
+    for k in odd:
+        del model[k]
+    st, gone = o.erase_if(orc.predicate((2, orc.CMP_GT, 4.0)))
+    big = [k for k, v in model.items() if v[2] > 4]
+    assert gone == len(big)
+    for k in big:
+        del model[k]
+    # erase of chosen keys: repeats and absent keys are ignored
+    victims = np.array(list(model)[:300] + list(model)[:5] + [999_999, 888_888], dtype=np.uint64)
+    st, gone = o.erase(victims)
+    assert st == 0 and gone == 300
+    for k in list(model)[:300]:
+        del model[k]
+    assert o.size() == len(model)
+    st, rec = o.dump()
+    assert sorted(rec["key"].tolist()) == sorted(model)
+    for k, v in zip(rec["key"], rec["value"]):
+        np.testing.assert_array_equal(v, model[int(k)])
+    st, rows, hit = o.pull(np.array(odd[:50] + list(model)[:50], dtype=np.uint64))
+    assert not hit[:50].any() and hit[50:].all() and not rows[:50].any()
+    check(None, lambda k, v: True)
+    assert o.erase_if(None) == (0, len(model)) and o.size() == 0
+    o.close()
