@@ -230,3 +230,63 @@ def test_c4_size_aggregation_matches_presummed(ps, wl):
     again, _ = pull(t, wl.keys_of_index_torch(uniq, 0), dim)
     assert torch.equal(again, got_a)
     t.close()
+
+
+def test_c2_size_for_each_and_erase_if(ps, wl):
+    """For-each and erase-if over 100M keys: the column sums of the closed form are integers, so
+    the float64 sums are exact in any order; erasing the keys with an odd index-derived column
+    leaves exactly the others, dense, with their values, and the table keeps working."""
+    import time
+    n_table, dim, batch = 100_000_000, 16, 1_000_000
+    t = build(ps, wl, n_table, dim, dict(optimizer=1, lr=0.5), batch, 8 * batch)
+    # expected column sums of the closed form, in chunks (exact integers in float64)
+    want = torch.zeros(dim, dtype=torch.float64, device="cuda")
+    n_sel = 0
+    sel_sum = torch.zeros(dim, dtype=torch.float64, device="cuda")
+    for start in range(0, n_table, 10_000_000):
+        idx = torch.arange(start, start + 10_000_000, device="cuda")
+        v = closed_form(idx, dim, dim).to(torch.float64)
+        want += v.sum(0)
+        m = v[:, 3] > 100.0                       # column 3 above 100: about a tenth of the keys
+        n_sel += int(m.sum())
+        sel_sum += v[m].sum(0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    st, cnt, sums = t.for_each()
+    dt_all = time.perf_counter() - t0
+    assert st == 0 and cnt == n_table
+    np.testing.assert_array_equal(sums, want.cpu().numpy())
+    where = ps.predicate((3, ps.CMP_GT, 100.0))
+    st, cnt, sums = t.for_each(where)
+    assert st == 0 and cnt == n_sel
+    np.testing.assert_array_equal(sums, sel_sum.cpu().numpy())
+
+    t0 = time.perf_counter()
+    st, erased = t.erase_if(where)
+    dt_erase = time.perf_counter() - t0
+    assert st == 0 and erased == n_sel and t.size() == n_table - n_sel
+    st, cnt, sums = t.for_each()
+    assert cnt == n_table - n_sel
+    np.testing.assert_array_equal(sums, (want - sel_sum).cpu().numpy())
+    assert t.for_each(where)[1] == 0
+    # erased keys miss, the others keep their rows; the slab is dense again
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(6)
+    idx = torch.randint(0, n_table, (batch,), device="cuda", generator=gen)
+    v = closed_form(idx, dim, dim)
+    gone = v[:, 3] > 100.0
+    out, hit = pull(t, wl.keys_of_index_torch(idx, 0), dim)
+    assert torch.equal(hit.bool(), ~gone)
+    assert torch.equal(out[~gone], v[~gone]) and not bool(out[gone].any())
+    st, rec = t.iterate(n_table - n_sel - 1000, 2000)
+    assert st == 0 and rec.size == 1000 and not (rec["value"][:, 3] > 100.0).any()
+    # pushes after the erase: erased keys come back as new keys (zero weights), others update
+    g = torch.ones(batch, dim, device="cuda")
+    uniq = torch.unique(idx)
+    push(t, wl.keys_of_index_torch(uniq, 0), g[: uniq.numel()])
+    vu = closed_form(uniq, dim, dim)
+    vu[vu[:, 3] > 100.0] = 0.0
+    out, hit = pull(t, wl.keys_of_index_torch(uniq, 0), dim)
+    assert bool(hit.all()) and torch.equal(out, vu - 0.5)
+    print(f"\nfor_each over {n_table} rows: {dt_all * 1e3:.2f} ms; erase_if of {n_sel} rows: {dt_erase * 1e3:.2f} ms")
+    t.close()
