@@ -10,6 +10,10 @@
 //   HbmDirectPushOperator  <- DirectPushOperator                       (operator/SparsePushOperator.h:520-574)
 //   HbmDumpOperator        <- BaseKVTextFileDumpOperator::apply_request (operator/DumpOperator.h:137-183)
 //   HbmLoadOperator        <- BaseKVTextFileLoadOperator::restore      (operator/LoadOperator.h:164-213)
+//   HbmForEachOperator     <- SparseTableForEachReadOperator           (operator/ForEachOperator.h:150-233)
+//   HbmEraseIfOperator     <- SparseTableEraseIfOperator               (operator/EraseIfOperator.h:18-58)
+//   HbmShuffleOperator     <- ShufflePushItemsGenerator / apply_purge_request (operator/UpdateContextOperator.h:143-297)
+//   HbmRestoreOperator     <- coordinated restore                      (operator/RestoreOperator.h:100-151)
 //
 // The client halves (generate_request, apply_response, ...) are not here: they run in the
 // application process and are inherited unchanged from the reference's templates.
@@ -476,6 +480,151 @@ public:
 
 private:
     size_t _block_size;
+};
+
+// Re-sharding after the set of servers changed (UpdateContextOperator.h:100-305). The host logic
+// that drives it stays as it is; what it needs from the storage is (1) the items of a shard that
+// now belong elsewhere, a bounded block at a time, and (2) the purge of those items.
+// PARTITIONER::partition(key, global_shard_num) is the reference's key partitioner
+// (common/Partitioner.h:43-61), evaluated on the host.
+template <class PARTITIONER>
+class HbmShuffleOperator {
+public:
+    explicit HbmShuffleOperator(const Configure& config)
+        : _block_items((size_t)config.number("shuffle_block_items", 4096)) {}
+
+    // PushItemsGenerator (UpdateContextOperator.h:214-297): walks the shard in slab order and hands
+    // out the items whose partition is no longer `shard_id` (all items when the shard changes node).
+    class PushItemsGenerator {
+    public:
+        PushItemsGenerator(HbmShardStorage& st, int32_t shard_id, int32_t global_shard_num, bool shard_node_change,
+                           size_t block_items, PARTITIONER& partitioner)
+            : _st(st), _shard_id(shard_id), _global_shard_num(global_shard_num),
+              _shard_node_change(shard_node_change), _block_items(block_items), _partitioner(partitioner) {}
+        // Appends up to one block of (key, value) to keys / vals; returns how many. 0 = finished.
+        size_t generate_push_items(std::vector<uint64_t>& keys, std::vector<float>& vals) {
+            const size_t rec = _st.record_bytes(), vf = _st.value_floats();
+            std::vector<char> buf(_block_items * rec);
+            size_t count = 0;
+            while (count == 0 && !_finished) {
+                size_t got = 0;
+                int32_t rc = pshbm_iterate(_st.get(_shard_id), _offset, _block_items, buf.data(), &got);
+                PSHBM_SCHECK(rc == PSHBM_OK, "iterate failed");
+                _offset += got;
+                _finished = got < _block_items;
+                for (size_t i = 0; i < got; ++i) {
+                    uint64_t key;
+                    std::memcpy(&key, buf.data() + i * rec, 8);
+                    if (_partitioner.partition(key, _global_shard_num) != _shard_id || _shard_node_change) {  // :273-277
+                        keys.push_back(key);
+                        const float* v = reinterpret_cast<const float*>(buf.data() + i * rec + 8);
+                        vals.insert(vals.end(), v, v + vf);
+                        ++count;
+                    }
+                }
+            }
+            return count;
+        }
+
+    private:
+        HbmShardStorage& _st;
+        int32_t _shard_id, _global_shard_num;
+        bool _shard_node_change;
+        size_t _block_items, _offset = 0;
+        bool _finished = false;
+        PARTITIONER& _partitioner;
+    };
+
+    std::unique_ptr<PushItemsGenerator> lock_push_items_generator(RuntimeInfo& new_rt, Storage* storage,
+                                                                  int32_t shard_id, bool shard_node_change) {
+        return std::make_unique<PushItemsGenerator>(*static_cast<HbmShardStorage*>(storage), shard_id,
+                                                    new_rt.global_shard_num(), shard_node_change, _block_items,
+                                                    _key_partitioner);
+    }
+
+    // apply_purge_request (UpdateContextOperator.h:143-196): a shard that stays local keeps only the
+    // keys that still map to it, and its hash array is rebuilt (safe_shrink); any other shard goes.
+    void apply_purge_request(RuntimeInfo& new_rt, PSRequest& req, Storage* storage, PSResponse& resp) {
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        int32_t shard_id;
+        req >> shard_id;
+        if (new_rt.local_shards().count(shard_id)) {
+            pshbm_table* t = st.get(shard_id);
+            const size_t rec = st.record_bytes();
+            std::vector<char> buf(_block_items * rec);
+            std::vector<uint64_t> gone;
+            for (size_t offset = 0;;) {  // the keys first: erasing moves rows, which would disturb the walk
+                size_t got = 0;
+                PSHBM_SCHECK(pshbm_iterate(t, offset, _block_items, buf.data(), &got) == PSHBM_OK, "iterate failed");
+                for (size_t i = 0; i < got; ++i) {
+                    uint64_t key;
+                    std::memcpy(&key, buf.data() + i * rec, 8);
+                    if (_key_partitioner.partition(key, new_rt.global_shard_num()) != shard_id) gone.push_back(key);
+                }
+                offset += got;
+                if (got < _block_items) break;
+            }
+            PSHBM_SCHECK(pshbm_erase(t, gone.data(), gone.size(), nullptr) == PSHBM_OK, "erase failed");
+            PSHBM_SCHECK(pshbm_compact(t) == PSHBM_OK, "compact failed");
+        } else {
+            st.erase_shard(shard_id);
+        }
+        resp = PSResponse(req);
+        resp << Status();
+    }
+
+private:
+    size_t _block_items;
+    PARTITIONER _key_partitioner;
+};
+
+// Coordinated restore of a dead node's shard from a live replica (RestoreOperator.h:100-151): the
+// serving side answers (offset, batch) slices of a shard, the restoring side inserts what it gets
+// and keeps what it already has.
+class HbmRestoreOperator {
+public:
+    explicit HbmRestoreOperator(const Configure&) {}
+    void apply_coordinated_restore_request(PSRequest& req, Storage* storage, PSResponse& resp) {
+        int32_t storage_id, iterator_id, shard_id;
+        uint64_t offset, batch_size;
+        req >> storage_id >> iterator_id >> offset >> batch_size >> shard_id;
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        if (st.get(shard_id) == nullptr) {  // :111-115
+            resp.rpc_response().set_error_code(RpcErrorCodeType::ELOGICERROR);
+            resp << Status::InvalidID("Invalid shard id");
+            return;
+        }
+        BinaryArchive ar;
+        const size_t num = st.iterate_batch_as_binary_archive(shard_id, offset, batch_size, ar);
+        const bool finished = num < batch_size;
+        resp = PSResponse(req);
+        resp << storage_id << shard_id << finished << iterator_id << (uint64_t)(offset + num) << (uint64_t)num;
+        ps_serialize(resp.lazy(), std::move(ar.buffer()));
+    }
+    // returns {finished, next_offset}
+    std::pair<bool, uint64_t> apply_coordinated_restore_response(PSResponse& resp, Storage* storage) {
+        int32_t storage_id, shard_id, iterator_id;
+        bool finished;
+        uint64_t next_offset, num;
+        resp >> storage_id >> shard_id >> finished >> iterator_id >> next_offset >> num;
+        std::vector<char> block;
+        ps_deserialize(resp.lazy(), block);
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        const size_t rec = st.record_bytes();
+        PSHBM_SCHECK(block.size() == num * rec, "restore block size mismatch");
+        // ht.insert keeps a key that is present (:141-146): drop those records before the load
+        std::vector<uint64_t> keys(num);
+        for (size_t i = 0; i < num; ++i) std::memcpy(&keys[i], block.data() + i * rec, 8);
+        std::vector<float> rows(num * st.dim());
+        std::vector<uint8_t> hit(num);
+        pshbm_table* t = st.get(shard_id);
+        PSHBM_SCHECK(pshbm_pull(t, keys.data(), num, rows.data(), hit.data(), 0) == PSHBM_OK, "pull failed");
+        std::vector<char> fresh;
+        for (size_t i = 0; i < num; ++i)
+            if (!hit[i]) fresh.insert(fresh.end(), block.begin() + i * rec, block.begin() + (i + 1) * rec);
+        PSHBM_SCHECK(pshbm_load(t, fresh.data(), fresh.size() / rec, PSHBM_LOAD_UNIQUE) == PSHBM_OK, "load failed");
+        return {finished, next_offset};
+    }
 };
 
 }  // namespace pshbm_host

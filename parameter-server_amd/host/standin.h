@@ -97,6 +97,7 @@ public:
     static Status Error(const std::string& m) { return Status(StatusCode::ERROR, m); }
     static Status Fatal(const std::string& m) { return Status(StatusCode::FATAL, m); }
     static Status InvalidConfig(const std::string& m) { return Status(StatusCode::INVALID_CONFIG, m); }
+    static Status InvalidID(const std::string& m) { return Status(StatusCode::INVALID_ID, m); }
     bool ok() const { return _code == StatusCode::OK; }
     bool IsOOM() const { return _code == StatusCode::OUT_OF_MEMORY; }
     StatusCode code() const { return _code; }

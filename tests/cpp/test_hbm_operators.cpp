@@ -309,6 +309,97 @@ int main(int argc, char** argv) {
         }
     }
 
+    // coordinated restore of a shard from a replica, slice by slice (RestoreOperator.h:100-151), into
+    // a storage that already holds some of the keys; then re-sharding from 2 to 3 shards: the items
+    // that leave shard 0, and its purge (UpdateContextOperator.h:143-297)
+    {
+        struct ModPartitioner {
+            int32_t partition(uint64_t key, int32_t global_shard_num) { return (int32_t)(key % (uint64_t)global_shard_num); }
+        };
+        std::unique_ptr<Storage> storage3 = storage_op.create_storage(rt, 2);
+        {   // a few keys are there already, with other values: the restore must keep them
+            HbmDirectPushOperator direct(op_config);
+            std::vector<Pair> items = {{0, {-1.0f, -1.0f}}, {2, {-2.0f, -2.0f}}};
+            PSRequest req;
+            req << (int32_t)NUM_SHARDS << (int32_t)1;
+            req << (int32_t)0 << (int32_t)items.size();
+            const char* p = reinterpret_cast<const char*>(items.data());
+            req.lazy().emplace_back(p, p + items.size() * sizeof(Pair));
+            req << (int32_t)1 << (int32_t)0;
+            PSResponse resp;
+            direct.apply_async_push_request(rt, req, storage3.get(), nullptr, resp);
+        }
+        HbmRestoreOperator restore_op(op_config);
+        for (int32_t sh = 0; sh < NUM_SHARDS; ++sh) {
+            uint64_t offset = 0;
+            for (bool finished = false; !finished;) {
+                PSRequest req;
+                req << (int32_t)0 << (int32_t)7 << offset << (uint64_t)37 << sh;
+                PSResponse resp;
+                restore_op.apply_coordinated_restore_request(req, storage.get(), resp);
+                EXPECT(resp.error_code() == RpcErrorCodeType::SUCC);
+                auto r = restore_op.apply_coordinated_restore_response(resp, storage3.get());
+                finished = r.first;
+                offset = r.second;
+            }
+        }
+        EXPECT(total_size(storage3.get()) == (uint64_t)TEST_KEY_NUM * NUM_RANKS);
+        bool ok;
+        auto v3 = pull(pull_op, rt, storage3.get(), all_keys, &ok);
+        for (size_t i = 0; i < all_keys.size(); ++i) {
+            const uint64_t key = all_keys[i];
+            const float count = 2.0f + ((key / TEST_KEY_NUM) % 2 == 0);
+            if (key == 0 || key == 2)
+                EXPECT(v3[i * 2] == -(float)(key / 2 + 1) && v3[i * 2 + 1] == -(float)(key / 2 + 1));
+            else
+                EXPECT(v3[i * 2] == (float)key * count && v3[i * 2 + 1] == count);
+        }
+        {   // a request for a shard that is not there
+            PSRequest req;
+            req << (int32_t)0 << (int32_t)7 << (uint64_t)0 << (uint64_t)10 << (int32_t)9;
+            PSResponse resp;
+            restore_op.apply_coordinated_restore_request(req, storage.get(), resp);
+            EXPECT(resp.error_code() == RpcErrorCodeType::ELOGICERROR);
+        }
+
+        Configure shuffle_config = op_config;
+        shuffle_config.set("shuffle_block_items", 64);
+        HbmShuffleOperator<ModPartitioner> shuffle_op(shuffle_config);
+        RuntimeInfo new_rt(0, {0, 1, 2});  // three shards now; this node keeps 0 and 1
+        auto& st3 = *static_cast<HbmShardStorage*>(storage3.get());
+        std::set<uint64_t> leaving;
+        for (int32_t sh = 0; sh < NUM_SHARDS; ++sh) {
+            auto gen = shuffle_op.lock_push_items_generator(new_rt, storage3.get(), sh, false);
+            std::vector<uint64_t> keys;
+            std::vector<float> vals;
+            size_t blocks = 0;
+            while (gen->generate_push_items(keys, vals)) ++blocks;
+            EXPECT(blocks >= 1 && vals.size() == keys.size() * 2);
+            for (size_t i = 0; i < keys.size(); ++i) {
+                EXPECT(keys[i] % NUM_SHARDS == (uint64_t)sh && keys[i] % 3 != (uint64_t)sh);
+                EXPECT(leaving.insert(keys[i]).second);
+                if (keys[i] != 0 && keys[i] != 2) EXPECT(vals[i * 2 + 1] == 2.0f + ((keys[i] / TEST_KEY_NUM) % 2 == 0));
+            }
+        }
+        size_t expect_leaving = 0;
+        for (uint64_t key : all_keys) expect_leaving += (key % 3 != key % NUM_SHARDS);
+        EXPECT(leaving.size() == expect_leaving);
+        for (int32_t sh = 0; sh < NUM_SHARDS; ++sh) {
+            PSRequest req;
+            req << sh;
+            PSResponse resp;
+            shuffle_op.apply_purge_request(new_rt, req, storage3.get(), resp);
+            Status s;
+            resp >> s;
+            EXPECT(s.ok());
+        }
+        EXPECT(total_size(storage3.get()) == all_keys.size() - expect_leaving);
+        v3 = pull(pull_op, rt, storage3.get(), all_keys, &ok);
+        for (size_t i = 0; i < all_keys.size(); ++i)
+            if (leaving.count(all_keys[i])) EXPECT(v3[i * 2] == 0.0f && v3[i * 2 + 1] == 0.0f);
+        (void)st3;
+    }
+
     // direct push overwrites whole values (SparsePushOperator.h:557-562)
     {
         HbmDirectPushOperator direct(op_config);
