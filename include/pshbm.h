@@ -73,6 +73,8 @@ typedef struct pshbm_config {
     int32_t read_only;           /* pulls never insert: PullOperator.h:45-47 */
     uint64_t max_batch;          /* workspace is pre-sized for batches of this many keys;
                                     larger batches grow it (which allocates and synchronizes) */
+    int32_t track_increment;     /* remember which keys pushes touch, for pshbm_take_increment */
+    int32_t reserved;
 } pshbm_config;
 
 typedef struct pshbm_stats {
@@ -241,6 +243,19 @@ int32_t pshbm_erase_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, uint64
  * their slots: the counterpart of safe_shrink (KVShardStorage.h:816-825). Erase calls do this by
  * themselves once the markers fill an eighth of the slots. */
 int32_t pshbm_compact(pshbm_table* t);
+
+/* ---- increment -----------------------------------------------------------------------------
+ * The reference copies every value that a push or a store writes into a second storage, the
+ * increment (safe_set(*incr_ht, ...), pico-ps/operator/SparsePushOperator.h:253-266,394-407), which
+ * the sync operator reads and empties from time to time (IncrementStorage::read_storage,
+ * pico-ps/service/IncrementStorage.h:29-36; operator/SyncOperator.h:185-266) to feed other
+ * clusters. Here a table created with track_increment marks the rows that pushes and stores
+ * update. pshbm_take_increment writes the {key, value} records of the marked keys, with the
+ * values they have now, and clears the marks; if capacity_records is too small nothing is
+ * cleared, *n_out is the number needed and the status is ERROR. Pulls that insert, set / load and
+ * keys that were erased since they were marked are not part of the increment. */
+int32_t pshbm_increment_size(pshbm_table* t, uint64_t* n);
+int32_t pshbm_take_increment(pshbm_table* t, void* records, size_t capacity_records, size_t* n_out);
 
 /* Empties the table and keeps its memory: KVShardStorage.h:902-908. */
 int32_t pshbm_clear(pshbm_table* t);

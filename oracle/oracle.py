@@ -32,6 +32,7 @@ class _Config(C.Structure):
         ("l2", C.c_float),
         ("capacity", C.c_uint64),
         ("read_only", C.c_int32),
+        ("track_increment", C.c_int32),
     ]
 
 
@@ -98,6 +99,8 @@ def lib():
         L.pso_for_each.argtypes = [vp, vp, C.POINTER(C.c_uint64), vp]
         L.pso_erase_if.argtypes = [vp, vp, C.POINTER(C.c_uint64)]
         L.pso_erase.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_uint64)]
+        L.pso_increment_size.argtypes = [vp, C.POINTER(C.c_uint64)]
+        L.pso_take_increment.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_size_t)]
         L.pso_clear.argtypes = [vp]
         L.pso_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         _lib = L
@@ -123,11 +126,12 @@ class Oracle:
     """One shard of the reference's KV storage with the operator loops on top (CPU, scalar)."""
 
     def __init__(self, dim, optimizer=OPT_SUM, lr=0.0, init_acc=0.0, alpha=0.0, beta=0.0, l1=0.0,
-                 l2=0.0, capacity=1 << 20, read_only=False):
+                 l2=0.0, capacity=1 << 20, read_only=False, track_increment=False):
         self.dim = dim
         self.optimizer = optimizer
         self.value_floats = lib().pso_value_floats(dim, optimizer)
-        cfg = _Config(dim, optimizer, lr, init_acc, alpha, beta, l1, l2, capacity, int(read_only))
+        cfg = _Config(dim, optimizer, lr, init_acc, alpha, beta, l1, l2, capacity, int(read_only),
+                      int(track_increment))
         self._h = C.c_void_p()
         st = lib().pso_create(C.byref(cfg), C.byref(self._h))
         if st != OK:
@@ -193,6 +197,19 @@ class Oracle:
         got = C.c_size_t()
         st = lib().pso_iterate(self._h, offset, batch, rec.ctypes.data, C.byref(got))
         return st, rec[: got.value]
+
+    def increment_size(self):
+        n = C.c_uint64()
+        lib().pso_increment_size(self._h, C.byref(n))
+        return OK, n.value
+
+    def take_increment(self, capacity=None):
+        if capacity is None:
+            capacity = self.increment_size()[1]
+        rec = np.empty(max(capacity, 1), dtype=record_dtype(self.value_floats))
+        got = C.c_size_t()
+        st = lib().pso_take_increment(self._h, rec.ctypes.data, capacity, C.byref(got))
+        return st, rec[: got.value if st == OK else 0]
 
     def for_each(self, where=None):
         n = C.c_uint64()

@@ -60,6 +60,7 @@ struct Config {
     float lr, init_acc, alpha, beta, l1, l2;
     uint64_t capacity;
     int32_t read_only;
+    int32_t track_increment;
 };
 
 struct Oracle {
@@ -71,6 +72,11 @@ struct Oracle {
     // sync-push queue (the MPSC queue of blocks, KVShardStorage.h:677-726), flattened
     std::vector<uint64_t> q_keys;
     std::vector<float> q_grads;
+    // the increment: keys whose values a push or a store wrote since the last take (the reference
+    // keeps copies of the values in a second storage, SparsePushOperator.h:253-266; the values are
+    // read when the increment is taken, which gives the same records as long as nothing is pushed
+    // in between)
+    std::unordered_set<uint64_t> touched;
 };
 
 uint32_t value_floats(uint32_t dim, int32_t opt) {
@@ -204,6 +210,7 @@ int32_t apply_unique(Oracle& o, const std::vector<uint64_t>& ukeys, const std::v
             r = it->second;
         }
         apply_update(o.c, &usum[u * o.c.dim], &o.rows[(size_t)r * o.vf]);
+        if (o.c.track_increment) o.touched.insert(ukeys[u]);  // safe_set(*incr_ht, ...), :253-266
     }
     return ST_OK;
 }
@@ -218,6 +225,7 @@ struct pso_config {
     float lr, init_acc, alpha, beta, l1, l2;
     uint64_t capacity;
     int32_t read_only;
+    int32_t track_increment;
 };
 
 uint32_t pso_value_floats(uint32_t dim, int32_t opt) { return value_floats(dim, opt); }
@@ -229,7 +237,8 @@ int32_t pso_create(const pso_config* cfg, void** out) {
         return ST_INVALID_CONFIG;
     auto* o = new Oracle();
     o->c = Config{cfg->dim, cfg->optimizer, cfg->lr,  cfg->init_acc,  cfg->alpha,
-                  cfg->beta, cfg->l1,       cfg->l2,  cfg->capacity,  cfg->read_only};
+                  cfg->beta, cfg->l1,       cfg->l2,  cfg->capacity,  cfg->read_only,
+                  cfg->track_increment};
     o->vf = value_floats(cfg->dim, cfg->optimizer);
     *out = o;
     return ST_OK;
@@ -442,6 +451,7 @@ static bool holds(const pso_predicate* p, uint64_t key, const float* v) {
 // place, so the slab stays dense; iteration order after an erase is unspecified, as in the reference.
 static void erase_row(Oracle& o, uint32_t r) {
     const uint32_t last = (uint32_t)o.row_keys.size() - 1;
+    o.touched.erase(o.row_keys[r]);
     o.map.erase(o.row_keys[r]);
     if (r != last) {
         o.row_keys[r] = o.row_keys[last];
@@ -504,12 +514,37 @@ int32_t pso_erase(void* h, const uint64_t* keys, size_t n, uint64_t* erased) {
     return ST_OK;
 }
 
+// IncrementStorage::read_storage + the sync operator's walk of it (service/IncrementStorage.h:29-36,
+// operator/SyncOperator.h:185-266): the {key, value} records of the keys pushes wrote since the
+// last take, then the increment is empty. Too little room: ST_ERROR, *n_out = records needed.
+int32_t pso_increment_size(void* h, uint64_t* n) {
+    *n = static_cast<Oracle*>(h)->touched.size();
+    return ST_OK;
+}
+int32_t pso_take_increment(void* h, void* records, size_t capacity_records, size_t* n_out) {
+    Oracle& o = *static_cast<Oracle*>(h);
+    *n_out = o.touched.size();
+    if (o.touched.size() > capacity_records) return ST_ERROR;
+    const size_t rec = 8 + (size_t)o.vf * 4;
+    char* p = static_cast<char*>(records);
+    size_t w = 0;
+    for (uint64_t k : o.touched) {
+        const uint32_t r = o.map.at(k);
+        std::memcpy(p + w * rec, &k, 8);
+        std::memcpy(p + w * rec + 8, &o.rows[(size_t)r * o.vf], (size_t)o.vf * 4);
+        ++w;
+    }
+    o.touched.clear();
+    return ST_OK;
+}
+
 // KVShardStorage::clear, KVShardStorage.h:902-908
 int32_t pso_clear(void* h) {
     Oracle& o = *static_cast<Oracle*>(h);
     o.map.clear();
     o.rows.clear();
     o.row_keys.clear();
+    o.touched.clear();
     return ST_OK;
 }
 

@@ -30,7 +30,7 @@ SYMBOLS = [
     "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
     "pshbm_queue", "pshbm_queue_dev", "pshbm_queue_pairs", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
     "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
-    "pshbm_for_each", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact",
+    "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
@@ -54,6 +54,8 @@ class Config(C.Structure):
         ("max_load_factor", C.c_float),
         ("read_only", C.c_int32),
         ("max_batch", C.c_uint64),
+        ("track_increment", C.c_int32),
+        ("reserved", C.c_int32),
     ]
 
 
@@ -169,6 +171,8 @@ def lib():
         L.pshbm_erase.argtypes = [vp, vp, sz, C.POINTER(C.c_uint64)]
         L.pshbm_erase_dev.argtypes = [vp, vp, sz, C.POINTER(C.c_uint64), vp]
         L.pshbm_compact.argtypes = [vp]
+        L.pshbm_increment_size.argtypes = [vp, C.POINTER(C.c_uint64)]
+        L.pshbm_take_increment.argtypes = [vp, vp, sz, C.POINTER(sz)]
         L.pshbm_clear.argtypes = [vp]
         L.pshbm_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pshbm_memory_usage.argtypes = [vp, C.POINTER(C.c_uint64)]
@@ -208,12 +212,12 @@ class Table:
 
     def __init__(self, dim, optimizer=OPT_SUM, lr=0.0, init_acc=0.0, alpha=0.0, beta=0.0, l1=0.0,
                  l2=0.0, capacity=1 << 20, max_load_factor=0.0, read_only=False, max_batch=0,
-                 device=0):
+                 device=0, track_increment=False):
         self.dim = dim
         self.optimizer = optimizer
         self._h = C.c_void_p()
         cfg = Config(C.sizeof(Config), device, dim, optimizer, lr, init_acc, alpha, beta, l1, l2,
-                     capacity, max_load_factor, int(read_only), max_batch)
+                     capacity, max_load_factor, int(read_only), max_batch, int(track_increment), 0)
         st = lib().pshbm_create(C.byref(cfg), C.byref(self._h))
         if st != OK:
             raise PshbmError(st, (lib().pshbm_last_error(None) or b"").decode())
@@ -290,6 +294,22 @@ class Table:
         got = C.c_size_t()
         st = lib().pshbm_iterate(self._h, offset, batch, rec.ctypes.data, C.byref(got))
         return st, rec[: got.value]
+
+    def increment_size(self):
+        n = C.c_uint64()
+        st = lib().pshbm_increment_size(self._h, C.byref(n))
+        return st, n.value
+
+    def take_increment(self, capacity=None):
+        """(status, records of the keys pushes touched since the last take)."""
+        if capacity is None:
+            st, capacity = self.increment_size()
+            if st != OK:
+                return st, np.empty(0, dtype=record_dtype(self.value_floats))
+        rec = np.empty(max(capacity, 1), dtype=record_dtype(self.value_floats))
+        got = C.c_size_t()
+        st = lib().pshbm_take_increment(self._h, rec.ctypes.data, capacity, C.byref(got))
+        return st, rec[: got.value if st == OK else 0]
 
     def for_each(self, where=None):
         """(status, count, column sums) over the records that satisfy `where` (a Predicate)."""

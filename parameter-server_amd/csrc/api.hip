@@ -374,6 +374,7 @@ void destroy_impl(pshbm_table* t) {
     if (t->d.rows) (void)hipFree(t->d.rows);
     if (t->d.row_keys) (void)hipFree(t->d.row_keys);
     if (t->d.counters) (void)hipFree(t->d.counters);
+    if (t->d.dirty) (void)hipFree(t->d.dirty);
     if (t->d_hist) (void)hipFree(t->d_hist);
     if (t->h_counters) (void)hipHostFree(t->h_counters);
     if (t->h_hist) (void)hipHostFree(t->h_hist);
@@ -541,6 +542,10 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.rows), t->rows_bytes));
     CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.row_keys), t->keys_bytes));
     CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.counters), CNT_WORDS * 4));
+    if (cfg->track_increment) {
+        CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.dirty), round_up(max_rows, 4)));
+        CREATE_TRY(hipMemset(d.dirty, 0, round_up(max_rows, 4)));
+    }
     CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&t->d_hist), 17 * 8));
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_counters), CNT_WORDS * 4, hipHostMallocDefault));
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_hist), 17 * 8, hipHostMallocDefault));
@@ -873,7 +878,10 @@ int32_t pshbm_load(pshbm_table* t, const void* records, size_t n, uint32_t flags
     return PSHBM_OK;
 }
 
-static int32_t dump_range(pshbm_table* t, size_t first, size_t count, void* records) {
+// Records of rows [first, first + count) of the slab, or, with row_list (device), of the rows
+// row_list[first .. first + count), whose marks are cleared on the way.
+static int32_t dump_range(pshbm_table* t, size_t first, size_t count, void* records,
+                          const uint32_t* row_list = nullptr) {
     ST_TRY(ensure_bulk(t));
     const size_t rec = 8 + (size_t)t->d.vf * 4;
     const size_t per_chunk = BULK_CHUNK_BYTES / rec;
@@ -889,8 +897,11 @@ static int32_t dump_range(pshbm_table* t, size_t first, size_t count, void* reco
             HIP_TRY(t, hipEventSynchronize(t->ev_copy[k]));
             std::memcpy(dst + pending_off[k] * rec, t->pin[k], pending_cnt[k] * rec);
         }
-        HIP_TRY(t, launch_pack_records(t->d, (uint32_t)(first + off), cnt,
-                                       static_cast<uint32_t*>(t->dbuf[k]), s));
+        if (row_list)
+            HIP_TRY(t, launch_pack_rows(t->d, row_list + first + off, cnt, static_cast<uint32_t*>(t->dbuf[k]), s));
+        else
+            HIP_TRY(t, launch_pack_records(t->d, (uint32_t)(first + off), cnt,
+                                           static_cast<uint32_t*>(t->dbuf[k]), s));
         HIP_TRY(t, hipEventRecord(t->ev_done[k], s));
         HIP_TRY(t, hipStreamWaitEvent(t->side, t->ev_done[k], 0));
         HIP_TRY(t, hipMemcpyAsync(t->pin[k], t->dbuf[k], cnt * rec, hipMemcpyDeviceToHost, t->side));
@@ -1040,6 +1051,57 @@ int32_t pshbm_compact(pshbm_table* t) {
     return compact_locked(t, s);
 }
 
+// ---- increment -------------------------------------------------------------------------------
+// Marked rows counted (and, with `list`, listed in ms_lists). The lock is held.
+static int32_t increment_scan(pshbm_table* t, hipStream_t s, bool list, uint32_t* marked) {
+    *marked = 0;
+    ST_TRY(ensure_maint(t));
+    ST_TRY(read_counters(t, s));
+    const uint32_t rows = t->h_counters[CNT_ROWS];
+    if (rows == 0) return PSHBM_OK;
+    ST_TRY(ensure(t, t->ms_tiles, (erase_tiles(rows) + 1) * 4));
+    uint32_t* tiles = static_cast<uint32_t*>(t->ms_tiles.p);
+    HIP_TRY(t, launch_erase_count(t->d, rows, t->d.dirty, tiles, t->d_info, s, false));
+    HIP_TRY(t, hipMemcpyAsync(t->h_info, t->d_info, 4 * sizeof(uint32_t), hipMemcpyDeviceToHost, s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    *marked = t->h_info[0];
+    if (list && *marked) {
+        ST_TRY(ensure(t, t->ms_lists, (size_t)*marked * 4));
+        HIP_TRY(t, launch_flag_list(rows, t->d.dirty, tiles, static_cast<uint32_t*>(t->ms_lists.p), s));
+    }
+    return PSHBM_OK;
+}
+
+int32_t pshbm_increment_size(pshbm_table* t, uint64_t* n) {
+    if (!t || !n) return PSHBM_INVALID_ID;
+    *n = 0;
+    if (!t->d.dirty) return fail(t, PSHBM_ERROR, "the table was created without track_increment");
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    ST_TRY(begin_op(t, t->stream));
+    uint32_t marked = 0;
+    ST_TRY(increment_scan(t, t->stream, false, &marked));
+    *n = marked;
+    return PSHBM_OK;
+}
+
+int32_t pshbm_take_increment(pshbm_table* t, void* records, size_t capacity_records, size_t* n_out) {
+    if (!t || !n_out) return PSHBM_INVALID_ID;
+    *n_out = 0;
+    if (!t->d.dirty) return fail(t, PSHBM_ERROR, "the table was created without track_increment");
+    DeviceGuard g(t->device);
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    ST_TRY(begin_op(t, t->stream));
+    uint32_t marked = 0;
+    ST_TRY(increment_scan(t, t->stream, true, &marked));
+    *n_out = marked;
+    if (marked == 0) return PSHBM_OK;
+    if (marked > capacity_records || !records)
+        return fail(t, PSHBM_ERROR, "take_increment: %u records, room for %zu", marked, capacity_records);
+    return dump_range(t, 0, marked, records, static_cast<const uint32_t*>(t->ms_lists.p));
+}
+
 int32_t pshbm_clear(pshbm_table* t) {
     if (!t) return PSHBM_INVALID_ID;
     DeviceGuard g(t->device);
@@ -1048,6 +1110,7 @@ int32_t pshbm_clear(pshbm_table* t) {
     ST_TRY(begin_op(t, s));
     HIP_TRY(t, hipMemsetAsync(t->d.slots, 0xFF, t->slots_bytes, s));
     HIP_TRY(t, hipMemsetAsync(t->d.counters, 0, CNT_WORDS * 4, s));
+    if (t->d.dirty) HIP_TRY(t, hipMemsetAsync(t->d.dirty, 0, round_up(t->d.max_rows, 4), s));
     HIP_TRY(t, hipStreamSynchronize(s));
     t->size_bound = 0;
     t->tombstones = 0;

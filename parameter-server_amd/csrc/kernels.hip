@@ -409,6 +409,7 @@ __device__ __forceinline__ void finalize(const TableDev& t, u32 row, u32 col, u3
     float* ap = reinterpret_cast<float*>(&av);
     float* bp = reinterpret_cast<float*>(&bv);
     opt_step_n<N>(t.opt, gp, wp, ap, bp);
+    if (t.dirty && col == 0) t.dirty[row] = 1;
     r[col] = wv;
     if (kind >= 2) r[units + col] = av;
     if (kind == 3) r[2 * units + col] = bv;
@@ -489,6 +490,7 @@ __device__ __forceinline__ void apply_runs(const TableDev& t, const T* s_val, co
 #pragma unroll
             for (int e = 0; e < N; ++e) opt_step<KIND>(t.opt, gp[e], wp[e], ap[e], bp[e]);
             T* r = rows + (u64)row[k] * stride_units + col;
+            if (t.dirty && col == 0) t.dirty[row[k]] = 1;
             r[0] = wv[k];
             if constexpr (STATES >= 1) r[units] = a0;
             if constexpr (STATES >= 2) r[2 * units] = b0;
@@ -843,6 +845,20 @@ __global__ __launch_bounds__(BLOCK) void pack_records_kernel(TableDev t, u32 fir
     }
 }
 
+__global__ __launch_bounds__(BLOCK) void pack_rows_kernel(TableDev t, const u32* __restrict__ row_list,
+                                                           u64 total, u32* __restrict__ rec, u32 rec_dw,
+                                                           u64 m64) {
+    const u32* rows = reinterpret_cast<const u32*>(t.rows);
+    const u32* rk = reinterpret_cast<const u32*>(t.row_keys);
+    for (u64 q = (u64)blockIdx.x * BLOCK + threadIdx.x; q < total; q += (u64)gridDim.x * BLOCK) {
+        u64 r = div_big(q, m64, rec_dw);
+        u32 off = (u32)(q - r * rec_dw);
+        u64 row = row_list[r];
+        rec[q] = off < 2 ? rk[row * 2 + off] : rows[row * t.stride_f + (off - 2)];
+        if (off == 0 && t.dirty) t.dirty[row] = 0;
+    }
+}
+
 __global__ __launch_bounds__(BLOCK) void unpack_records_kernel(const u32* __restrict__ rec, u64 total,
                                                                 u32 stride_dw, u32 fpr, u32* keys,
                                                                 float* values, u64 m64) {
@@ -1054,6 +1070,15 @@ hipError_t launch_pack_records(const TableDev& t, u32 first_row, size_t n, u32* 
     const u64 total = (u64)n * rec_dw;
     pack_records_kernel<<<grid_for(total, BLOCK * 4, 65536), BLOCK, 0, s>>>(
         t, first_row, total, records, rec_dw, magic64(rec_dw));
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_rows(const TableDev& t, const u32* row_list, size_t n, u32* records, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const u32 rec_dw = t.vf + 2;
+    const u64 total = (u64)n * rec_dw;
+    pack_rows_kernel<<<grid_for(total, BLOCK * 4, 65536), BLOCK, 0, s>>>(t, row_list, total, records, rec_dw,
+                                                                        magic64(rec_dw));
     return hipGetLastError();
 }
 

@@ -141,7 +141,7 @@ __global__ __launch_bounds__(ER_BLOCK) void erase_count_kernel(const uint8_t* __
 // of the table is set to the rows left.
 __global__ __launch_bounds__(ER_BLOCK) void erase_scan_kernel(TableDev t, u32* __restrict__ tile_cnt,
                                                               u32 n_tiles, u32 n_rows,
-                                                              u32* __restrict__ info) {
+                                                              u32* __restrict__ info, int set_row_count) {
     __shared__ u32 wsum[ER_BLOCK / 64];
     __shared__ u32 carry;
     const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(ER_BLOCK) void erase_scan_kernel(TableDev t, u32* _
         info[0] = carry;
         info[1] = n_rows - carry;
         info[2] = 0;  // holes; set by erase_lists_kernel when there are any
-        t.counters[CNT_ROWS] = n_rows - carry;
+        if (set_row_count) t.counters[CNT_ROWS] = n_rows - carry;
     }
 }
 
@@ -215,6 +215,33 @@ __global__ __launch_bounds__(ER_BLOCK) void erase_lists_kernel(const uint8_t* __
     }
 }
 
+// flagged rows, ascending (the prefix of the flags is in tile_off)
+__global__ __launch_bounds__(ER_BLOCK) void flag_list_kernel(const uint8_t* __restrict__ flags, u32 n_rows,
+                                                             const u32* __restrict__ tile_off,
+                                                             u32* __restrict__ list) {
+    __shared__ u32 wsum[ER_BLOCK / 64];
+    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const u64 base = (u64)blockIdx.x * ER_TILE + (u64)tid * ER_ITEMS;
+    u32 d[ER_ITEMS], c = 0;
+#pragma unroll
+    for (u32 j = 0; j < ER_ITEMS; ++j) {
+        d[j] = base + j < n_rows ? flags[base + j] : 0u;
+        c += d[j];
+    }
+    u32 incl = c;
+    for (u32 off = 1; off < 64; off <<= 1) {
+        const u32 o = __shfl_up(incl, off);
+        if (lane >= off) incl += o;
+    }
+    if (lane == 63) wsum[w] = incl;
+    __syncthreads();
+    u32 before = tile_off[blockIdx.x] + incl - c;
+    for (u32 x = 0; x < w; ++x) before += wsum[x];
+#pragma unroll
+    for (u32 j = 0; j < ER_ITEMS; ++j)
+        if (d[j]) list[before++] = (u32)(base + j);
+}
+
 // The slots of the erased keys become markers. 4 lanes per key.
 __global__ __launch_bounds__(BLOCK) void erase_slots_kernel(TableDev t, const u32* __restrict__ dead_list,
                                                              const u32* __restrict__ info) {
@@ -244,7 +271,10 @@ __global__ __launch_bounds__(BLOCK) void erase_move_kernel(TableDev t, const u32
         const u32 c = (u32)(q - j * units);
         const u32 dst = hole_list[j], src = mover_list[j];
         rows[(u64)dst * units + c] = rows[(u64)src * units + c];
-        if (c == 0) t.row_keys[dst] = t.row_keys[src];
+        if (c == 0) {
+            t.row_keys[dst] = t.row_keys[src];
+            if (t.dirty) t.dirty[dst] = t.dirty[src];  // the mark travels with the key
+        }
     }
 }
 
@@ -365,12 +395,19 @@ hipError_t launch_mark_rows(const uint32_t* rows, size_t n, uint32_t n_rows, uin
 size_t erase_tiles(uint32_t n_rows) { return ((size_t)n_rows + ER_TILE - 1) / ER_TILE; }
 
 hipError_t launch_erase_count(const TableDev& t, uint32_t n_rows, const uint8_t* dead, uint32_t* tile_cnt,
-                              uint32_t* info, hipStream_t s) {
+                              uint32_t* info, hipStream_t s, bool set_row_count) {
     const u32 n_tiles = (u32)erase_tiles(n_rows);
     erase_count_kernel<<<n_tiles, ER_BLOCK, 0, s>>>(dead, n_rows, tile_cnt);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    erase_scan_kernel<<<1, ER_BLOCK, 0, s>>>(t, tile_cnt, n_tiles, n_rows, info);
+    erase_scan_kernel<<<1, ER_BLOCK, 0, s>>>(t, tile_cnt, n_tiles, n_rows, info, set_row_count ? 1 : 0);
+    return hipGetLastError();
+}
+
+hipError_t launch_flag_list(uint32_t n_rows, const uint8_t* flags, const uint32_t* tile_off, uint32_t* list,
+                            hipStream_t s) {
+    if (n_rows == 0) return hipSuccess;
+    flag_list_kernel<<<(u32)erase_tiles(n_rows), ER_BLOCK, 0, s>>>(flags, n_rows, tile_off, list);
     return hipGetLastError();
 }
 

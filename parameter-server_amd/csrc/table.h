@@ -45,6 +45,7 @@ struct TableDev {
     float* rows;         // max_rows * stride_f
     uint64_t* row_keys;  // max_rows
     uint32_t* counters;  // CNT_WORDS
+    uint8_t* dirty;      // max_rows bytes, or null: 1 = a push updated the row since the last take
     uint32_t bucket_mask;
     uint32_t max_rows;
     uint32_t dim;       // weights per key
@@ -178,7 +179,13 @@ hipError_t launch_mark_rows(const uint32_t* rows, size_t n, uint32_t n_rows, uin
 // are packed into [0, rows left) and their slots follow them.
 size_t erase_tiles(uint32_t n_rows);
 hipError_t launch_erase_count(const TableDev& t, uint32_t n_rows, const uint8_t* dead, uint32_t* tile_cnt,
-                              uint32_t* info, hipStream_t s);
+                              uint32_t* info, hipStream_t s, bool set_row_count = true);
+// The flagged rows, ascending, after launch_erase_count(..., false): list holds info[0] words.
+hipError_t launch_flag_list(uint32_t n_rows, const uint8_t* flags, const uint32_t* tile_off,
+                            uint32_t* list, hipStream_t s);
+// {key, value} records of the listed rows; clears their dirty marks.
+hipError_t launch_pack_rows(const TableDev& t, const uint32_t* row_list, size_t n, uint32_t* records,
+                            hipStream_t s);
 hipError_t launch_erase_apply(const TableDev& t, uint32_t n_rows, uint32_t erased, const uint8_t* dead,
                               const uint32_t* tile_off, uint32_t* info, uint32_t* lists, hipStream_t s);
 // Every row < n_rows claims a slot for its key in a hash array that the caller has emptied.

@@ -48,6 +48,7 @@ inline pshbm_config table_config(const Configure& c) {
     cfg.max_load_factor = (float)c.number("hbm_table.max_load_factor", 0.0);
     cfg.max_batch = (uint64_t)c.number("hbm_table.max_batch", 0);
     cfg.read_only = (int32_t)c.number("read_only", 0);
+    cfg.track_increment = (int32_t)c.number("hbm_table.track_increment", 0);
     return cfg;
 }
 
