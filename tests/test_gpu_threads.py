@@ -1,0 +1,58 @@
+"""Several host threads on one table: the host-pointer entry points are synchronous and
+thread-safe (pulls share the table, everything else takes it exclusively, the discipline of
+pico-ps/operator/SparsePullOperator.h:188-192 and SparsePushOperator.h:220; the reference's server
+calls the operator halves from 4 + 4 threads, pico-ps/service/Server.h:24-26)."""
+import threading
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_concurrent_pushes_pulls_and_scans(ps, orc, wl):
+    rng = np.random.default_rng(12)
+    dim, n = 8, 20000
+    t = ps.Table(dim, ps.OPT_SUM, capacity=60000)
+    r = orc.Oracle(dim, orc.OPT_SUM, capacity=60000)
+    keys = wl.table_keys_np(0, n, seed=5)
+    vals = rng.integers(-5, 6, (n, dim)).astype(np.float32)
+    assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+    n_threads, rounds = 6, 12
+    work = []
+    for w in range(n_threads):
+        mine = []
+        for it in range(rounds):
+            q = np.concatenate([keys[rng.integers(0, n, 3000)], wl.fresh_keys_np(rng, 40)])
+            g = rng.integers(-3, 4, (q.size, dim)).astype(np.float32)   # integer sums: order-free
+            mine.append((q, g))
+        work.append(mine)
+    errors = []
+
+    def worker(w):
+        try:
+            for q, g in work[w]:
+                assert t.push(q, g) == 0
+                st, rows, hit = t.pull(q[:500])
+                assert st == 0 and hit.all()           # the thread's own pushed keys are there
+                st, cnt, sums = t.for_each()
+                assert st == 0 and cnt >= n
+                if w == 0:
+                    assert t.size() >= n
+        except Exception as e:  # noqa: BLE001 - reported by the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(w,)) for w in range(n_threads)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    for mine in work:                                   # any order gives the same integer sums
+        for q, g in mine:
+            assert r.push(q, g) == 0
+    a = np.sort(t.dump()[1], order="key")
+    b = np.sort(r.dump()[1], order="key")
+    np.testing.assert_array_equal(a["key"], b["key"])
+    np.testing.assert_array_equal(a["value"], b["value"])
+    t.close()
