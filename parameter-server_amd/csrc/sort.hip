@@ -46,12 +46,18 @@ constexpr u32 SPIN_LIMIT = 1u << 24;
 constexpr u32 GROUP = 16;                      // tiles per group of the two-level tile prefix
 constexpr u32 LOOKBACK_TILES = GROUP * GROUP;  // largest input of the one-launch passes, in tiles
 
-// temp layout in 32-bit words: two heads {digit totals [MAX_PASSES][RADIX_MAX], pad} used by
-// alternate sorts -- each sort zeroes the other one for its successor, which saves a fill launch --
-// then rows of RADIX_MAX words: one-launch passes use, per pass, [n_tiles] tile rows and
+constexpr u32 SEGMENTS = 16;  // three-launch passes: the tiles are cut into this many ranges
+
+// temp layout in 32-bit words: two heads {digit totals [MAX_PASSES][SEGMENTS][RADIX_MAX], pad} used
+// by alternate sorts -- each sort zeroes the other one for its successor, which saves a fill
+// launch -- then rows of RADIX_MAX words: one-launch passes use, per pass, [n_tiles] tile rows and
 // [n_groups] group rows; three-launch passes use [n_tiles] rows of counts, reused by every pass.
+// One-launch passes keep their digit totals in segment 0. Three-launch passes keep one set of
+// totals per range of tiles: 16 times fewer atomic additions meet on one word, and the scan of a
+// range needs nothing from the scans of the others.
 constexpr size_t HEAD_TOTALS = 0;
-constexpr size_t HEAD_WORDS = MAX_PASSES * RADIX_MAX + 16;
+constexpr size_t PASS_TOTALS = (size_t)SEGMENTS * RADIX_MAX;  // words of totals per pass
+constexpr size_t HEAD_WORDS = MAX_PASSES * PASS_TOTALS + 16;
 constexpr size_t OFF_ROWS = 2 * HEAD_WORDS;
 
 // The tile's four keys per thread, with the keys that became known only after the caller's
@@ -111,10 +117,10 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(u32* __restrict__
 }
 
 // Three-launch passes, first launch: counts[tile][d] = pairs of the tile whose digit is d, and the
-// digit totals over the whole input.
+// digit totals of every range of tiles_per_seg tiles (totals[segment][d]).
 __global__ __launch_bounds__(SORT_BLOCK) void sort_tile_count_kernel(u32* __restrict__ keys, u32 n,
                                                                       SortLateKeys late, u32 shift,
-                                                                      u32 bits,
+                                                                      u32 bits, u32 tiles_per_seg,
                                                                       u32* __restrict__ totals,
                                                                       u32* __restrict__ counts,
                                                                       u32* __restrict__ next_head) {
@@ -134,7 +140,7 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_tile_count_kernel(u32* __rest
     if (tid < radix) {
         const u32 c = h[tid];
         counts[(size_t)tile * RADIX_MAX + tid] = c;
-        if (c) atomicAdd(&totals[tid], c);
+        if (c) atomicAdd(&totals[(size_t)(tile / tiles_per_seg) * RADIX_MAX + tid], c);
     }
     if (next_head && tile == 0)
         for (u32 x = tid; x < HEAD_WORDS; x += SORT_BLOCK) next_head[x] = 0;
@@ -158,22 +164,36 @@ __device__ __forceinline__ u32 scan_block_exclusive(u32 v, u32 tid, u32* sums) {
 
 // Three-launch passes, second launch: counts[tile][d] becomes the position of the tile's first
 // pair with digit d in the sorted output = (pairs with a smaller digit) + (pairs with digit d in
-// earlier tiles). A workgroup owns 64 digits (lane = digit, so rows are read 256 bytes at a time);
-// its 16 wavefronts split the tiles into 16 consecutive ranges.
+// earlier tiles). Workgroup (x, y) owns 64 digits (lane = digit, so rows are read 256 bytes at a
+// time) of the y-th range of tiles, which its 16 wavefronts split into 16 consecutive parts; what
+// lies before the range comes from the per-range totals.
 __global__ __launch_bounds__(SORT_BLOCK) void sort_scan_kernel(u32* __restrict__ counts,
                                                                 const u32* __restrict__ totals,
-                                                                u32 n_tiles, u32 radix) {
+                                                                u32 n_tiles, u32 tiles_per_seg,
+                                                                u32 radix) {
     __shared__ u32 sums[SORT_WAVES];
     __shared__ u32 dbase[64];
     __shared__ u32 part[SORT_WAVES][64];
     const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
-    const u32 d0 = blockIdx.x * 64u;
-    // pairs with a smaller digit: exclusive scan of the totals (every workgroup repeats it)
-    const u32 base = scan_block_exclusive(tid < radix ? totals[tid] : 0u, tid, sums);
-    if (tid >= d0 && tid < d0 + 64u) dbase[tid - d0] = base;
-    const u32 per = (n_tiles + SORT_WAVES - 1) / SORT_WAVES;
-    const u32 t0 = w * per < n_tiles ? w * per : n_tiles;
-    const u32 t1 = t0 + per < n_tiles ? t0 + per : n_tiles;
+    const u32 d0 = blockIdx.x * 64u, seg = blockIdx.y;
+    // pairs with a smaller digit: exclusive scan of the totals over all ranges (every workgroup
+    // repeats it); pairs with this digit in earlier ranges
+    u32 tot = 0, before = 0;
+    if (tid < radix) {
+#pragma unroll
+        for (u32 x = 0; x < SEGMENTS; ++x) {
+            const u32 v = totals[(size_t)x * RADIX_MAX + tid];
+            tot += v;
+            if (x < seg) before += v;
+        }
+    }
+    const u32 base = scan_block_exclusive(tot, tid, sums);
+    if (tid >= d0 && tid < d0 + 64u) dbase[tid - d0] = base + before;
+    const u32 s0 = seg * tiles_per_seg < n_tiles ? seg * tiles_per_seg : n_tiles;
+    const u32 s1 = s0 + tiles_per_seg < n_tiles ? s0 + tiles_per_seg : n_tiles;
+    const u32 per = (s1 - s0 + SORT_WAVES - 1) / SORT_WAVES;
+    const u32 t0 = s0 + w * per < s1 ? s0 + w * per : s1;
+    const u32 t1 = t0 + per < s1 ? t0 + per : s1;
     u32* col = counts + d0 + lane;
     u32 s = 0;
     for (u32 t = t0; t < t1; t += 8) {
@@ -448,8 +468,9 @@ hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, uint32_t* 
         sort_hist_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys, (u32)n, lk, n_tiles, passes, bits,
                                                         plan->totals, plan->status, next_head);
     else
-        sort_tile_count_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys, (u32)n, lk, 0u, bits, plan->totals,
-                                                              plan->status, next_head);
+        sort_tile_count_kernel<<<n_tiles, SORT_BLOCK, 0, s>>>(keys, (u32)n, lk, 0u, bits,
+                                                              (n_tiles + SEGMENTS - 1) / SEGMENTS,
+                                                              plan->totals, plan->status, next_head);
     return hipGetLastError();
 }
 
@@ -458,23 +479,26 @@ hipError_t sort_pass(const SortPlan& plan, unsigned p, const uint32_t* kin, cons
     if (plan.n == 0) return hipSuccess;
     if (p >= plan.passes) return hipErrorInvalidValue;
     const u32 shift = plan.bits * p;
-    u32* totals = plan.totals + p * RADIX_MAX;
+    u32* totals = plan.totals + p * PASS_TOTALS;
     if (plan.lookback) {
-        u32* totals_next = p + 1 < plan.passes ? plan.totals + (p + 1) * RADIX_MAX : nullptr;
+        u32* totals_next = p + 1 < plan.passes ? plan.totals + (p + 1) * PASS_TOTALS : nullptr;
         u32* status = plan.status + (size_t)p * plan.rows * RADIX_MAX;
         u32* group_status = plan.status + ((size_t)p * plan.rows + plan.n_tiles) * RADIX_MAX;
         return launch_pass<true>(plan.bits, plan.n_tiles, s, kin, vin, kout, vout, plan.n, shift, totals,
                                  totals_next, status, group_status, nullptr, err_flag);
     }
     const SortLateKeys none{0u, nullptr, nullptr};
+    const u32 tiles_per_seg = (plan.n_tiles + SEGMENTS - 1) / SEGMENTS;
     if (p > 0) {  // pass 0 was counted by sort_begin
-        sort_tile_count_kernel<<<plan.n_tiles, SORT_BLOCK, 0, s>>>(
-            const_cast<u32*>(kin), plan.n, none, shift, plan.bits, totals, plan.status, nullptr);
+        sort_tile_count_kernel<<<plan.n_tiles, SORT_BLOCK, 0, s>>>(const_cast<u32*>(kin), plan.n, none,
+                                                                   shift, plan.bits, tiles_per_seg,
+                                                                   totals, plan.status, nullptr);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     const u32 radix = 1u << plan.bits;
-    sort_scan_kernel<<<radix / 64, SORT_BLOCK, 0, s>>>(plan.status, totals, plan.n_tiles, radix);
+    sort_scan_kernel<<<dim3(radix / 64, SEGMENTS), SORT_BLOCK, 0, s>>>(plan.status, totals, plan.n_tiles,
+                                                                       tiles_per_seg, radix);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     return launch_pass<false>(plan.bits, plan.n_tiles, s, kin, vin, kout, vout, plan.n, shift, nullptr,
