@@ -658,6 +658,24 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
                                  r_present ? 1u : 0u);
 }
 
+// Sum of p[x * stride] for x = first, first + step, ... < end, four loads in flight at a time (the
+// order of the additions is fixed by first / end / step alone).
+template <typename T>
+__device__ __forceinline__ T strided_sum(const T* __restrict__ p, u64 first, u64 end, u32 step, u64 stride) {
+    T a0 = vzero(T()), a1 = vzero(T()), a2 = vzero(T()), a3 = vzero(T());
+    u64 x = first;
+    for (; x + 3 * (u64)step < end; x += 4 * (u64)step) {
+        const T v0 = p[x * stride], v1 = p[(x + step) * stride], v2 = p[(x + 2 * (u64)step) * stride],
+                v3 = p[(x + 3 * (u64)step) * stride];
+        a0 = vadd(a0, v0);
+        a1 = vadd(a1, v1);
+        a2 = vadd(a2, v2);
+        a3 = vadd(a3, v3);
+    }
+    for (; x < end; x += step) a0 = vadd(a0, p[x * stride]);
+    return vadd(vadd(a0, a1), vadd(a2, a3));
+}
+
 // A key repeated hundreds of thousands of times in a batch spans thousands of chunks. So that the
 // wavefront that joins its partial sums need not visit every one of them, a first pass looks at
 // windows of 64 chunks: if all 64 chunks of a window lie inside one run (each chunk is a single run
@@ -696,9 +714,7 @@ __global__ __launch_bounds__(BLOCK) void fixup_windows_kernel(const uint4* __res
     const bool lane_on = g < P && c < lp;
     const u32 col = col0 + c;
     T acc = vzero(T());
-    if (lane_on)
-        for (u64 y = (u64)v * WINDOW + g; y < (u64)(v + 1) * WINDOW; y += P)
-            acc = vadd(acc, part_val[(y * 2) * units + col]);
+    if (lane_on) acc = strided_sum(part_val + col, (u64)v * WINDOW + g, (u64)(v + 1) * WINDOW, P, 2 * (u64)units);
     u32 top = 1;
     while (top < P) top <<= 1;
     for (u32 off = top >> 1; off >= 1; off >>= 1) {
@@ -779,11 +795,11 @@ __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* _
     if (lane_on) {
         if (g == 0) acc = part_val[((u64)w * 2 + 1) * units + col];
         if (fs >= fe) {
-            for (u64 x = A + g; x <= B; x += P) acc = vadd(acc, part_val[(x * 2) * units + col]);
+            acc = vadd(acc, strided_sum(part_val + col, A + g, B + 1, P, 2 * (u64)units));
         } else {
-            for (u64 x = A + g; x < fs; x += P) acc = vadd(acc, part_val[(x * 2) * units + col]);
-            for (u64 v = fs / WINDOW + g; v < fe / WINDOW; v += P) acc = vadd(acc, win_val[v * units + col]);
-            for (u64 x = fe + g; x <= B; x += P) acc = vadd(acc, part_val[(x * 2) * units + col]);
+            acc = vadd(acc, strided_sum(part_val + col, A + g, fs, P, 2 * (u64)units));
+            acc = vadd(acc, strided_sum(win_val + col, fs / WINDOW + g, fe / WINDOW, P, (u64)units));
+            acc = vadd(acc, strided_sum(part_val + col, fe + g, B + 1, P, 2 * (u64)units));
         }
     }
     u32 top = 1;
