@@ -3,7 +3,7 @@
 
 A step = one pull of a key batch followed by one push of gradients for the same batch, both
 through the device-pointer C ABI with every input already resident in HBM. The default workload
-is BASELINE.json's configs[1] ("c2": 100M uint64 keys, dim-16 fp32 rows, plain SGD lr 0.01, 1M-key
+is the headline configuration ("c2": 100M uint64 keys, dim-16 fp32 rows, plain SGD lr 0.01, 1M-key
 Zipf(1.05) batches, duplicates summed before the update).
 
 Prints ONE JSON line: metric/value (pulled + pushed keys per second), the roofline of the kernel

@@ -1,4 +1,4 @@
-"""Properties of the HIP path at the full sizes of BASELINE.json's configs (needs an MI355X).
+"""Properties of the HIP path at the full sizes of the benchmark's configurations (needs an MI355X).
 
 At 10^8 keys the CPU oracle is out of reach, so these tests use what the domain fixes without it:
   * stored values are a closed form of the key's index, so any pulled row is known in advance;
