@@ -255,8 +255,11 @@ __global__ __launch_bounds__(BLOCK) void erase_slots_kernel(TableDev t, const u3
         const bool active = i < n;
         const u64 key = active ? t.row_keys[dead_list[i]] : KEY_EMPTY;
         const Found f = probe_find(t, key, active, grp, sub);
-        if (active && sub == 0 && f.slot != SLOT_NONE)
-            t.slots[f.slot] = make_uint4((u32)KEY_DELETED, (u32)(KEY_DELETED >> 32), ROW_NONE, 0u);
+        if (active && sub == 0) {
+            if (f.slot != SLOT_NONE)
+                t.slots[f.slot] = make_uint4((u32)KEY_DELETED, (u32)(KEY_DELETED >> 32), ROW_NONE, 0u);
+            if (t.dirty) t.dirty[dead_list[i]] = 0;  // rows past the row count carry no marks
+        }
     }
 }
 
@@ -273,7 +276,10 @@ __global__ __launch_bounds__(BLOCK) void erase_move_kernel(TableDev t, const u32
         rows[(u64)dst * units + c] = rows[(u64)src * units + c];
         if (c == 0) {
             t.row_keys[dst] = t.row_keys[src];
-            if (t.dirty) t.dirty[dst] = t.dirty[src];  // the mark travels with the key
+            if (t.dirty) {  // the mark travels with the key
+                t.dirty[dst] = t.dirty[src];
+                t.dirty[src] = 0;
+            }
         }
     }
 }

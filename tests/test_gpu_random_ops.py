@@ -1,0 +1,113 @@
+"""Random operation sequences on the HIP path and the oracle side by side (needs an MI355X).
+
+Each case draws a table shape (dim, optimizer) and a sequence of pulls, pushes, queued pushes and
+stores, sets, erases, erase-ifs, for-eachs, dump / load round trips and increment takes, with
+gradients that are small integers (times a power of two for the optimizers with a learning rate)
+so that duplicate sums are exact and every value can be compared bit for bit after every step --
+except under FTRL and Adagrad, whose steps are not exact; those cases push distinct keys only.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+OPTS = [
+    dict(optimizer=0),
+    dict(optimizer=1, lr=0.5),
+    dict(optimizer=2, lr=0.05, init_acc=0.1),
+    dict(optimizer=3, alpha=0.05, beta=1.0, l1=1e-4, l2=1e-5),
+]
+
+
+def _same(t, r):
+    a = np.sort(t.dump()[1], order="key")
+    b = np.sort(r.dump()[1], order="key")
+    np.testing.assert_array_equal(a["key"], b["key"])
+    np.testing.assert_array_equal(a["value"].view(np.uint32), b["value"].view(np.uint32))
+    assert t.size() == r.size()
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_operation_sequences(ps, orc, wl, seed):
+    rng = np.random.default_rng(1000 + seed)
+    dim = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 31, 32, 64, 100, 128, 257]))
+    opt = OPTS[seed % 4]
+    exact_dups = opt["optimizer"] in (0, 1)
+    cap = int(rng.integers(3000, 20000))
+    t = ps.Table(dim, capacity=cap, track_increment=True, **opt)
+    r = orc.Oracle(dim, capacity=cap, track_increment=True, **opt)
+    vf = t.value_floats
+    universe = wl.table_keys_np(0, cap // 2, seed=seed + 50)
+
+    def grads(n):
+        return rng.integers(-4, 5, (n, dim)).astype(np.float32)
+
+    def batch(n):
+        q = universe[rng.integers(0, universe.size, n)]
+        if not exact_dups:
+            q = np.unique(q)
+            rng.shuffle(q)
+        return q
+
+    for step in range(14):
+        op = rng.choice(["push", "push", "push", "queue_store", "set", "pull", "pull_insert", "erase",
+                         "erase_if", "for_each", "dump_load", "increment", "push_no_insert"])
+        n = int(rng.integers(1, 4000))
+        if op in ("push", "push_no_insert"):
+            q = batch(n)
+            g = grads(q.size)
+            flags = ps.PUSH_NO_INSERT if op == "push_no_insert" else 0
+            a, b = t.push(q, g, flags), r.push(q, g, flags)
+            assert a == b, (op, a, b)
+        elif op == "queue_store":
+            for _ in range(int(rng.integers(1, 4))):
+                q = batch(n)
+                if not exact_dups:
+                    break
+                g = grads(q.size)
+                assert t.queue(q, g) == 0 and r.queue(q, g) == 0
+            assert t.store() == r.store()
+        elif op == "set":
+            q = np.unique(universe[rng.integers(0, universe.size, n)])
+            v = rng.integers(-9, 10, (q.size, vf)).astype(np.float32)
+            if opt["optimizer"] >= 2:
+                v[:, dim:] = np.abs(v[:, dim:]) + 1.0       # accumulators stay positive
+            assert t.set(q, v) == r.set(q, v)
+        elif op in ("pull", "pull_insert"):
+            q = universe[rng.integers(0, universe.size, n)]
+            flags = ps.PULL_INSERT_ON_MISS if op == "pull_insert" else 0
+            a, b = t.pull(q, flags), r.pull(q, flags)
+            assert a[0] == b[0]
+            if a[0] == 0:
+                np.testing.assert_array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+                np.testing.assert_array_equal(a[2], b[2])
+        elif op == "erase":
+            q = universe[rng.integers(0, universe.size, n)]
+            assert t.erase(q) == r.erase(q)
+        elif op == "erase_if":
+            m = int(rng.integers(2, 6))
+            terms = [(-1, 6, (m, int(rng.integers(0, m))))]
+            if rng.random() < 0.5:
+                terms.append((int(rng.integers(0, vf)), int(rng.integers(0, 6)), float(rng.integers(-3, 4))))
+            assert t.erase_if(ps.predicate(*terms)) == r.erase_if(orc.predicate(*terms))
+        elif op == "for_each":
+            terms = [(int(rng.integers(0, vf)), int(rng.integers(0, 6)), float(rng.integers(-3, 4)))]
+            a, b = t.for_each(ps.predicate(*terms)), r.for_each(orc.predicate(*terms))
+            assert a[:2] == b[:2]
+            np.testing.assert_allclose(a[2], b[2], rtol=1e-12, atol=1e-9)
+        elif op == "dump_load":
+            st, rec = t.dump()
+            t2 = ps.Table(dim, capacity=cap, track_increment=True, **opt)
+            assert t2.load(rec, ps.LOAD_UNIQUE) == 0
+            t.close()
+            t = t2
+            r.take_increment()                       # a fresh table has no marks
+        elif op == "increment":
+            a, b = t.take_increment(), r.take_increment()
+            assert a[0] == b[0] == 0
+            x, y = np.sort(a[1], order="key"), np.sort(b[1], order="key")
+            np.testing.assert_array_equal(x["key"], y["key"])
+            np.testing.assert_array_equal(x["value"].view(np.uint32), y["value"].view(np.uint32))
+        _same(t, r)
+    t.close()
+    r.close()
