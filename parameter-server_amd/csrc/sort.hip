@@ -112,8 +112,8 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_hist_kernel(u32* __restrict__
         }
     }
     // the totals of the NEXT sort (the other half of the head) start at zero
-    if (tile == 0)
-        for (u32 x = tid; x < HEAD_WORDS; x += SORT_BLOCK) next_head[x] = 0;
+    for (size_t x = (size_t)tile * SORT_BLOCK + tid; x < HEAD_WORDS; x += (size_t)n_tiles * SORT_BLOCK)
+        next_head[x] = 0;
 }
 
 // Three-launch passes, first launch: counts[tile][d] = pairs of the tile whose digit is d, and the
@@ -142,8 +142,9 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_tile_count_kernel(u32* __rest
         counts[(size_t)tile * RADIX_MAX + tid] = c;
         if (c) atomicAdd(&totals[(size_t)(tile / tiles_per_seg) * RADIX_MAX + tid], c);
     }
-    if (next_head && tile == 0)
-        for (u32 x = tid; x < HEAD_WORDS; x += SORT_BLOCK) next_head[x] = 0;
+    if (next_head)  // the totals of the NEXT sort (the other half of the head) start at zero
+        for (size_t x = (size_t)tile * SORT_BLOCK + tid; x < HEAD_WORDS; x += (size_t)gridDim.x * SORT_BLOCK)
+            next_head[x] = 0;
 }
 
 // exclusive scan over the values held by the 1024 threads of the block; all threads must call it
