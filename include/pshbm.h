@@ -227,6 +227,24 @@ typedef struct pshbm_predicate {
 int32_t pshbm_for_each(pshbm_table* t, const pshbm_predicate* where, uint64_t* count,
                        double* column_sums);
 
+/* Writing for-each: replaces SparseTableForEachWriteOperator::apply_request
+ * (ForEachOperator.h:277-359) for hooks that rewrite value columns in place: on every record that
+ * satisfies `where` (NULL = all), columns [first_column, first_column + n_columns) become
+ *   PSHBM_UPD_AFFINE  a * v + b      (decay: b = 0; reset: a = 0)
+ *   PSHBM_UPD_CLAMP   min(max(v, a), b)
+ * in fp32, the product and the sum rounded separately. *count (may be NULL) = records rewritten
+ * (the hook's merged result). Any other hook: pshbm_iterate + pshbm_set on the host. */
+#define PSHBM_UPD_AFFINE 0
+#define PSHBM_UPD_CLAMP 1
+typedef struct pshbm_update {
+    uint32_t struct_size; /* = sizeof(pshbm_update) */
+    int32_t op;           /* PSHBM_UPD_* */
+    uint32_t first_column, n_columns;
+    float a, b;
+} pshbm_update;
+int32_t pshbm_for_each_write(pshbm_table* t, const pshbm_predicate* where, const pshbm_update* what,
+                             uint64_t* count);
+
 /* Erases every record that satisfies `where` (NULL = all, like pshbm_clear): replaces
  * SparseTableEraseIfOperator::apply_request (EraseIfOperator.h:27-55). *erased (may be NULL) =
  * records removed. The rows that remain are packed to the front of the slab, so dump / iterate

@@ -66,6 +66,18 @@ def predicate(*terms):
     return p
 
 
+UPD_AFFINE, UPD_CLAMP = 0, 1
+
+
+class Update(C.Structure):
+    _fields_ = [("struct_size", C.c_uint32), ("op", C.c_int32), ("first_column", C.c_uint32),
+                ("n_columns", C.c_uint32), ("a", C.c_float), ("b", C.c_float)]
+
+
+def update(op, first_column, n_columns, a, b):
+    return Update(C.sizeof(Update), op, first_column, n_columns, a, b)
+
+
 def build():
     """Compiles the oracle with g++ (a few seconds)."""
     subprocess.run(["make", "-C", _HERE, "-B", "libps_oracle.so"], check=True, capture_output=True)
@@ -97,6 +109,7 @@ def lib():
         L.pso_iterate.argtypes = [vp, C.c_size_t, C.c_size_t, vp, C.POINTER(C.c_size_t)]
         L.pso_dump.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_size_t)]
         L.pso_for_each.argtypes = [vp, vp, C.POINTER(C.c_uint64), vp]
+        L.pso_for_each_write.argtypes = [vp, vp, vp, C.POINTER(C.c_uint64)]
         L.pso_erase_if.argtypes = [vp, vp, C.POINTER(C.c_uint64)]
         L.pso_erase.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_uint64)]
         L.pso_increment_size.argtypes = [vp, C.POINTER(C.c_uint64)]
@@ -217,6 +230,12 @@ class Oracle:
         st = lib().pso_for_each(self._h, C.byref(where) if where is not None else None, C.byref(n),
                                 sums.ctypes.data)
         return st, n.value, sums
+
+    def for_each_write(self, what, where=None):
+        n = C.c_uint64()
+        st = lib().pso_for_each_write(self._h, C.byref(where) if where is not None else None,
+                                      C.byref(what), C.byref(n))
+        return st, n.value
 
     def erase_if(self, where=None):
         n = C.c_uint64()

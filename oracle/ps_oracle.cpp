@@ -481,6 +481,39 @@ int32_t pso_for_each(void* h, const pso_predicate* where, uint64_t* count, doubl
     return ST_OK;
 }
 
+// SparseTableForEachWriteOperator::apply_request, ForEachOperator.h:277-359, with the hook "rewrite
+// columns [first, first + n) of the value": op 0: a * v + b (two roundings), op 1: clamp to [a, b].
+// The predicate sees the value before the rewrite. *count = records rewritten.
+struct pso_update {
+    uint32_t struct_size;
+    int32_t op;
+    uint32_t first_column, n_columns;
+    float a, b;
+};
+int32_t pso_for_each_write(void* h, const pso_predicate* where, const pso_update* what, uint64_t* count) {
+    Oracle& o = *static_cast<Oracle*>(h);
+    if (o.c.read_only) return ST_ERROR;
+    if (!what || (uint64_t)what->first_column + what->n_columns > o.vf || what->op < 0 || what->op > 1)
+        return ST_INVALID_CONFIG;
+    uint64_t n = 0;
+    for (size_t r = 0; r < o.row_keys.size(); ++r) {
+        float* v = &o.rows[r * o.vf];
+        if (!holds(where, o.row_keys[r], v)) continue;
+        ++n;
+        for (uint32_t c = what->first_column; c < what->first_column + what->n_columns; ++c) {
+            if (what->op == 0) {
+                const float p = what->a * v[c];
+                v[c] = p + what->b;
+            } else {
+                v[c] = std::fmin(std::fmax(v[c], what->a), what->b);
+            }
+        }
+        if (o.c.track_increment) o.touched.insert(o.row_keys[r]);
+    }
+    if (count) *count = n;
+    return ST_OK;
+}
+
 // SparseTableEraseIfOperator::apply_request, EraseIfOperator.h:38-47.
 int32_t pso_erase_if(void* h, const pso_predicate* where, uint64_t* erased) {
     Oracle& o = *static_cast<Oracle*>(h);

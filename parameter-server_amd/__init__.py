@@ -30,7 +30,7 @@ SYMBOLS = [
     "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
     "pshbm_queue", "pshbm_queue_dev", "pshbm_queue_pairs", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
     "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
-    "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact",
+    "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
@@ -104,6 +104,19 @@ def predicate(*terms):
     return p
 
 
+UPD_AFFINE, UPD_CLAMP = 0, 1
+
+
+class Update(C.Structure):
+    """pshbm_update: what a writing for-each does to columns [first_column, first_column + n_columns)."""
+    _fields_ = [("struct_size", C.c_uint32), ("op", C.c_int32), ("first_column", C.c_uint32),
+                ("n_columns", C.c_uint32), ("a", C.c_float), ("b", C.c_float)]
+
+
+def update(op, first_column, n_columns, a, b):
+    return Update(C.sizeof(Update), op, first_column, n_columns, a, b)
+
+
 class Profile(C.Structure):
     _fields_ = [("ms", C.c_double * 12), ("launches", C.c_uint64 * 12)]
 
@@ -167,6 +180,7 @@ def lib():
         L.pshbm_dump.argtypes = [vp, vp, sz, C.POINTER(sz)]
         L.pshbm_iterate.argtypes = [vp, sz, sz, vp, C.POINTER(sz)]
         L.pshbm_for_each.argtypes = [vp, vp, C.POINTER(C.c_uint64), vp]
+        L.pshbm_for_each_write.argtypes = [vp, vp, vp, C.POINTER(C.c_uint64)]
         L.pshbm_erase_if.argtypes = [vp, vp, C.POINTER(C.c_uint64)]
         L.pshbm_erase.argtypes = [vp, vp, sz, C.POINTER(C.c_uint64)]
         L.pshbm_erase_dev.argtypes = [vp, vp, sz, C.POINTER(C.c_uint64), vp]
@@ -318,6 +332,13 @@ class Table:
         st = lib().pshbm_for_each(self._h, C.byref(where) if where is not None else None, C.byref(n),
                                   sums.ctypes.data)
         return st, n.value, sums
+
+    def for_each_write(self, what, where=None):
+        """(status, records rewritten): columns rewritten by `what` (an Update) where `where` holds."""
+        n = C.c_uint64()
+        st = lib().pshbm_for_each_write(self._h, C.byref(where) if where is not None else None,
+                                        C.byref(what), C.byref(n))
+        return st, n.value
 
     def erase_if(self, where=None):
         n = C.c_uint64()

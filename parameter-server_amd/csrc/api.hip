@@ -983,6 +983,37 @@ int32_t pshbm_for_each(pshbm_table* t, const pshbm_predicate* where, uint64_t* c
     return PSHBM_OK;
 }
 
+int32_t pshbm_for_each_write(pshbm_table* t, const pshbm_predicate* where, const pshbm_update* what,
+                             uint64_t* count) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (count) *count = 0;
+    if (t->cfg.read_only) return fail(t, PSHBM_ERROR, "for_each_write: the table is read-only");
+    if (!what || what->struct_size != sizeof(pshbm_update))
+        return fail(t, PSHBM_INVALID_CONFIG, "for_each_write: update struct_size");
+    if (what->op != PSHBM_UPD_AFFINE && what->op != PSHBM_UPD_CLAMP)
+        return fail(t, PSHBM_INVALID_CONFIG, "for_each_write: no such operation");
+    if ((uint64_t)what->first_column + what->n_columns > t->d.vf)
+        return fail(t, PSHBM_INVALID_CONFIG, "for_each_write: columns %u..%u of %u", what->first_column,
+                    what->first_column + what->n_columns, t->d.vf);
+    pshbm_predicate pred;
+    ST_TRY(check_predicate(t, where, &pred));
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    hipStream_t s = t->stream;
+    ST_TRY(begin_op(t, s));
+    ST_TRY(ensure_maint(t));
+    ST_TRY(read_counters(t, s));
+    const uint32_t rows = t->h_counters[CNT_ROWS];
+    if (rows == 0) return PSHBM_OK;
+    ST_TRY(ensure(t, t->ms_fe, for_each_scratch_bytes(t->d)));
+    double* scratch = static_cast<double*>(t->ms_fe.p);
+    HIP_TRY(t, launch_for_each_write(t->d, rows, pred, *what, scratch, s));
+    HIP_TRY(t, hipMemcpyAsync(t->h_fe, scratch, sizeof(double), hipMemcpyDeviceToHost, s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    if (count) *count = (uint64_t)t->h_fe[0];
+    return PSHBM_OK;
+}
+
 int32_t pshbm_erase_if(pshbm_table* t, const pshbm_predicate* where, uint64_t* erased) {
     if (!t) return PSHBM_INVALID_ID;
     if (t->cfg.read_only) return fail(t, PSHBM_ERROR, "erase_if: the table is read-only");

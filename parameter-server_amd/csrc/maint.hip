@@ -99,6 +99,46 @@ __global__ __launch_bounds__(BLOCK) void for_each_final_kernel(const double* __r
     out[c] = s;
 }
 
+// Writing for-each: thread per row; the predicate is evaluated on the row as it is before the
+// rewrite. counts: one partial per workgroup, added up in workgroup order afterwards.
+__global__ __launch_bounds__(BLOCK) void for_each_write_kernel(TableDev t, u32 n_rows, pshbm_predicate pred,
+                                                                pshbm_update what,
+                                                                double* __restrict__ partial) {
+    __shared__ u32 wsum[BLOCK / 64];
+    u32 mine = 0;
+    for (u64 r = (u64)blockIdx.x * BLOCK + threadIdx.x; r < n_rows; r += (u64)gridDim.x * BLOCK) {
+        float* row = t.rows + r * t.stride_f;
+        if (!eval_pred(pred, t.row_keys[r], row)) continue;
+        ++mine;
+        for (u32 c = what.first_column; c < what.first_column + what.n_columns; ++c) {
+            const float v = row[c];
+            float out;
+            if (what.op == PSHBM_UPD_AFFINE) {
+                const float p = what.a * v;
+                out = p + what.b;
+            } else {
+                out = fminf(fmaxf(v, what.a), what.b);
+            }
+            row[c] = out;
+        }
+        if (t.dirty) t.dirty[r] = 1;
+    }
+    for (u32 off = 32; off >= 1; off >>= 1) mine += __shfl_down(mine, off);
+    if ((threadIdx.x & 63u) == 0) wsum[threadIdx.x >> 6] = mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        u32 s = 0;
+        for (u32 x = 0; x < BLOCK / 64; ++x) s += wsum[x];
+        partial[blockIdx.x] = (double)s;
+    }
+}
+
+__global__ void sum_partials_kernel(const double* __restrict__ partial, u32 n, double* __restrict__ out) {
+    double s = 0.0;
+    for (u32 b = 0; b < n; ++b) s += partial[b];
+    out[0] = s;
+}
+
 // ---- erase ---------------------------------------------------------------------------------
 __global__ __launch_bounds__(BLOCK) void mark_pred_kernel(TableDev t, u32 n_rows, pshbm_predicate pred,
                                                            uint8_t* __restrict__ dead) {
@@ -381,6 +421,17 @@ hipError_t launch_for_each(const TableDev& t, uint32_t n_rows, const pshbm_predi
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     for_each_final_kernel<<<(t.vf + 1 + BLOCK - 1) / BLOCK, BLOCK, 0, s>>>(partial, n_blocks, t.vf, scratch);
+    return hipGetLastError();
+}
+
+hipError_t launch_for_each_write(const TableDev& t, uint32_t n_rows, const pshbm_predicate& pred,
+                                 const pshbm_update& what, double* scratch, hipStream_t s) {
+    const u32 n_blocks = blocks_for(n_rows, BLOCK * 4, FE_BLOCKS_MAX);
+    double* partial = scratch + (t.vf + 1);
+    for_each_write_kernel<<<n_blocks, BLOCK, 0, s>>>(t, n_rows, pred, what, partial);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    sum_partials_kernel<<<1, 1, 0, s>>>(partial, n_blocks, scratch);
     return hipGetLastError();
 }
 

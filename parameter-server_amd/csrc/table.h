@@ -167,6 +167,10 @@ hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long l
 size_t for_each_scratch_bytes(const TableDev& t);
 hipError_t launch_for_each(const TableDev& t, uint32_t n_rows, const ::pshbm_predicate& pred,
                            double* scratch, hipStream_t s);
+// Rewrites columns of the rows that satisfy `pred` (see pshbm_update); scratch as for
+// launch_for_each, the count of rewritten rows is left in its first double.
+hipError_t launch_for_each_write(const TableDev& t, uint32_t n_rows, const ::pshbm_predicate& pred,
+                                 const ::pshbm_update& what, double* scratch, hipStream_t s);
 // dead[r] = 1 where row r satisfies `pred`, else 0 / dead[rows[i]] = 1 for every rows[i] < n_rows.
 hipError_t launch_mark_pred(const TableDev& t, uint32_t n_rows, const ::pshbm_predicate& pred,
                             uint8_t* dead, hipStream_t s);

@@ -51,7 +51,8 @@ def test_random_operation_sequences(ps, orc, wl, seed):
 
     for step in range(14):
         op = rng.choice(["push", "push", "push", "queue_store", "set", "pull", "pull_insert", "erase",
-                         "erase_if", "for_each", "dump_load", "increment", "push_no_insert"])
+                         "erase_if", "for_each", "for_each_write", "dump_load", "increment",
+                         "push_no_insert"])
         n = int(rng.integers(1, 4000))
         if op in ("push", "push_no_insert"):
             q = batch(n)
@@ -95,6 +96,18 @@ def test_random_operation_sequences(ps, orc, wl, seed):
             a, b = t.for_each(ps.predicate(*terms)), r.for_each(orc.predicate(*terms))
             assert a[:2] == b[:2]
             np.testing.assert_allclose(a[2], b[2], rtol=1e-12, atol=1e-9)
+        elif op == "for_each_write":
+            c0 = int(rng.integers(0, vf))
+            nc = int(rng.integers(0, vf - c0 + 1))
+            kind = int(rng.integers(0, 2))
+            a, b2 = (float(rng.choice([0.0, 0.5, 2.0, -1.0])), float(rng.integers(-2, 3))) if kind == 0 \
+                else (-2.0, 3.0)
+            if opt["optimizer"] >= 2 and c0 + nc > dim:
+                a, b2, kind = 1.0, 1.0, 0               # accumulators stay positive
+            terms = [(-1, 6, (3, int(rng.integers(0, 3))))]
+            x = t.for_each_write(ps.update(kind, c0, nc, a, b2), ps.predicate(*terms))
+            y = r.for_each_write(orc.update(kind, c0, nc, a, b2), orc.predicate(*terms))
+            assert x == y and x[0] == 0
         elif op == "dump_load":
             st, rec = t.dump()
             t2 = ps.Table(dim, capacity=cap, track_increment=True, **opt)
