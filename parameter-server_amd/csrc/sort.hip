@@ -427,13 +427,13 @@ hipError_t launch_pass(u32 bits, u32 n_tiles, hipStream_t s, const u32* kin, con
 
 }  // namespace
 
+// Grows with n, so that a workspace sized for the largest batch serves every smaller one: the
+// one-launch scheme of a batch of up to 2^20 pairs can need more rows than the counts of a larger one.
 size_t sort_pairs_temp_bytes(size_t n) {
     const size_t n_tiles = tiles_of(n);
-    size_t rows;
-    if (n_tiles <= LOOKBACK_TILES)
-        rows = MAX_PASSES * ((n_tiles ? n_tiles : 1) + (n_tiles + GROUP - 1) / GROUP + 1);
-    else
-        rows = n_tiles;
+    const size_t lb_tiles = n_tiles < LOOKBACK_TILES ? (n_tiles ? n_tiles : 1) : LOOKBACK_TILES;
+    const size_t lb_rows = MAX_PASSES * (lb_tiles + (lb_tiles + GROUP - 1) / GROUP + 1);
+    const size_t rows = n_tiles > lb_rows ? n_tiles : lb_rows;
     return (OFF_ROWS + rows * RADIX_MAX) * 4;
 }
 

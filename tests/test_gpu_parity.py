@@ -170,6 +170,10 @@ def test_aggregation_exact_large_batch(ps, orc, n):
     assert t.push(keys2, g2, ps.PUSH_NO_INSERT) == 0
     assert r.push(keys2, g2, orc.PUSH_NO_INSERT) == 0
     assert_same_table(t, r, exact=True)
+    # smaller batches on the workspace of the large one: both sort schemes, and a tiny batch
+    for m in (1 << 20, 300_000, 77):
+        assert t.push(keys[:m], g[:m]) == 0 and r.push(keys[:m], g[:m]) == 0
+    assert_same_table(t, r, exact=True)
     t.close()
 
 
