@@ -293,12 +293,12 @@ int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out);
  * SparsePushOperator.h:202,328). Costs two event records per launch; leave it off in production. */
 #define PSHBM_PHASE_PULL 0          /* fused probe + gather of a pull */
 #define PSHBM_PHASE_LOCATE 1        /* probe (+ claim) of a push, a set or an inserting pull */
-#define PSHBM_PHASE_SORT_HIST 2     /* radix sort of (slot, index): digit histogram */
+#define PSHBM_PHASE_SORT_HIST 2     /* radix sort of (row, index): digit histogram */
 #define PSHBM_PHASE_SEGREDUCE 3     /* duplicate aggregation + update inside wave chunks */
 #define PSHBM_PHASE_FIXUP 4         /* runs that cross chunk borders */
 #define PSHBM_PHASE_UPDATE_UNIQUE 5 /* update of a batch declared duplicate-free */
 #define PSHBM_PHASE_GATHER 6        /* row gather of an inserting pull */
-#define PSHBM_PHASE_SORT_PASS 7     /* radix sort of (slot, index): one 8-bit digit pass */
+#define PSHBM_PHASE_SORT_PASS 7     /* radix sort of (row, index): one digit pass */
 #define PSHBM_PHASE_FIXUP_WINDOWS 8 /* window sums of runs that span many chunks */
 #define PSHBM_PHASE_ASSIGN_ROWS 9   /* rows for the slots an inserting operation claimed */
 #define PSHBM_PHASES 12

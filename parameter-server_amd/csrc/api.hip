@@ -35,7 +35,6 @@ struct pshbm_table {
     TableDev d{};
     int device = 0;
     uint64_t nbuckets = 0;
-    uint32_t slot_bits = 0;
     uint32_t row_bits = 0;  // row ids and ROW_NONE differ in their low row_bits bits
     size_t slots_bytes = 0, rows_bytes = 0, keys_bytes = 0;
 
@@ -511,8 +510,6 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
         return bad("table needs more than 2^31 slots");
     }
     t->nbuckets = nb;
-    t->slot_bits = 0;
-    while ((1ull << t->slot_bits) < nb * 4) ++t->slot_bits;
     t->row_bits = 1;
     while ((1ull << t->row_bits) <= max_rows) ++t->row_bits;
 

@@ -415,19 +415,19 @@ __device__ __forceinline__ void finalize(const TableDev& t, u32 row, u32 col, u3
     if (kind == 3) r[2 * units + col] = bv;
 }
 
-// ---- duplicate aggregation + update over slot-sorted pairs -------------------------------------
-// Each wavefront owns `wch` consecutive sorted positions (a chunk). It copies the chunk's slots
+// ---- duplicate aggregation + update over row-sorted pairs --------------------------------------
+// Each wavefront owns `wch` consecutive sorted positions (a chunk). It copies the chunk's row ids
 // and the gradient rows they point to into LDS (16 independent row loads per lane in flight),
-// lists the starts of the runs of equal slots with ballots, and then gives each run to one group
+// lists the starts of the runs of equal row ids with ballots, and then gives each run to one group
 // of `lp` lanes, which adds the run's rows in sorted order, one LDS read per row. A run longer
 // than 2 P rows is added by all P groups together (strided, then a shuffle tree). A run that
 // begins and ends inside the chunk is complete: its sum is applied to the table row, four runs
 // per lane group at a time so that the row loads of different runs overlap. A run that crosses a
 // chunk border leaves a partial sum in part_val (entry 0: the run that entered from the left,
 // entry 1: the run that leaves to the right) for fixup_kernel to join.
-// part_hdr[w] = {slot of entry 0, flags of entry 0 (1 present, 2 run ends in this chunk),
-//               slot of entry 1, flags of entry 1 (1 present)}.
-// LDS per wavefront: wch * lp_full elements of T, then three arrays of wch + 1 words (slots;
+// part_hdr[w] = {row of entry 0, flags of entry 0 (1 present, 2 run ends in this chunk),
+//               row of entry 1, flags of entry 1 (1 present)}.
+// LDS per wavefront: wch * lp_full elements of T, then three arrays of wch + 1 words (row ids;
 // batch indices, later one action word per run; run starts).
 constexpr int SEG_BLOCK = 128;  // 2 wavefronts
 
@@ -500,7 +500,7 @@ __device__ __forceinline__ void apply_runs(const TableDev& t, const T* s_val, co
 
 template <typename T>
 __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
-    TableDev t, const u32* __restrict__ sslot, const u32* __restrict__ sidx, u32 n,
+    TableDev t, const u32* __restrict__ srow, const u32* __restrict__ sidx, u32 n,
     const T* __restrict__ grads, uint4* __restrict__ part_hdr, T* __restrict__ part_val, u32 units,
     u32 lp_full, u32 P, u32 wch, u32 n_chunks, u32 val_bytes, u32 arr_bytes) {
     extern __shared__ uint4 seg_lds[];
@@ -510,7 +510,7 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
     if (w >= n_chunks) return;  // no workgroup barriers below
     char* base = reinterpret_cast<char*>(seg_lds) + (size_t)wv * (val_bytes + 3 * arr_bytes);
     T* s_val = reinterpret_cast<T*>(base);
-    u32* s_slot = reinterpret_cast<u32*>(base + val_bytes);
+    u32* s_row = reinterpret_cast<u32*>(base + val_bytes);
     u32* s_aux = reinterpret_cast<u32*>(base + val_bytes + arr_bytes);
     u32* s_start = reinterpret_cast<u32*>(base + val_bytes + 2 * arr_bytes);
 
@@ -522,20 +522,20 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
     const u32 cs = w * wch;
     const u32 cnt = (n - cs) < wch ? (n - cs) : wch;
 
-    // slots and batch indices of the chunk
+    // row ids and batch indices of the chunk
     for (u32 pl = lane; pl < wch; pl += 64) {
         u32 sl = SLOT_NONE, ix = 0;
         if (pl < cnt) {
-            sl = sslot[cs + pl];
+            sl = srow[cs + pl];
             ix = sidx[cs + pl];
         }
-        s_slot[pl] = sl;
+        s_row[pl] = sl;
         s_aux[pl] = ix;
     }
-    const u32 first_slot = sslot[cs];
-    const u32 last_slot = sslot[cs + cnt - 1];
-    const bool open_left = cs > 0 && sslot[cs - 1] == first_slot;
-    const u32 after = cs + cnt < n ? sslot[cs + cnt] : SLOT_NONE;
+    const u32 first_row = srow[cs];
+    const u32 last_row = srow[cs + cnt - 1];
+    const bool open_left = cs > 0 && srow[cs - 1] == first_row;
+    const u32 after = cs + cnt < n ? srow[cs + cnt] : SLOT_NONE;
     wave_sync();
 
     // gradient rows into LDS: position r * P + g in round r
@@ -545,7 +545,7 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
         for (u32 r = 0; r < SEG_ROUNDS; ++r) {
             const u32 pl = r * P + g;
             v[r] = vzero(T());
-            if (lane_on && pl < cnt && s_slot[pl] != SLOT_NONE)
+            if (lane_on && pl < cnt && s_row[pl] != SLOT_NONE)
                 v[r] = grads[(u64)s_aux[pl] * units + col0 + c];
         }
 #pragma unroll
@@ -562,8 +562,8 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
         const u32 pl = k0 + lane;
         u32 sl = SLOT_NONE, pv = SLOT_NONE;
         if (pl < wch) {
-            sl = s_slot[pl];
-            if (pl > 0) pv = s_slot[pl - 1];
+            sl = s_row[pl];
+            if (pl > 0) pv = s_row[pl - 1];
         }
         const bool real = sl != SLOT_NONE;
         const bool head = real && (pl == 0 || pv != sl);
@@ -579,7 +579,7 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
     // run's action word becomes 1; a sum that crosses a border goes to part_val.
     bool my_l = false, my_le = false, my_r = false;
     auto classify = [&](u32 j, u32 st, u32 en, T acc) {
-        const u32 sl = s_slot[st];
+        const u32 sl = s_row[st];
         const bool first_run = open_left && j == 0;
         const bool last_open = en == cnt && after == sl;
         u32 act = 0;
@@ -635,26 +635,26 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
     const u32 col = col0 + c;
     switch (t.opt.kind) {
         case 0:
-            apply_runs<T, 0, SEG_ROUNDS>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+            apply_runs<T, 0, SEG_ROUNDS>(t, s_val, s_row, s_aux, s_start, nruns, P, g, c, lane_on,
                                          lp_full, units, col);
             break;
         case 1:
-            apply_runs<T, 1, SEG_ROUNDS>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+            apply_runs<T, 1, SEG_ROUNDS>(t, s_val, s_row, s_aux, s_start, nruns, P, g, c, lane_on,
                                          lp_full, units, col);
             break;
         case 2:
-            apply_runs<T, 2, SEG_ROUNDS / 2>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+            apply_runs<T, 2, SEG_ROUNDS / 2>(t, s_val, s_row, s_aux, s_start, nruns, P, g, c, lane_on,
                                              lp_full, units, col);
             break;
         default:
-            apply_runs<T, 3, SEG_ROUNDS / 4>(t, s_val, s_slot, s_aux, s_start, nruns, P, g, c, lane_on,
+            apply_runs<T, 3, SEG_ROUNDS / 4>(t, s_val, s_row, s_aux, s_start, nruns, P, g, c, lane_on,
                                              lp_full, units, col);
             break;
     }
 
     const bool l_present = __any(my_l) != 0, l_ends = __any(my_le) != 0, r_present = __any(my_r) != 0;
     if (lane == 0 && blockIdx.y == 0)
-        part_hdr[w] = make_uint4(first_slot, (l_present ? 1u : 0u) | (l_ends ? 2u : 0u), last_slot,
+        part_hdr[w] = make_uint4(first_row, (l_present ? 1u : 0u) | (l_ends ? 2u : 0u), last_row,
                                  r_present ? 1u : 0u);
 }
 
@@ -680,13 +680,13 @@ __device__ __forceinline__ T strided_sum(const T* __restrict__ p, u64 first, u64
 // wavefront that joins its partial sums need not visit every one of them, a first pass looks at
 // windows of 64 chunks: if all 64 chunks of a window lie inside one run (each chunk is a single run
 // that is open on both sides), their partial sums are added up into win_val[window] and
-// win_slot[window] names the run's slot; any other window gets SLOT_NONE.
+// win_row[window] names the run's row; any other window gets SLOT_NONE.
 constexpr u32 WINDOW = 64;
 
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void fixup_windows_kernel(const uint4* __restrict__ part_hdr,
                                                                const T* __restrict__ part_val,
-                                                               u32* __restrict__ win_slot,
+                                                               u32* __restrict__ win_row,
                                                                T* __restrict__ win_val, u32 units,
                                                                u32 lp_full, u32 P, u32 n_chunks,
                                                                u32 n_windows) {
@@ -704,7 +704,7 @@ __global__ __launch_bounds__(BLOCK) void fixup_windows_kernel(const uint4* __res
     const u32 s0 = __shfl(sl, 0);
     const bool whole = __ballot(through && sl == s0) == ~0ull;
     if (!whole) {
-        if (lane == 0 && blockIdx.y == 0) win_slot[v] = SLOT_NONE;
+        if (lane == 0 && blockIdx.y == 0) win_row[v] = SLOT_NONE;
         return;
     }
     const u32 col0 = blockIdx.y * 64u;
@@ -722,20 +722,20 @@ __global__ __launch_bounds__(BLOCK) void fixup_windows_kernel(const uint4* __res
         if (g + off < P) acc = vadd(acc, o);
     }
     if (lane_on && g == 0) win_val[(u64)v * units + col] = acc;
-    if (lane == 0 && blockIdx.y == 0) win_slot[v] = s0;
+    if (lane == 0 && blockIdx.y == 0) win_row[v] = s0;
 }
 
 // Joins the partial sums of runs that cross chunk borders. One wavefront per chunk: if a run
 // leaves that chunk to the right, the wavefront finds where the run ends (the first following
 // chunk whose left entry is marked as the run's end; whole windows of the run are skipped through
-// win_slot), its P lane groups add, in a strided fashion, the left entries of the chunks in
+// win_row), its P lane groups add, in a strided fashion, the left entries of the chunks in
 // between -- window sums where a window lies wholly inside the run --, a shuffle tree joins the P
 // sums, and group 0 applies the step. The order of the additions depends only on the chunk
 // layout, so results repeat from run to run.
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* __restrict__ part_hdr,
                                                        const T* __restrict__ part_val,
-                                                       const u32* __restrict__ win_slot,
+                                                       const u32* __restrict__ win_row,
                                                        const T* __restrict__ win_val, u32 units,
                                                        u32 lp_full, u32 P, u32 n_chunks, u32 n_windows) {
     const u32 lane = threadIdx.x & 63u;
@@ -777,7 +777,7 @@ __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* _
         // whole windows of this run, 64 window words per step
         while (x0 < n_chunks) {
             const u32 vv = x0 / WINDOW + lane;
-            const bool mine = vv < n_windows && win_slot[vv] == h.z;
+            const bool mine = vv < n_windows && win_row[vv] == h.z;
             const u64 nm = ~__ballot(mine);
             const u32 k = nm ? (u32)__ffsll((unsigned long long)nm) - 1u : 64u;
             if (k) {
@@ -813,7 +813,7 @@ __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* _
 
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void update_unique_kernel(TableDev t,
-                                                               const u32* __restrict__ slot_idx,
+                                                               const u32* __restrict__ row_idx,
                                                                u32 n, const T* __restrict__ grads,
                                                                u32 units, u32 lp_full, u32 P) {
     const u32 lane = threadIdx.x & 63u;
@@ -825,7 +825,7 @@ __global__ __launch_bounds__(BLOCK) void update_unique_kernel(TableDev t,
     const u64 wave = ((u64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
     const u64 nwaves = ((u64)gridDim.x * BLOCK) >> 6;
     for (u64 i = wave * P + g; i < n; i += nwaves * P) {
-        u32 s = slot_idx[i];
+        u32 s = row_idx[i];
         if (s == SLOT_NONE) continue;
         T gv = grads[i * units + col0 + c];
         finalize<T>(t, s, col0 + c, units, gv);
@@ -999,7 +999,7 @@ hipError_t launch_rollback(const TableDev& t, const u32* slot_idx, size_t n, u32
     return hipGetLastError();
 }
 
-hipError_t launch_segreduce(const TableDev& t, const u32* sorted_slot, const u32* sorted_idx, size_t n,
+hipError_t launch_segreduce(const TableDev& t, const u32* sorted_row, const u32* sorted_idx, size_t n,
                             const float* grads, uint4* part_hdr, float* part_val, hipStream_t s) {
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads, part_val);
@@ -1010,18 +1010,18 @@ hipError_t launch_segreduce(const TableDev& t, const u32* sorted_slot, const u32
     dim3 grid((g.n_chunks + SEG_BLOCK / 64 - 1) / (SEG_BLOCK / 64), g.col_blocks);
     if (v4)
         segreduce_kernel<float4><<<grid, SEG_BLOCK, lds, s>>>(
-            t, sorted_slot, sorted_idx, (u32)n, reinterpret_cast<const float4*>(grads), part_hdr,
+            t, sorted_row, sorted_idx, (u32)n, reinterpret_cast<const float4*>(grads), part_hdr,
             reinterpret_cast<float4*>(part_val), g.units, g.lp, g.p, g.wch, g.n_chunks, val_bytes,
             arr_bytes);
     else
-        segreduce_kernel<float><<<grid, SEG_BLOCK, lds, s>>>(t, sorted_slot, sorted_idx, (u32)n, grads,
+        segreduce_kernel<float><<<grid, SEG_BLOCK, lds, s>>>(t, sorted_row, sorted_idx, (u32)n, grads,
                                                              part_hdr, part_val, g.units, g.lp, g.p,
                                                              g.wch, g.n_chunks, val_bytes, arr_bytes);
     return hipGetLastError();
 }
 
 hipError_t launch_fixup_windows(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
-                                const float* part_val, u32* win_slot, float* win_val, hipStream_t s) {
+                                const float* part_val, u32* win_row, float* win_val, hipStream_t s) {
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads, part_val) && vec4_ok(t, win_val);  // the layout launch_segreduce chose
     const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
@@ -1029,16 +1029,16 @@ hipError_t launch_fixup_windows(const TableDev& t, size_t n, const float* grads,
     dim3 grid((n_windows + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per window
     if (v4)
         fixup_windows_kernel<float4><<<grid, BLOCK, 0, s>>>(
-            part_hdr, reinterpret_cast<const float4*>(part_val), win_slot,
+            part_hdr, reinterpret_cast<const float4*>(part_val), win_row,
             reinterpret_cast<float4*>(win_val), g.units, g.lp, g.p, g.n_chunks, n_windows);
     else
-        fixup_windows_kernel<float><<<grid, BLOCK, 0, s>>>(part_hdr, part_val, win_slot, win_val,
+        fixup_windows_kernel<float><<<grid, BLOCK, 0, s>>>(part_hdr, part_val, win_row, win_val,
                                                            g.units, g.lp, g.p, g.n_chunks, n_windows);
     return hipGetLastError();
 }
 
 hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
-                        const float* part_val, const u32* win_slot, const float* win_val,
+                        const float* part_val, const u32* win_row, const float* win_val,
                         hipStream_t s) {
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads, part_val) && vec4_ok(t, win_val);
@@ -1047,15 +1047,15 @@ hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const u
     dim3 grid((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per chunk
     if (v4)
         fixup_kernel<float4><<<grid, BLOCK, 0, s>>>(
-            t, part_hdr, reinterpret_cast<const float4*>(part_val), win_slot,
+            t, part_hdr, reinterpret_cast<const float4*>(part_val), win_row,
             reinterpret_cast<const float4*>(win_val), g.units, g.lp, g.p, g.n_chunks, n_windows);
     else
-        fixup_kernel<float><<<grid, BLOCK, 0, s>>>(t, part_hdr, part_val, win_slot, win_val, g.units,
+        fixup_kernel<float><<<grid, BLOCK, 0, s>>>(t, part_hdr, part_val, win_row, win_val, g.units,
                                                    g.lp, g.p, g.n_chunks, n_windows);
     return hipGetLastError();
 }
 
-hipError_t launch_update_unique(const TableDev& t, const u32* slot_idx, size_t n, const float* grads,
+hipError_t launch_update_unique(const TableDev& t, const u32* row_idx, size_t n, const float* grads,
                                 hipStream_t s) {
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads);
@@ -1063,9 +1063,9 @@ hipError_t launch_update_unique(const TableDev& t, const u32* slot_idx, size_t n
     dim3 grid(grid_for(n, g.p * (BLOCK / 64), 16384), g.col_blocks);
     if (v4)
         update_unique_kernel<float4><<<grid, BLOCK, 0, s>>>(
-            t, slot_idx, (u32)n, reinterpret_cast<const float4*>(grads), g.units, g.lp, g.p);
+            t, row_idx, (u32)n, reinterpret_cast<const float4*>(grads), g.units, g.lp, g.p);
     else
-        update_unique_kernel<float><<<grid, BLOCK, 0, s>>>(t, slot_idx, (u32)n, grads, g.units, g.lp,
+        update_unique_kernel<float><<<grid, BLOCK, 0, s>>>(t, row_idx, (u32)n, grads, g.units, g.lp,
                                                            g.p);
     return hipGetLastError();
 }

@@ -6,8 +6,9 @@
 // that had a free slot when it was inserted; buckets never lose keys while inserts run, so a
 // lookup stops at the first bucket that still has an empty slot.
 // Rows: dense slab `rows[row * stride_f]`, `vf` floats used per row (weights then optimizer
-// state), handed out by an atomic counter; `row_keys[row]` is the key that owns the row, which
-// makes Dump / iterate a linear walk of the slab.
+// state), numbered densely in batch order as keys are inserted and kept dense by erase (the last
+// rows move into the holes); `row_keys[row]` is the key that owns the row, which makes Dump /
+// iterate a linear walk of the slab.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -131,13 +132,13 @@ hipError_t launch_segreduce(const TableDev& t, const uint32_t* sorted_row, const
                             size_t n, const float* grads, uint4* part_hdr, float* part_val,
                             hipStream_t s);
 // launch_fixup_windows first adds up every window of 64 chunks that lies wholly inside one run
-// (win_slot: n_chunks/64 + 1 words, win_val: as many rows of dim floats), so that launch_fixup can
+// (win_row: n_chunks/64 + 1 words, win_val: as many rows of dim floats), so that launch_fixup can
 // cross such a run a window at a time.
 hipError_t launch_fixup_windows(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
-                                const float* part_val, uint32_t* win_slot, float* win_val,
+                                const float* part_val, uint32_t* win_row, float* win_val,
                                 hipStream_t s);
 hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
-                        const float* part_val, const uint32_t* win_slot, const float* win_val,
+                        const float* part_val, const uint32_t* win_row, const float* win_val,
                         hipStream_t s);
 
 // One optimizer step per located key, no aggregation (keys distinct); rows[i] = row of key i.
