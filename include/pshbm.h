@@ -13,11 +13,16 @@
  *  - Pointers named `d_*` are device pointers on the table's GPU; all others are host pointers
  *    (pageable or pinned) owned by the caller and valid for the duration of the call.
  *  - `*_dev` entry points enqueue work on `stream` (a hipStream_t passed as void*; NULL = the
- *    null stream) and return without waiting, except where noted. The caller orders calls
- *    that touch one table: use one stream, or events between streams. Host-pointer entry
- *    points are synchronous and may be called from several host threads: pulls without
- *    insertion share the table, everything else takes it exclusively — the locking discipline
- *    of pico-ps/operator/SparsePullOperator.h:188-192 and SparsePushOperator.h:220.
+ *    null stream) and return without waiting, except where noted. Calls on one table take
+ *    effect in the order in which they are made, whatever their streams: the library puts the
+ *    events between streams itself. Pulls without insertion share the table — on different
+ *    streams they run side by side on the device and wait only for the last mutating call —
+ *    and everything else takes it exclusively: the locking discipline of
+ *    pico-ps/operator/SparsePullOperator.h:188-192 and SparsePushOperator.h:220. A stream
+ *    handed to a call must stay valid until the table's next mutating call has returned or
+ *    the table is destroyed (that call records an event on it).
+ *    Host-pointer entry points are synchronous. Every entry point may be called from several
+ *    host threads.
  *  - A row is `dim` fp32 weights followed by its optimizer state: SUM and SGD none, ADAGRAD
  *    `dim` accumulators, FTRL `dim` z then `dim` n. `pshbm_value_floats()` gives the total.
  *  - Keys 0xFFFFFFFFFFFFFFFF and 0xFFFFFFFFFFFFFFFE are reserved (the reference's key types
@@ -107,7 +112,9 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out);
 /* Releases the table: the storage destructor (KVShardStorage.h:866-873 erase of each shard). */
 int32_t pshbm_destroy(pshbm_table* t);
 
-/* Message of the last failure on this table (owned by the table, valid until the next call). */
+/* Message of the calling thread's last failed call, on any table or in pshbm_create (the argument
+ * is not used and may be NULL). Kept per thread, as errno is, because calls on one table may fail
+ * on several threads at once; valid until the same thread's next failing call. */
 const char* pshbm_last_error(const pshbm_table* t);
 
 /* Floats per stored value (weights + optimizer state) for a dim and optimizer; 0 if invalid. */

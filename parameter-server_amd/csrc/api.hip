@@ -45,7 +45,7 @@ struct pshbm_table {
     // per-batch workspace of the mutating paths
     size_t ws_cap = 0;
     unsigned sort_parity = 0;  // which half of the sort head the next sort uses
-    DevBuf ws_slot, ws_row, ws_idx, ws_sslot, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wslot, ws_wval, ws_won;
+    DevBuf ws_slot, ws_row, ws_idx, ws_srow, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wrow, ws_wval, ws_won;
     unsigned won_parity = 0;  // which half of ws_won the next inserting operation counts into
 
     // staging of the host-pointer entry points
@@ -71,12 +71,12 @@ struct pshbm_table {
 
     hipStream_t stream = nullptr, side = nullptr;
     hipEvent_t order_ev{};
-    hipStream_t last_stream = nullptr;
-    bool has_last = false;
+    hipStream_t writer_stream = nullptr;      // stream of the last mutating call
+    bool has_writer = false;
+    std::vector<hipStream_t> reader_streams;  // streams of the reading calls since
 
     std::shared_mutex mu;
     uint64_t size_bound = 0;  // upper bound of the rows handed out
-    std::string err;
 
     // optional per-kernel timing (pshbm_profile_*)
     bool prof_on = false;
@@ -97,13 +97,17 @@ struct DeviceGuard {
     }
 };
 
-int32_t fail(pshbm_table* t, int32_t code, const char* fmt, ...) {
+// Message of the calling thread's last failed call: calls on one table may fail on several threads
+// at once, so the text is kept per thread, as errno is.
+thread_local std::string g_error;
+
+int32_t fail(pshbm_table*, int32_t code, const char* fmt, ...) {
     char buf[512];
     va_list ap;
     va_start(ap, fmt);
     vsnprintf(buf, sizeof buf, fmt, ap);
     va_end(ap);
-    if (t) t->err = buf;
+    g_error = buf;
     return code;
 }
 
@@ -171,7 +175,7 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     ST_TRY(ensure(t, t->ws_slot, cap * 4));
     ST_TRY(ensure(t, t->ws_idx, cap * 4));
     ST_TRY(ensure(t, t->ws_row, cap * 4));
-    ST_TRY(ensure(t, t->ws_sslot, cap * 4));
+    ST_TRY(ensure(t, t->ws_srow, cap * 4));
     ST_TRY(ensure(t, t->ws_sidx, cap * 4));
     ST_TRY(ensure(t, t->ws_sort, sort_pairs_temp_bytes(cap)));
     HIP_TRY(t, hipMemset(t->ws_sort.p, 0, sort_pairs_head_bytes()));
@@ -182,7 +186,7 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     size_t chunks = std::max(g1.n_chunks, g4.n_chunks);
     ST_TRY(ensure(t, t->ws_hdr, chunks * sizeof(uint4)));
     ST_TRY(ensure(t, t->ws_pval, chunks * 2 * (size_t)t->d.dim * 4));
-    ST_TRY(ensure(t, t->ws_wslot, (chunks / 64 + 1) * 4));
+    ST_TRY(ensure(t, t->ws_wrow, (chunks / 64 + 1) * 4));
     ST_TRY(ensure(t, t->ws_wval, (chunks / 64 + 1) * (size_t)t->d.dim * 4));
     // winner counts per 1024-key block, two arrays used by alternate operations, zero between uses
     ST_TRY(ensure(t, t->ws_won, 2 * (assign_blocks(cap) + 1) * 4));
@@ -192,14 +196,30 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     return PSHBM_OK;
 }
 
-// Orders this call after the table's previous call when that ran on another stream.
-int32_t begin_op(pshbm_table* t, hipStream_t s) {
-    if (t->has_last && t->last_stream != s) {
-        HIP_TRY(t, hipEventRecord(t->order_ev, t->last_stream));
+// Orders this call, on stream s, after the table's earlier calls that it must not overlap. A
+// reading call (a pull that inserts nothing) waits for the last mutating call only, so pulls on
+// different streams run side by side on the device, as the reference's pulls share a shard
+// (SparsePullOperator.h:188-192); a mutating call waits for the last mutating call and for every
+// reading call since (the exclusive side of the same lock, SparsePushOperator.h:220).
+int32_t begin_op(pshbm_table* t, hipStream_t s, bool reads_only = false) {
+    if (t->has_writer && t->writer_stream != s) {
+        HIP_TRY(t, hipEventRecord(t->order_ev, t->writer_stream));
         HIP_TRY(t, hipStreamWaitEvent(s, t->order_ev, 0));
     }
-    t->last_stream = s;
-    t->has_last = true;
+    if (reads_only) {
+        if (!(t->has_writer && t->writer_stream == s) &&
+            std::find(t->reader_streams.begin(), t->reader_streams.end(), s) == t->reader_streams.end())
+            t->reader_streams.push_back(s);
+        return PSHBM_OK;
+    }
+    for (hipStream_t r : t->reader_streams) {
+        if (r == s) continue;
+        HIP_TRY(t, hipEventRecord(t->order_ev, r));
+        HIP_TRY(t, hipStreamWaitEvent(s, t->order_ev, 0));
+    }
+    t->reader_streams.clear();
+    t->writer_stream = s;
+    t->has_writer = true;
     return PSHBM_OK;
 }
 
@@ -297,7 +317,7 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
     if (unique) {
         HIP_TRY_PROF(t, s, PSHBM_PHASE_UPDATE_UNIQUE, launch_update_unique(t->d, row, n, d_grads, s));
     } else {
-        uint32_t* sslot = static_cast<uint32_t*>(t->ws_sslot.p);
+        uint32_t* srow = static_cast<uint32_t*>(t->ws_srow.p);
         uint32_t* sidx = static_cast<uint32_t*>(t->ws_sidx.p);
         SortPlan plan;
         // a key inserted by this batch more than once: only the claiming occurrence got the row
@@ -305,7 +325,7 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
         HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_HIST,
                      sort_begin(t->ws_sort.p, t->ws_sort.bytes, t->sort_parity++, row, n, t->row_bits,
                                 &plan, s, insert ? &late : nullptr));
-        uint32_t *kin = row, *vin = idx, *kout = sslot, *vout = sidx;
+        uint32_t *kin = row, *vin = idx, *kout = srow, *vout = sidx;
         for (uint32_t p = 0; p < plan.passes; ++p) {
             HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_PASS,
                          sort_pass(plan, p, kin, vin, kout, vout, t->d.counters + CNT_SORT_ERR, s));
@@ -313,17 +333,17 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
             std::swap(vin, vout);
         }
         const bool in_b = (plan.passes & 1u) != 0;
-        const uint32_t* fs = in_b ? sslot : row;
+        const uint32_t* fs = in_b ? srow : row;
         const uint32_t* fi = in_b ? sidx : idx;
         uint4* hdr = static_cast<uint4*>(t->ws_hdr.p);
         float* pval = static_cast<float*>(t->ws_pval.p);
         HIP_TRY_PROF(t, s, PSHBM_PHASE_SEGREDUCE,
                      launch_segreduce(t->d, fs, fi, n, d_grads, hdr, pval, s));
-        uint32_t* wslot = static_cast<uint32_t*>(t->ws_wslot.p);
+        uint32_t* wrow = static_cast<uint32_t*>(t->ws_wrow.p);
         float* wval = static_cast<float*>(t->ws_wval.p);
         HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP_WINDOWS,
-                     launch_fixup_windows(t->d, n, d_grads, hdr, pval, wslot, wval, s));
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP, launch_fixup(t->d, n, d_grads, hdr, pval, wslot, wval, s));
+                     launch_fixup_windows(t->d, n, d_grads, hdr, pval, wrow, wval, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP, launch_fixup(t->d, n, d_grads, hdr, pval, wrow, wval, s));
     }
     return PSHBM_OK;
 }
@@ -357,8 +377,8 @@ int32_t ensure_bulk(pshbm_table* t) {
 void destroy_impl(pshbm_table* t) {
     DeviceGuard g(t->device);
     (void)hipDeviceSynchronize();
-    DevBuf* bufs[] = {&t->ws_slot, &t->ws_row, &t->ws_idx,  &t->ws_sslot, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
-                      &t->ws_pval, &t->ws_wslot, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
+    DevBuf* bufs[] = {&t->ws_slot, &t->ws_row, &t->ws_idx,  &t->ws_srow, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
+                      &t->ws_pval, &t->ws_wrow, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
                       &t->ms_dead, &t->ms_tiles, &t->ms_lists, &t->ms_fe,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
@@ -386,8 +406,6 @@ void destroy_impl(pshbm_table* t) {
     if (t->side) (void)hipStreamDestroy(t->side);
     delete t;
 }
-
-thread_local std::string g_create_error;
 
 // ---- for-each / erase ----------------------------------------------------------------------
 int32_t check_predicate(pshbm_table* t, const pshbm_predicate* w, pshbm_predicate* out) {
@@ -465,15 +483,13 @@ uint32_t pshbm_value_floats(uint32_t dim, int32_t optimizer) {
     return 0;
 }
 
-const char* pshbm_last_error(const pshbm_table* t) {
-    return t ? t->err.c_str() : g_create_error.c_str();
-}
+const char* pshbm_last_error(const pshbm_table*) { return g_error.c_str(); }
 
 int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     if (!cfg || !out) return PSHBM_INVALID_CONFIG;
     *out = nullptr;
     auto bad = [&](const char* m) {
-        g_create_error = m;
+        g_error = m;
         return PSHBM_INVALID_CONFIG;
     };
     if (cfg->struct_size != sizeof(pshbm_config)) return bad("struct_size does not match this library");
@@ -489,7 +505,7 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     int ndev = 0;
     hipError_t e = hipGetDeviceCount(&ndev);
     if (e != hipSuccess || ndev == 0) {
-        g_create_error = std::string("no HIP device: ") + hipGetErrorString(e);
+        g_error = std::string("no HIP device: ") + hipGetErrorString(e);
         return PSHBM_ERROR;
     }
     if (cfg->device < 0 || cfg->device >= ndev) return bad("device ordinal out of range");
@@ -525,7 +541,7 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     t->keys_bytes = max_rows * 8;
 
     auto bail = [&](hipError_t err, const char* what) {
-        g_create_error = std::string(what) + ": " + hipGetErrorString(err);
+        g_error = std::string(what) + ": " + hipGetErrorString(err);
         int32_t code = err == hipErrorOutOfMemory ? PSHBM_OUT_OF_MEMORY : PSHBM_ERROR;
         destroy_impl(t);
         return code;
@@ -555,7 +571,6 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
 #undef CREATE_TRY
     int32_t st = ensure_workspace(t, cfg->max_batch ? cfg->max_batch : 65536);
     if (st != PSHBM_OK) {
-        g_create_error = t->err;
         destroy_impl(t);
         return st;
     }
@@ -580,7 +595,7 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool insert = (flags & PSHBM_PULL_INSERT_ON_MISS) && !t->cfg.read_only;
     std::unique_lock<std::shared_mutex> lk(t->mu);
-    ST_TRY(begin_op(t, s));
+    ST_TRY(begin_op(t, s, !insert));
     if (!insert) {
         HIP_TRY_PROF(t, s, PSHBM_PHASE_PULL, launch_pull(t->d, d_keys, n, d_out_rows, d_hit, s));
         return PSHBM_OK;

@@ -56,3 +56,42 @@ def test_concurrent_pushes_pulls_and_scans(ps, orc, wl):
     np.testing.assert_array_equal(a["key"], b["key"])
     np.testing.assert_array_equal(a["value"], b["value"])
     t.close()
+
+
+def test_pulls_on_several_streams_between_pushes(ps, orc, wl):
+    """Pulls enqueued on four streams overlap on the device; each must still see every push that
+    was made before it and none that was made after it."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(31)
+    dim, n, batch = 16, 200000, 50000
+    t = ps.Table(dim, ps.OPT_SUM, capacity=n + 1000, max_batch=batch)
+    r = orc.Oracle(dim, orc.OPT_SUM, capacity=n + 1000)
+    keys = wl.table_keys_np(0, n, seed=9)
+    vals = rng.integers(-5, 6, (n, dim)).astype(np.float32)
+    assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    push_stream = torch.cuda.Stream()
+    plan = []
+    for it in range(6):                                  # inputs first: nothing waits in the loop below
+        q = keys[rng.integers(0, n, batch)]
+        g = rng.integers(-3, 4, (batch, dim)).astype(np.float32)
+        pulls = []
+        for s in streams:
+            pq = keys[rng.integers(0, n, batch)]
+            pulls.append((pq, torch.from_numpy(pq.view(np.int64)).cuda(),
+                          torch.empty(batch, dim, device="cuda"),
+                          torch.empty(batch, dtype=torch.uint8, device="cuda")))
+        plan.append((q, g, torch.from_numpy(q.view(np.int64)).cuda(), torch.from_numpy(g).cuda(), pulls))
+    torch.cuda.synchronize()
+    for q, g, dq, dg, pulls in plan:
+        assert t.push_dev(dq.data_ptr(), dg.data_ptr(), batch, 0, push_stream.cuda_stream) == 0
+        for s, (pq, dpq, out, hit) in zip(streams, pulls):
+            assert t.pull_dev(dpq.data_ptr(), batch, out.data_ptr(), hit.data_ptr(), 0, s.cuda_stream) == 0
+    torch.cuda.synchronize()
+    for q, g, dq, dg, pulls in plan:
+        assert r.push(q, g) == 0
+        for pq, dpq, out, hit in pulls:
+            st, rows, rhit = r.pull(pq)
+            np.testing.assert_array_equal(out.cpu().numpy(), rows)
+            np.testing.assert_array_equal(hit.cpu().numpy(), rhit)
+    t.close()
