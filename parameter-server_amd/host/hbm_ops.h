@@ -8,6 +8,8 @@
 //   HbmSparsePullOperator  <- SparseTablePullOperator::apply_request   (operator/SparsePullOperator.h:156-254)
 //   HbmSparsePushOperator  <- SparseTablePushOperator server halves    (operator/SparsePushOperator.h:197-416)
 //   HbmDirectPushOperator  <- DirectPushOperator                       (operator/SparsePushOperator.h:520-574)
+//   HbmDensePushOperator   <- DenseTablePushOperator server halves     (operator/DensePushOperator.h:137-316)
+//   HbmDensePullOperator   <- DenseTablePullOperator::apply_request    (operator/DensePullOperator.h:118-181)
 //   HbmDumpOperator        <- BaseKVTextFileDumpOperator::apply_request (operator/DumpOperator.h:137-183)
 //   HbmLoadOperator        <- BaseKVTextFileLoadOperator::restore      (operator/LoadOperator.h:164-213)
 //   HbmForEachOperator     <- SparseTableForEachReadOperator           (operator/ForEachOperator.h:150-233)
@@ -19,6 +21,7 @@
 // application process and are inherited unchanged from the reference's templates.
 #pragma once
 
+#include <algorithm>
 #include <functional>
 #include <memory>
 
@@ -320,6 +323,202 @@ public:
         } else {
             resp.rpc_response().set_error_code(RpcErrorCodeType::ELOGICERROR);
             resp << Status::OOM("PServer OOM during direct push");
+        }
+    }
+};
+
+// ---- dense tables ----------------------------------------------------------------------------
+// A dense parameter is a vector stored under a dense_key_t (an int64 id >= 0) and cut by the
+// client's value partitioner into slices; the server keeps one map entry per slice under
+// dense_slice_key_t {id, slice_id} (pico-ps/common/dense_common.h:19-104). On an HBM table a slice
+// is one row of `dim` floats under the 64-bit key  id << 24 | slice_id  (ids below 2^39, slice ids
+// below 2^24; the reference's empty and deleted slice keys have negative fields and cannot occur).
+// Rows have one length, so every slice on the wire is exactly `dim` floats: the client uses
+// HbmDenseValuePartitioner, which pads the last slice of a parameter with zeros, and
+// HbmDenseValueMerger, which drops the padding again.
+inline uint64_t dense_slice_key(int64_t id, int32_t slice_id) {
+    PSHBM_SCHECK(id >= 0 && id < (int64_t(1) << 39) && slice_id >= 0 && slice_id < (1 << 24),
+                 "dense slice key out of range");  // dense_common.h:77-83
+    return (uint64_t)id << 24 | (uint32_t)slice_id;
+}
+
+// VAL_PARTITIONER of a dense table (the role of DenseValuePartitioner, dense_common.h:137-151, and of
+// TestValuePartitioner, pico-ps/test/TestOps.h:307-319): slices of `block` elements, the last padded.
+struct HbmDenseValuePartitioner {
+    struct PartitionResult {
+        std::vector<size_t> serialized_size;
+        std::vector<std::vector<float>> parts;
+    };
+    explicit HbmDenseValuePartitioner(size_t block) : _block(block) {}
+    PartitionResult partition(int64_t /*key*/, const std::vector<float>& origin) const {
+        PartitionResult r;
+        for (size_t l = 0; l < origin.size(); l += _block) {
+            const size_t e = std::min(l + _block, origin.size());
+            r.parts.emplace_back(origin.begin() + l, origin.begin() + e);
+            r.parts.back().resize(_block, 0.0f);
+            r.serialized_size.push_back(_block * sizeof(float));
+        }
+        return r;
+    }
+
+private:
+    size_t _block;
+};
+
+// VAL_MERGER of a dense table (DenseValueMerger, dense_common.h:153-175; TestValueMerger,
+// TestOps.h:321-335): slice `idx` lands at idx * block of the pulled vector, cut at its end.
+struct HbmDenseValueMerger {
+    explicit HbmDenseValueMerger(size_t block) : _block(block) {}
+    size_t slice_number(int64_t /*key*/, const std::vector<float>& val) const { return (val.size() + _block - 1) / _block; }
+    void merge(std::vector<float>& merged, const std::vector<float>& slice, size_t idx) const {
+        const size_t at = idx * _block;
+        PSHBM_SCHECK(at <= merged.size(), "dense slice beyond the pulled vector");
+        std::copy(slice.begin(), slice.begin() + std::min(slice.size(), merged.size() - at), merged.begin() + at);
+    }
+
+private:
+    size_t _block;
+};
+
+// Server halves of the dense push (DenseTablePushOperator, operator/DensePushOperator.h:137-316).
+// Request: dense key, i32 shards_num; per shard {i32 shard_id, i32 shard_slices_num; per slice
+// {i32 slice_id; one lazy block = the slice's push value, `dim` raw floats}} (:97-127). The slices
+// of one shard go to the table as one batch. The update is the table's optimizer: a slice that is
+// absent is created by its first push, as init_store_value of the test operator does
+// (pico-ps/test/TestOps.h:355-359), a present one goes through store_push_value (:372-376).
+class HbmDensePushOperator {
+public:
+    explicit HbmDensePushOperator(const Configure&) {}
+
+    void apply_async_push_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, Storage* /*incr_storage*/,
+                                  PSResponse& resp) {  // :137-200
+        Status status;
+        for_each_shard(rt, req, storage, [&](pshbm_table* t, const std::vector<uint64_t>& keys, const std::vector<float>& vals) {
+            int32_t rc = pshbm_push(t, keys.data(), vals.data(), keys.size(), 0);
+            if (rc == PSHBM_OUT_OF_MEMORY) status = Status::OOM(pshbm_last_error(t));
+            else if (rc != PSHBM_OK) status = Status::Error(pshbm_last_error(t));
+        });
+        PSHBM_SCHECK(req.archive().is_exhausted(), "request not exhausted");  // :197
+        resp = PSResponse(req);
+        if (!status.ok()) resp.rpc_response().set_error_code(RpcErrorCodeType::ELOGICERROR);
+        resp << status;
+    }
+
+    // :202-253: the slices are merged into the delta storage (merge_push_value); here they are
+    // queued in the shard's table and summed at the store.
+    void apply_sync_push_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp) {
+        Status status;
+        for_each_shard(rt, req, storage, [&](pshbm_table* t, const std::vector<uint64_t>& keys, const std::vector<float>& vals) {
+            if (pshbm_queue(t, keys.data(), vals.data(), keys.size()) != PSHBM_OK) status = Status::Error(pshbm_last_error(t));
+        });
+        PSHBM_SCHECK(req.archive().is_exhausted(), "request not exhausted");  // :250
+        resp = PSResponse(req);
+        resp << status;
+    }
+
+    // :255-316: acknowledge first (:290-292), then apply every merged slice.
+    void apply_store_request(RuntimeInfo& rt, PSRequest& req, Storage* delta_storage, Storage* storage,
+                             Storage* /*incr_storage*/, std::function<void(PSResponse&&)> send_response) {
+        int32_t shard_id;
+        req >> shard_id;
+        PSHBM_SCHECK(req.archive().is_exhausted(), "request not exhausted");                 // :262
+        PSHBM_SCHECK(rt.local_shards().count(shard_id), "Bad Request: invalid shard_id");  // :263-264
+        PSResponse resp(req);
+        resp << Status();
+        send_response(std::move(resp));
+        if (delta_storage == nullptr) return;  // :266-271
+        pshbm_store(static_cast<HbmShardStorage*>(storage)->get(shard_id), 0);
+    }
+
+    std::unique_ptr<Storage> create_delta_storage(RuntimeInfo&) { return std::make_unique<HbmDeltaStorage>(); }  // :325-327
+
+private:
+    template <class F>
+    static void for_each_shard(RuntimeInfo& rt, PSRequest& req, Storage* storage, F&& f) {
+        int64_t key;
+        int32_t shards_num;
+        req >> key >> shards_num;
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        const size_t dim = st.dim();
+        std::vector<uint64_t> keys;
+        std::vector<float> vals;
+        while (shards_num--) {
+            int32_t shard_id, shard_slices_num;
+            req >> shard_id >> shard_slices_num;
+            PSHBM_SCHECK(rt.local_shards().count(shard_id) != 0, "Bad Request: invalid shard_id");  // :157-158
+            keys.clear();
+            vals.clear();
+            while (shard_slices_num--) {
+                int32_t slice_id;
+                req >> slice_id;
+                std::vector<char> push_val;
+                ps_deserialize(req.lazy(), push_val);
+                PSHBM_SCHECK(push_val.size() == dim * 4, "dense slice is not `dim` floats");
+                keys.push_back(dense_slice_key(key, slice_id));
+                const float* v = reinterpret_cast<const float*>(push_val.data());
+                vals.insert(vals.end(), v, v + dim);
+            }
+            if (!keys.empty()) f(st.get(shard_id), keys, vals);
+        }
+    }
+};
+
+// Server half of the dense pull (DenseTablePullOperator::apply_request, operator/DensePullOperator.h:118-181).
+// Request: dense key, i32 shards_num; per shard {i32 shard_id, i32 shard_slices_num; the slice ids}
+// (:100-112). Response: i32 shards_num; per shard {i32 shard_slices_num; per slice {i32 slice_id}},
+// with one lazy block of `dim` floats per slice, in request order. A slice that is not stored is a
+// programmer error there (SCHECK(it != ht.end()), :154) and here.
+class HbmDensePullOperator {
+public:
+    explicit HbmDensePullOperator(const Configure&) {}
+    void apply_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp) {
+        int64_t key;
+        int32_t shards_num;
+        req >> key >> shards_num;
+        resp = PSResponse(req);
+        resp << shards_num;
+        bool healthy = true;
+        std::string why;
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        const size_t dim = st.dim();
+        std::vector<std::vector<char>> blocks;
+        std::vector<uint64_t> keys;
+        std::vector<float> rows;
+        std::vector<uint8_t> hit;
+        while (shards_num--) {
+            int32_t shard_id, shard_slices_num;
+            req >> shard_id >> shard_slices_num;
+            resp << shard_slices_num;
+            PSHBM_SCHECK(rt.local_shards().count(shard_id) != 0, "Bad Request: invalid shard_id");  // :140-141
+            keys.clear();
+            for (int32_t i = 0; i < shard_slices_num; ++i) {
+                int32_t slice_id;
+                req >> slice_id;
+                resp << slice_id;
+                keys.push_back(dense_slice_key(key, slice_id));
+            }
+            if (keys.empty()) continue;
+            rows.resize(keys.size() * dim);
+            hit.assign(keys.size(), 0);
+            pshbm_table* t = st.get(shard_id);
+            if (pshbm_pull(t, keys.data(), keys.size(), rows.data(), hit.data(), 0) != PSHBM_OK) {
+                healthy = false;
+                why = pshbm_last_error(t);
+                continue;
+            }
+            for (size_t i = 0; i < keys.size(); ++i) {
+                PSHBM_SCHECK(hit[i], "dense slice is not stored");  // :154
+                const char* p = reinterpret_cast<const char*>(rows.data() + i * dim);
+                blocks.emplace_back(p, p + dim * 4);
+            }
+        }
+        PSHBM_SCHECK(req.archive().is_exhausted(), "request not exhausted");  // :180
+        if (healthy) {
+            for (auto& b : blocks) ps_serialize(resp.lazy(), std::move(b));
+        } else {  // :170-179
+            resp = PSResponse(req);
+            resp.rpc_response().set_error_code(RpcErrorCodeType::ELOGICERROR);
+            resp << Status::OOM("PServer OOM during dense pull: " + why);
         }
     }
 };

@@ -118,6 +118,208 @@ struct FileReader {  // stands for TestDsReader (TestOpsDs.h:47-75); dim-2 SUM v
     }
 };
 
+
+// ---- dense tables: the flow of test_dense (pico-ps/test/ps_service_test.cpp:241-409) -------------
+// Every "rank" owns the dense keys [rank*100, (rank+1)*100); the parameter of key k is the vector
+// {k, k+1, ..., 2k-1} (k elements, :262-266), cut into slices of DENSE_BLOCK_SIZE = 5
+// (pico-ps/test/TestOps.h:270); the test operator adds what is pushed (TestOps.h:351-377).
+static constexpr size_t DENSE_BLOCK_SIZE = 5;
+static int32_t dense_partition(int64_t key, int32_t slice_id) { return (int32_t)((key * 31 + slice_id) % NUM_SHARDS); }
+
+static std::vector<float> dense_arg(int32_t key) {
+    std::vector<float> v(key);
+    for (int32_t i = 0; i < key; ++i) v[i] = (float)(key + i);
+    return v;
+}
+
+// generate_push_request of the dense push (operator/DensePushOperator.h:89-131)
+static bool make_dense_push_request(int64_t key, const std::vector<float>& arg, PSRequest& req) {
+    HbmDenseValuePartitioner partitioner(DENSE_BLOCK_SIZE);
+    auto parted = partitioner.partition(key, arg);
+    std::vector<std::vector<int32_t>> shards_slices(NUM_SHARDS);
+    for (size_t slice_id = 0; slice_id < parted.parts.size(); ++slice_id)
+        shards_slices[dense_partition(key, (int32_t)slice_id)].push_back((int32_t)slice_id);
+    req << key << (int32_t)NUM_SHARDS;
+    int32_t total = 0;
+    for (int32_t shard_id = 0; shard_id < NUM_SHARDS; ++shard_id) {
+        req << shard_id << (int32_t)shards_slices[shard_id].size();
+        for (int32_t slice_id : shards_slices[shard_id]) {
+            req << slice_id;
+            const auto& part = parted.parts[slice_id];
+            const char* p = reinterpret_cast<const char*>(part.data());
+            ps_serialize(req.lazy(), std::vector<char>(p, p + part.size() * 4));
+            ++total;
+        }
+    }
+    return total != 0;  // a request without slices is not sent (:127-129)
+}
+
+// generate_request + apply_response of the dense pull (operator/DensePullOperator.h:60-116, 183-221)
+static std::vector<float> dense_pull(HbmDensePullOperator& op, RuntimeInfo& rt, Storage* st, int64_t key, size_t len) {
+    HbmDenseValueMerger merger(DENSE_BLOCK_SIZE);
+    std::vector<float> pull_arg(len, -1.0f);
+    const int32_t slices_num = (int32_t)merger.slice_number(key, pull_arg);
+    if (slices_num == 0) return pull_arg;
+    std::vector<std::vector<int32_t>> shards_slices(NUM_SHARDS);
+    for (int32_t slice_id = 0; slice_id < slices_num; ++slice_id) shards_slices[dense_partition(key, slice_id)].push_back(slice_id);
+    PSRequest req;
+    req << key << (int32_t)NUM_SHARDS;
+    for (int32_t shard_id = 0; shard_id < NUM_SHARDS; ++shard_id) {
+        req << shard_id << (int32_t)shards_slices[shard_id].size();
+        for (int32_t slice_id : shards_slices[shard_id]) req << slice_id;
+    }
+    PSResponse resp;
+    op.apply_request(rt, req, st, resp);
+    EXPECT(resp.error_code() == RpcErrorCodeType::SUCC);
+    int32_t shards_num;
+    resp >> shards_num;
+    int32_t seen = 0;
+    while (shards_num--) {
+        int32_t shard_slices_num;
+        resp >> shard_slices_num;
+        while (shard_slices_num--) {
+            int32_t slice_id;
+            resp >> slice_id;
+            EXPECT(0 <= slice_id && slice_id < slices_num);
+            std::vector<char> block;
+            ps_deserialize(resp.lazy(), block);
+            EXPECT(block.size() == DENSE_BLOCK_SIZE * 4);
+            std::vector<float> slice(DENSE_BLOCK_SIZE);
+            std::memcpy(slice.data(), block.data(), block.size());
+            merger.merge(pull_arg, slice, slice_id);
+            ++seen;
+        }
+    }
+    EXPECT(seen == slices_num && resp.archive().is_exhausted() && resp.lazy().empty());
+    return pull_arg;
+}
+
+template <size_t VF>
+struct FixedReader {
+    std::ifstream f;
+    bool open(const std::string& name) {
+        f.open(name, std::ios::binary);
+        return f.good();
+    }
+    bool read(uint64_t& key, float* value) {
+        f.read(reinterpret_cast<char*>(&key), 8);
+        f.read(reinterpret_cast<char*>(value), VF * 4);
+        return f.good();
+    }
+};
+
+static void test_dense(const std::string& dir) {
+    Configure op_config;
+    op_config.set("dim", (double)DENSE_BLOCK_SIZE);
+    op_config.set("optimizer", "sum");
+    op_config.set("hbm_table.expected_max_items", 40000);
+    op_config.set("block_size", 100);
+    RuntimeInfo rt(0, {0, 1});
+    HbmStorageOperator storage_op(op_config);
+    std::unique_ptr<Storage> storage = storage_op.create_storage(rt, 0);
+    HbmDensePushOperator push_op(op_config);
+    HbmDensePullOperator pull_op(op_config);
+    std::unique_ptr<Storage> delta = push_op.create_delta_storage(rt);
+    const int32_t max_key = NUM_RANKS * TEST_KEY_NUM;
+
+    auto push = [&](int32_t key, bool sync) {
+        PSRequest req;
+        if (!make_dense_push_request(key, dense_arg(key), req)) return;
+        PSResponse resp;
+        Status status;
+        if (sync) push_op.apply_sync_push_request(rt, req, storage.get(), resp);
+        else push_op.apply_async_push_request(rt, req, storage.get(), nullptr, resp);
+        resp >> status;
+        EXPECT(status.ok());
+    };
+    auto store = [&]() {
+        for (int32_t shard = 0; shard < NUM_SHARDS; ++shard) {
+            PSRequest req;
+            req << shard;
+            bool acked = false;
+            push_op.apply_store_request(rt, req, delta.get(), storage.get(), nullptr, [&](PSResponse&& r) {
+                Status s;
+                r >> s;
+                acked = s.ok();
+            });
+            EXPECT(acked);
+        }
+    };
+    auto expect_all = [&](HbmDensePullOperator& op, Storage* st, int odd_factor, int even_factor) {
+        for (int32_t key = 0; key < max_key; ++key) {
+            const int rank = key / TEST_KEY_NUM;
+            const float f = (float)(rank % 2 == 0 ? even_factor : odd_factor);
+            auto got = dense_pull(op, rt, st, key, key);
+            bool same = got.size() == (size_t)key;
+            for (int32_t i = 0; same && i < key; ++i) same = got[i] == (float)(key + i) * f;
+            EXPECT(same);
+        }
+    };
+    for (int32_t key = 0; key < max_key; ++key) {  // :259-272
+        push(key, false);
+        push(key, true);
+    }
+    store();                                         // :274-277
+    for (int32_t key = 0; key < max_key; ++key)      // :280-291: even ranks once more
+        if ((key / TEST_KEY_NUM) % 2 == 0) push(key, true);
+    store();                                         // :296-298
+    expect_all(pull_op, storage.get(), 2, 3);
+    for (int32_t key = 0; key < max_key; ++key) {    // :307-326
+        push(key, false);
+        push(key, true);
+        if ((key / TEST_KEY_NUM) % 2 == 0) push(key, true);
+    }
+    expect_all(pull_op, storage.get(), 3, 4);        // :332-347: (key + i) * (3 + (rank even)); the queue is not applied yet
+    store();                                         // :356-357
+    // one table row per slice of DENSE_BLOCK_SIZE elements
+    uint64_t slices = 0;
+    for (int32_t key = 0; key < max_key; ++key) slices += (key + DENSE_BLOCK_SIZE - 1) / DENSE_BLOCK_SIZE;
+    auto* hst = static_cast<HbmShardStorage*>(storage.get());
+    EXPECT(hst->shard_size(0) + hst->shard_size(1) == slices);
+
+    // dump (:359-361), then load into a storage created anew (:368-377) and pull (:393-409)
+    HbmDumpOperator<FileWriter> dump_op(op_config);
+    std::vector<std::string> files;
+    for (int32_t file_id = 0; file_id < 2; ++file_id) {
+        PSRequest req;
+        DumpArgs args{dir, 2};
+        std::vector<int32_t> shard_ids{file_id};
+        req.archive() << args << file_id << shard_ids;
+        PSResponse resp;
+        dump_op.apply_request(rt, req, storage.get(), resp);
+        Status status;
+        resp >> status;
+        EXPECT(status.ok());
+        files.push_back(dir + "/model_0_" + std::to_string(file_id));
+    }
+    std::unique_ptr<Storage> loaded = storage_op.create_storage(rt, 1);
+    HbmLoadOperator<FixedReader<DENSE_BLOCK_SIZE>> load_op(op_config);
+    load_op.restore(files, rt, loaded.get(), [](uint64_t k) { return dense_partition((int64_t)(k >> 24), (int32_t)(k & 0xFFFFFF)); });
+    HbmDensePullOperator pull_loaded(op_config);
+    expect_all(pull_loaded, loaded.get(), 4, 6);     // (key + i) * (2 + (rank even)) * 2, :401
+
+    // a slice that was never pushed is a programmer error (DensePullOperator.h:154)
+    bool threw = false;
+    try {
+        dense_pull(pull_loaded, rt, loaded.get(), max_key + 7, 12);
+    } catch (const std::logic_error&) {
+        threw = true;
+    }
+    EXPECT(threw);
+    // a slice of the wrong length is refused
+    threw = false;
+    try {
+        PSRequest req;
+        req << (int64_t)3 << (int32_t)1 << (int32_t)0 << (int32_t)1 << (int32_t)0;
+        ps_serialize(req.lazy(), std::vector<char>(12));
+        PSResponse resp;
+        push_op.apply_async_push_request(rt, req, storage.get(), nullptr, resp);
+    } catch (const std::logic_error&) {
+        threw = true;
+    }
+    EXPECT(threw);
+}
+
 int main(int argc, char** argv) {
     const std::string dir = argc > 1 ? argv[1] : "/tmp";
     Configure op_config;
@@ -444,6 +646,7 @@ int main(int argc, char** argv) {
         EXPECT(total_size(storage.get()) == (uint64_t)TEST_KEY_NUM * NUM_RANKS + 1);
     }
 
+    test_dense(dir);
     if (g_failed) {
         std::printf("FAILED: %d expectation(s)\n", g_failed);
         return 1;

@@ -101,8 +101,62 @@ def native_ps_roundtrip(num_process=2, per_rank=150):
             "cite": "pico-ps/test/ps_predictor_native_ps_test.cpp:108-170", "ops": ops}
 
 
+DENSE_BLOCK_SIZE = 5  # pico-ps/test/TestOps.h:270
+
+
+def test_dense(num_process=3, per_rank=3):
+    """pico-ps/test/ps_service_test.cpp:241-409 (test_dense). The dense parameter of key k is the
+    vector {k, k+1, ..., 2k-1} (:262-266), cut into slices of DENSE_BLOCK_SIZE (TestValuePartitioner,
+    TestOps.h:307-319); the test operator adds what is pushed (TestOps.h:351-377). A slice
+    {id, slice_id} (pico-ps/common/dense_common.h:67-104) is the table row of key id << 24 | slice_id,
+    the last slice of a parameter padded with zeros. (The reference uses 100 keys per rank; the
+    fixture keeps the stride of 100 and the first `per_rank` keys of every rank.)"""
+    def slices(k):
+        arg = [k + i for i in range(k)]
+        out = []
+        for s in range(0, k, DENSE_BLOCK_SIZE):
+            part = arg[s:s + DENSE_BLOCK_SIZE]
+            out.append(((k << 24) | (s // DENSE_BLOCK_SIZE), part + [0] * (DENSE_BLOCK_SIZE - len(part))))
+        return out
+
+    ranks = []
+    for rank in range(num_process):
+        items = [it for k in range(rank * TEST_KEY_NUM, rank * TEST_KEY_NUM + per_rank) for it in slices(k)]
+        ranks.append(([it[0] for it in items], [it[1] for it in items]))
+    ops = []
+    for keys, grads in ranks:                                             # :259-272
+        ops.append({"op": "push", "keys": keys, "grads": grads})
+        ops.append({"op": "queue", "keys": keys, "grads": grads})
+    ops.append({"op": "store"})                                           # :274-277
+    for rank, (keys, grads) in enumerate(ranks):                          # :280-291
+        if rank % 2 == 0:
+            ops.append({"op": "queue", "keys": keys, "grads": grads})
+    ops.append({"op": "store"})                                           # :296-298
+    for rank, (keys, grads) in enumerate(ranks):                          # :307-326
+        ops.append({"op": "push", "keys": keys, "grads": grads})
+        ops.append({"op": "queue", "keys": keys, "grads": grads})
+        if rank % 2 == 0:
+            ops.append({"op": "queue", "keys": keys, "grads": grads})
+
+    def expect(factor):
+        keys, rows = [], []
+        for rank, (ks, gs) in enumerate(ranks):
+            keys += ks
+            rows += [[v * factor(rank) for v in g] for g in gs]
+        return {"op": "expect_pull", "keys": keys, "rows": rows, "hit": [1] * len(keys)}
+
+    ops.append(expect(lambda rank: 3 + (rank % 2 == 0)))                  # :332-347: queued pushes not applied yet
+    ops.append({"op": "store"})                                           # :356-357
+    n_slices = sum(len(ks) for ks, _ in ranks)
+    ops.append({"op": "dump_load_roundtrip", "expect_size": n_slices})   # :359-390
+    for _ in range(2):
+        ops.append(expect(lambda rank: (2 + (rank % 2 == 0)) * 2))       # :393-409
+    return {"name": f"test_dense_{num_process}", "dim": DENSE_BLOCK_SIZE, "optimizer": "SUM",
+            "cite": "pico-ps/test/ps_service_test.cpp:241-409, pico-ps/test/TestOps.h:270-399", "ops": ops}
+
+
 def main():
-    scenarios = [test_sparse(1), test_sparse(3), pmem_three_pushes(), native_ps_roundtrip()]
+    scenarios = [test_sparse(1), test_sparse(3), pmem_three_pushes(), native_ps_roundtrip(), test_dense()]
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_known_answers.json")
     with open(out, "w") as f:
         json.dump({"scenarios": scenarios}, f, separators=(",", ":"))
