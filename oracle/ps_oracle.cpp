@@ -23,6 +23,19 @@
 //       pinned by the reference's test operators (pico-ps/test/TestOps.h:138-185: erase the odd
 //       keys; count and sum every record) and the counts its service test asserts
 //       (pico-ps/test/ps_service_test.cpp:158-166,176-184), and by a brute-force dict model.
+//   pso_for_each_write
+//       the loop is the reference's (ForEachOperator.h:277-359: every record, hook on a writable
+//       value); the hook (affine map / clamp of a column range under a predicate) is this
+//       repository's, the reference ships none that writes: PARITY UNPINNED BY THE REFERENCE,
+//       pinned by an independent numpy model of the two formulas (tests/test_for_each_write.py).
+//   pso_increment_size, pso_take_increment
+//       which keys a push or store touched (the second storage the reference mirrors them into,
+//       SparsePushOperator.h:253-266,394-407, read and emptied by IncrementStorage.h:29-36);
+//       pinned by a dict-and-set model of those lines (tests/test_increment.py). The reference has
+//       no test of its own for the increment.
+//   Dense tables need nothing of their own here: a slice {id, slice_id} is the key
+//       id << 24 | slice_id of the same functions; the reference's test_dense
+//       (pico-ps/test/ps_service_test.cpp:241-409) is one of the known-answer scenarios.
 //   SGD / ADAGRAD / FTRL arithmetic (apply_update below)
 //       PARITY UNPINNED BY THE REFERENCE: pico-ps ships no optimizer (the update is the user
 //       hook SparsePushOperator.h:448). The formulas are this repository's definition; they are
