@@ -50,28 +50,57 @@ __device__ __forceinline__ bool eval_pred(const pshbm_predicate& p, u64 key, con
 }
 
 // ---- for-each ------------------------------------------------------------------------------
-// A workgroup of 256 threads = G groups of lp lanes (lp = columns handled at once); group g takes
-// rows blockIdx.x * G + g, then every gridDim.x * G-th row after it, and lane c adds up column c of
-// the rows that satisfy the predicate. The G sums of a column are then added in group order, and
+// A workgroup of 256 threads = G groups of lp lanes (lp = columns handled at once); the workgroups
+// take spans of G * FE_UNROLL consecutive rows in turn, group g every G-th row of a span, and lane c
+// adds up column c of the rows that satisfy the predicate. The G sums of a column are then added in group order, and
 // the per-workgroup results in workgroup order by for_each_final_kernel: a fixed order throughout.
 // partial: [gridDim.x][vf + 1] doubles, the last one the count.
+constexpr u32 FE_UNROLL = 8;
 __global__ __launch_bounds__(BLOCK) void for_each_kernel(TableDev t, u32 n_rows, pshbm_predicate pred,
                                                           double* __restrict__ partial, u32 lp,
                                                           u32 G) {
     __shared__ double sh[BLOCK];
     __shared__ unsigned long long cnts[BLOCK];
+    __shared__ uint8_t okf[BLOCK * FE_UNROLL];
     const u32 tid = threadIdx.x;
     const u32 g = tid / lp, cl = tid - g * lp;
     const u32 c = blockIdx.y * 256u + cl;
+    const bool has_pred = pred.n_terms != 0;
+    const u32 span = G * FE_UNROLL;  // consecutive rows the workgroup reads per step
     double acc = 0.0;
     unsigned long long cnt = 0;
-    if (g < G) {
-        for (u64 r = (u64)blockIdx.x * G + g; r < n_rows; r += (u64)gridDim.x * G) {
-            const float* row = t.rows + r * t.stride_f;
-            if (eval_pred(pred, t.row_keys[r], row)) {
-                if (c < t.vf) acc += (double)row[c];
-                ++cnt;
+    for (u64 s0 = (u64)blockIdx.x * span; s0 < n_rows; s0 += (u64)gridDim.x * span) {
+        if (has_pred) {  // once per row, a thread per row; the flags go through LDS
+            __syncthreads();
+            for (u32 x = tid; x < span; x += BLOCK) {
+                const u64 r = s0 + x;
+                okf[x] = r < n_rows && eval_pred(pred, t.row_keys[r], t.rows + r * t.stride_f) ? 1 : 0;
             }
+            __syncthreads();
+        }
+        if (g < G) {
+            // FE_UNROLL rows per step, their loads issued together; a group adds its rows in
+            // ascending order
+            float v[FE_UNROLL];
+            bool ok[FE_UNROLL];
+#pragma unroll
+            for (u32 k = 0; k < FE_UNROLL; ++k) {
+                const u32 x = k * G + g;
+                const u64 r = s0 + x;
+                ok[k] = r < n_rows;
+                v[k] = 0.0f;
+                if (ok[k] && c < t.vf) v[k] = t.rows[r * t.stride_f + c];
+            }
+            if (has_pred) {
+#pragma unroll
+                for (u32 k = 0; k < FE_UNROLL; ++k) ok[k] = ok[k] && okf[k * G + g] != 0;
+            }
+#pragma unroll
+            for (u32 k = 0; k < FE_UNROLL; ++k)
+                if (ok[k]) {
+                    acc += (double)v[k];
+                    ++cnt;
+                }
         }
     }
     sh[tid] = acc;
@@ -89,14 +118,22 @@ __global__ __launch_bounds__(BLOCK) void for_each_kernel(TableDev t, u32 n_rows,
     }
 }
 
+// Workgroup c adds up column c (c = vf: the count) of the per-workgroup results: thread x takes
+// every BLOCK-th of them in ascending order, then the BLOCK sums are added in thread order.
 __global__ __launch_bounds__(BLOCK) void for_each_final_kernel(const double* __restrict__ partial,
                                                                 u32 n_blocks, u32 vf,
                                                                 double* __restrict__ out) {
-    const u32 c = blockIdx.x * BLOCK + threadIdx.x;
-    if (c > vf) return;
+    __shared__ double sh[BLOCK];
+    const u32 c = blockIdx.x;
     double s = 0.0;
-    for (u32 b = 0; b < n_blocks; ++b) s += partial[(u64)b * (vf + 1) + c];
-    out[c] = s;
+    for (u32 b = threadIdx.x; b < n_blocks; b += BLOCK) s += partial[(u64)b * (vf + 1) + c];
+    sh[threadIdx.x] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double tot = 0.0;
+        for (u32 x = 0; x < BLOCK; ++x) tot += sh[x];
+        out[c] = tot;
+    }
 }
 
 // Writing for-each: thread per row; the predicate is evaluated on the row as it is before the
@@ -133,10 +170,18 @@ __global__ __launch_bounds__(BLOCK) void for_each_write_kernel(TableDev t, u32 n
     }
 }
 
-__global__ void sum_partials_kernel(const double* __restrict__ partial, u32 n, double* __restrict__ out) {
+__global__ __launch_bounds__(BLOCK) void sum_partials_kernel(const double* __restrict__ partial, u32 n,
+                                                              double* __restrict__ out) {
+    __shared__ double sh[BLOCK];
     double s = 0.0;
-    for (u32 b = 0; b < n; ++b) s += partial[b];
-    out[0] = s;
+    for (u32 b = threadIdx.x; b < n; b += BLOCK) s += partial[b];
+    sh[threadIdx.x] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double tot = 0.0;
+        for (u32 x = 0; x < BLOCK; ++x) tot += sh[x];
+        out[0] = tot;
+    }
 }
 
 // ---- erase ---------------------------------------------------------------------------------
@@ -420,7 +465,7 @@ hipError_t launch_for_each(const TableDev& t, uint32_t n_rows, const pshbm_predi
     for_each_kernel<<<grid, BLOCK, 0, s>>>(t, n_rows, pred, partial, lp, G);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    for_each_final_kernel<<<(t.vf + 1 + BLOCK - 1) / BLOCK, BLOCK, 0, s>>>(partial, n_blocks, t.vf, scratch);
+    for_each_final_kernel<<<t.vf + 1, BLOCK, 0, s>>>(partial, n_blocks, t.vf, scratch);
     return hipGetLastError();
 }
 
@@ -431,7 +476,7 @@ hipError_t launch_for_each_write(const TableDev& t, uint32_t n_rows, const pshbm
     for_each_write_kernel<<<n_blocks, BLOCK, 0, s>>>(t, n_rows, pred, what, partial);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    sum_partials_kernel<<<1, 1, 0, s>>>(partial, n_blocks, scratch);
+    sum_partials_kernel<<<1, BLOCK, 0, s>>>(partial, n_blocks, scratch);
     return hipGetLastError();
 }
 
