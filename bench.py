@@ -126,6 +126,38 @@ def run_steps(t, torch, cfg, batches, out, steps, first=0):
             raise RuntimeError(f"step {i} failed: {st} {t.last_error()}")
 
 
+def scan_table(ps, t, cfg, n_table):
+    """Whole-table operations at the table's full size: every row and key is read once, so the
+    algorithmic bytes of a for-each are rows * (8 + 4 * value floats). Median of 5 calls (the first
+    call, which allocates scratch, is not counted); the erase-if runs once, last."""
+    rec = 8 + 4 * t.value_floats
+    where = ps.predicate((3 % cfg["dim"], ps.CMP_GT, 0.0128))   # weights are N(0, 0.01): about a tenth
+
+    def timed(f, reps):
+        f()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            r = f()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2], r
+
+    rows = t.size()
+    dt_all, (st, cnt, _) = timed(lambda: t.for_each(), 5)
+    assert st == 0 and cnt == rows
+    dt_sel, (st, n_sel, _) = timed(lambda: t.for_each(where), 5)
+    assert st == 0
+    t0 = time.perf_counter()
+    st, erased = t.erase_if(where)
+    dt_erase = time.perf_counter() - t0
+    assert st == 0 and erased == n_sel and t.size() == rows - n_sel
+    return {"rows": rows, "record_bytes": rec,
+            "for_each_ms": round(dt_all * 1e3, 3), "for_each_GBps": round(rows * rec / dt_all / 1e9, 1),
+            "for_each_where_ms": round(dt_sel * 1e3, 3), "selected": int(n_sel),
+            "erase_if_ms": round(dt_erase * 1e3, 3), "erased": int(erased),
+            "note": "wall clock of the synchronous calls, read-back of the result included"}
+
+
 def cpu_baseline(cfg, wl, budget_keys):
     """The oracle (a scalar port of the reference's operator loops) on a bounded sample of the same
     workload: a table of budget_keys keys and a few batches of the configured size, one thread."""
@@ -233,6 +265,10 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device copy, a kernel of known HBM traffic that "
                          "rocprofv3 --pmc runs of this script use to scale FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--scan", action="store_true",
+                    help="after the steps, also time the whole-table operations on the same table: "
+                         "for-each (count + column sums), for-each under a predicate on a value "
+                         "column, erase-if of about a tenth of the keys; reported under \"scan\"")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -306,6 +342,8 @@ def main():
         "roofline": roofline,
         "phases": phases,
     }
+    if args.scan:
+        result["scan"] = scan_table(ps, t, cfg, n_table)
     t.close()
     del out, batches
     torch.cuda.empty_cache()
