@@ -147,6 +147,10 @@ def scan_table(ps, t, cfg, n_table):
     assert st == 0 and cnt == rows
     dt_sel, (st, n_sel, _) = timed(lambda: t.for_each(where), 5)
     assert st == 0
+    # the writing for-each with the identity map 1 * v + 0 on every column: rows read and written
+    ident = ps.update(ps.UPD_AFFINE, 0, t.value_floats, 1.0, 0.0)
+    dt_write, (st, n_written) = timed(lambda: t.for_each_write(ident), 3)
+    assert st == 0 and n_written == rows
     t0 = time.perf_counter()
     st, erased = t.erase_if(where)
     dt_erase = time.perf_counter() - t0
@@ -154,6 +158,8 @@ def scan_table(ps, t, cfg, n_table):
     return {"rows": rows, "record_bytes": rec,
             "for_each_ms": round(dt_all * 1e3, 3), "for_each_GBps": round(rows * rec / dt_all / 1e9, 1),
             "for_each_where_ms": round(dt_sel * 1e3, 3), "selected": int(n_sel),
+            "for_each_write_ms": round(dt_write * 1e3, 3),
+            "for_each_write_GBps": round(rows * (rec + rec - 8) / dt_write / 1e9, 1),
             "erase_if_ms": round(dt_erase * 1e3, 3), "erased": int(erased),
             "note": "wall clock of the synchronous calls, read-back of the result included"}
 

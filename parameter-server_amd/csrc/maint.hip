@@ -136,34 +136,66 @@ __global__ __launch_bounds__(BLOCK) void for_each_final_kernel(const double* __r
     }
 }
 
-// Writing for-each: thread per row; the predicate is evaluated on the row as it is before the
-// rewrite. counts: one partial per workgroup, added up in workgroup order afterwards.
+// Writing for-each, in the layout of for_each_kernel: the workgroups take spans of G * FE_UNROLL
+// consecutive rows in turn; a thread per row evaluates the predicate on the row as it is before
+// the rewrite (flags through LDS, the mark of a selected row is set here), then group g rewrites
+// every G-th row of the span, lane c the columns c, c + 256, ... that `what` names.
+// partial: the selected rows of every workgroup, added up in a fixed order afterwards.
 __global__ __launch_bounds__(BLOCK) void for_each_write_kernel(TableDev t, u32 n_rows, pshbm_predicate pred,
                                                                 pshbm_update what,
-                                                                double* __restrict__ partial) {
+                                                                double* __restrict__ partial, u32 lp,
+                                                                u32 G) {
     __shared__ u32 wsum[BLOCK / 64];
+    __shared__ uint8_t okf[BLOCK * FE_UNROLL];
+    const u32 tid = threadIdx.x;
+    const u32 g = tid / lp, cl = tid - g * lp;
+    const bool has_pred = pred.n_terms != 0;
+    const u32 c_end = what.first_column + what.n_columns;
+    const u32 span = G * FE_UNROLL;
     u32 mine = 0;
-    for (u64 r = (u64)blockIdx.x * BLOCK + threadIdx.x; r < n_rows; r += (u64)gridDim.x * BLOCK) {
-        float* row = t.rows + r * t.stride_f;
-        if (!eval_pred(pred, t.row_keys[r], row)) continue;
-        ++mine;
-        for (u32 c = what.first_column; c < what.first_column + what.n_columns; ++c) {
-            const float v = row[c];
-            float out;
-            if (what.op == PSHBM_UPD_AFFINE) {
-                const float p = what.a * v;
-                out = p + what.b;
-            } else {
-                out = fminf(fmaxf(v, what.a), what.b);
+    for (u64 s0 = (u64)blockIdx.x * span; s0 < n_rows; s0 += (u64)gridDim.x * span) {
+        __syncthreads();
+        for (u32 x = tid; x < span; x += BLOCK) {
+            const u64 r = s0 + x;
+            const bool ok = r < n_rows &&
+                            (!has_pred || eval_pred(pred, t.row_keys[r], t.rows + r * t.stride_f));
+            okf[x] = ok ? 1 : 0;
+            if (ok) {
+                ++mine;
+                if (t.dirty) t.dirty[r] = 1;
             }
-            row[c] = out;
         }
-        if (t.dirty) t.dirty[r] = 1;
+        __syncthreads();
+        if (g >= G) continue;
+        for (u32 c = cl; c < c_end; c += 256u) {
+            if (c < what.first_column) continue;
+            float v[FE_UNROLL];
+            bool ok[FE_UNROLL];
+#pragma unroll
+            for (u32 k = 0; k < FE_UNROLL; ++k) {
+                const u32 x = k * G + g;
+                ok[k] = s0 + x < n_rows && okf[x] != 0;
+                v[k] = 0.0f;
+                if (ok[k]) v[k] = t.rows[(s0 + x) * t.stride_f + c];
+            }
+#pragma unroll
+            for (u32 k = 0; k < FE_UNROLL; ++k) {
+                if (!ok[k]) continue;
+                float out;
+                if (what.op == PSHBM_UPD_AFFINE) {
+                    const float p = what.a * v[k];
+                    out = p + what.b;
+                } else {
+                    out = fminf(fmaxf(v[k], what.a), what.b);
+                }
+                t.rows[(s0 + k * G + g) * t.stride_f + c] = out;
+            }
+        }
     }
     for (u32 off = 32; off >= 1; off >>= 1) mine += __shfl_down(mine, off);
-    if ((threadIdx.x & 63u) == 0) wsum[threadIdx.x >> 6] = mine;
+    if ((tid & 63u) == 0) wsum[tid >> 6] = mine;
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (tid == 0) {
         u32 s = 0;
         for (u32 x = 0; x < BLOCK / 64; ++x) s += wsum[x];
         partial[blockIdx.x] = (double)s;
@@ -471,9 +503,10 @@ hipError_t launch_for_each(const TableDev& t, uint32_t n_rows, const pshbm_predi
 
 hipError_t launch_for_each_write(const TableDev& t, uint32_t n_rows, const pshbm_predicate& pred,
                                  const pshbm_update& what, double* scratch, hipStream_t s) {
-    const u32 n_blocks = blocks_for(n_rows, BLOCK * 4, FE_BLOCKS_MAX);
+    u32 lp, G;
+    const u32 n_blocks = for_each_blocks(t, n_rows, &lp, &G);
     double* partial = scratch + (t.vf + 1);
-    for_each_write_kernel<<<n_blocks, BLOCK, 0, s>>>(t, n_rows, pred, what, partial);
+    for_each_write_kernel<<<n_blocks, BLOCK, 0, s>>>(t, n_rows, pred, what, partial, lp, G);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     sum_partials_kernel<<<1, BLOCK, 0, s>>>(partial, n_blocks, scratch);
