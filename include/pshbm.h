@@ -175,15 +175,18 @@ int32_t pshbm_set_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_val
                       void* stream);
 
 /* Bulk load of n records {uint64 key; float value[pshbm_value_floats()]} from host memory,
- * streamed to the device through pinned staging on a side stream and upserted block by block.
- * Replaces BaseKVTextFileLoadOperator::restore (pico-ps/operator/LoadOperator.h:164-213) once the
- * file is decoded; with PSHBM_LOAD_UNIQUE a key that is already present (or repeated) fails with
- * PSHBM_ERROR the way restore aborts on it (:194,210), and the records loaded before the failing
- * block stay. */
+ * streamed to the device on a side stream, 32 MiB at a time, and upserted block by block. Records
+ * in page-locked memory (pshbm_host_alloc) are fetched by the copy engine as they lie; others
+ * pass through a pair of pinned staging buffers. Replaces BaseKVTextFileLoadOperator::restore
+ * (pico-ps/operator/LoadOperator.h:164-213) once the file is decoded; with PSHBM_LOAD_UNIQUE a key
+ * that is already present (or repeated) fails with PSHBM_ERROR the way restore aborts on it
+ * (:194,210), and the records loaded before the failing block stay. A record with a reserved key
+ * is left out and the call returns PSHBM_ERROR after loading the others. */
 int32_t pshbm_load(pshbm_table* t, const void* records, size_t n, uint32_t flags);
 
-/* Bulk dump of every (key, value) as the same records, in row-slab order, through the same
- * staging. Replaces the shard walk of BaseKVTextFileDumpOperator::apply_request
+/* Bulk dump of every (key, value) as the same records, in row-slab order, the same way (written by
+ * the copy engine directly when `records` is page-locked, through the staging pair otherwise).
+ * Replaces the shard walk of BaseKVTextFileDumpOperator::apply_request
  * (pico-ps/operator/DumpOperator.h:163-174). *n_out = records written; ERROR if capacity_records
  * is smaller than the table. The order is unspecified as the reference's is (map iteration order). */
 int32_t pshbm_dump(pshbm_table* t, void* records, size_t capacity_records, size_t* n_out);

@@ -376,17 +376,21 @@ int32_t pso_load(void* h, const void* records, size_t n, uint32_t flags) {
     Oracle& o = *static_cast<Oracle*>(h);
     const size_t rec = 8 + (size_t)o.vf * 4;
     const char* p = static_cast<const char*>(records);
+    bool skipped = false;  // a record with a reserved key is left out and the load reports an error
     for (size_t i = 0; i < n; ++i) {
         uint64_t key;
         std::memcpy(&key, p + i * rec, 8);
-        if (reserved(key)) return ST_ERROR;
+        if (reserved(key)) {
+            skipped = true;
+            continue;
+        }
         auto it = o.map.find(key);
         if (it != o.map.end() && (flags & LOAD_UNIQUE)) return ST_ERROR;
         if (it == o.map.end() && o.map.size() + 1 > o.c.capacity) return ST_OOM;
         uint32_t r = it == o.map.end() ? append_row(o, key) : it->second;
         std::memcpy(&o.rows[(size_t)r * o.vf], p + i * rec + 8, (size_t)o.vf * 4);
     }
-    return ST_OK;
+    return skipped ? ST_ERROR : ST_OK;
 }
 
 // KVShardIterator::iterate_batch_as_binary_archive, KVShardStorage.h:64-87: records

@@ -10,6 +10,7 @@ raise.
 import ctypes as C
 import os
 import subprocess
+import weakref
 
 import numpy as np
 
@@ -211,6 +212,21 @@ def record_dtype(vf):
     return np.dtype([("key", "<u8"), ("value", "<f4", (vf,))])
 
 
+def pinned_empty(shape, dtype):
+    """An uninitialised numpy array in page-locked host memory (pshbm_host_alloc), freed when the
+    array and its views are gone. Load and Dump move such buffers without staging copies."""
+    dtype = np.dtype(dtype)
+    n = int(np.prod(shape)) if not np.isscalar(shape) else int(shape)
+    nbytes = max(n * dtype.itemsize, 1)
+    p = C.c_void_p()
+    st = lib().pshbm_host_alloc(C.byref(p), nbytes)
+    if st != OK:
+        raise PshbmError(st, "pshbm_host_alloc failed")
+    buf = (C.c_char * nbytes).from_address(p.value)
+    weakref.finalize(buf, lib().pshbm_host_free, C.c_void_p(p.value))
+    return np.frombuffer(buf, dtype=dtype, count=n).reshape(shape)
+
+
 def _u64(a):
     return np.ascontiguousarray(a, dtype=np.uint64)
 
@@ -296,11 +312,19 @@ class Table:
         r = np.ascontiguousarray(records, dtype=record_dtype(self.value_floats))
         return lib().pshbm_load(self._h, r.ctypes.data, r.size, flags)
 
-    def dump(self):
+    def dump(self, pinned=False, out=None):
+        """(status, records). pinned=True returns them in page-locked memory, which the copy
+        engine writes directly; `out` reuses a record array of the caller (page-locking a large
+        buffer costs more than the dump itself)."""
         n = self.size()
-        rec = np.empty(n, dtype=record_dtype(self.value_floats))
+        if out is not None:
+            if out.dtype != record_dtype(self.value_floats) or out.size < n or not out.flags.c_contiguous:
+                raise ValueError("out: a contiguous record array of at least size() records")
+            rec = out
+        else:
+            rec = (pinned_empty if pinned else np.empty)(n, dtype=record_dtype(self.value_floats))
         got = C.c_size_t()
-        st = lib().pshbm_dump(self._h, rec.ctypes.data, n, C.byref(got))
+        st = lib().pshbm_dump(self._h, rec.ctypes.data, rec.size, C.byref(got))
         return st, rec[: got.value]
 
     def iterate(self, offset, batch):

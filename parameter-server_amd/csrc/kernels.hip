@@ -154,6 +154,31 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
             bool done = !active || f.slot != SLOT_NONE;
             u32 b = (u32)hash64(key) & t.bucket_mask;
             u32 steps = 0;
+            // A key that is not seen goes straight for the first slot that looked empty. The view
+            // may be old, but only in one direction (slots go from empty to a key and stay), so the
+            // first slot that is truly empty is not before this one, and a copy of the key that
+            // another group stored during this launch is either seen, or in this slot, or behind
+            // a slot that looked empty and is not -- the compare-and-swap tells which: it finds
+            // the slot empty (claimed), holding the key (a repeat), or holding another key (then
+            // the bucket is looked at again, with loads that bypass the caches).
+            if (__ballot(!done)) {
+                const bool try_it = !done && f.empty != SLOT_NONE;
+                u64 old = 0;
+                if (try_it && sub == 0)
+                    old = atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[f.empty]),
+                                    (unsigned long long)KEY_EMPTY, (unsigned long long)key);
+                const u64 oldb = shfl64(old, grp * 4);
+                if (try_it) {
+                    b = f.empty >> 2;  // the buckets before it are full and stay full
+                    if (oldb == KEY_EMPTY || oldb == key) {
+                        slot = f.empty;
+                        row = ROW_PENDING;
+                        won = oldb == KEY_EMPTY;
+                        dup = !won;
+                        done = true;
+                    }
+                }
+            }
             while (__ballot(!done)) {
                 u64 skey = 0;
                 u32 srow = ROW_NONE;
@@ -213,9 +238,15 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
             // block: rows are handed out afterwards by assign_rows_kernel. (One shared row counter
             // bumped from here costs a device-scope atomic on one address per wavefront, which
             // serialises: 1.5 ms for 200,000 inserts.)
-            if (won && sub == 0) {
-                atomicAdd(&won_count[i / ASSIGN_KEYS], 1u);
-                slot |= WON_BIT;
+            // (Nor does every winner count itself: additions to one address are resolved one
+            // after the other, about 120 ns each, and the 1024 keys of a block are probed at about
+            // the same time. The 16 keys of a round lie in one block: one addition per wavefront.)
+            static_assert(ASSIGN_KEYS % KEYS_PER_ROUND == 0, "a round's keys share a block");
+            const u64 wm = __ballot(won && sub == 0);
+            if (wm) {
+                if (lane == (u32)__ffsll((unsigned long long)wm) - 1u)
+                    atomicAdd(&won_count[base / ASSIGN_KEYS], (u32)__popcll(wm));
+                if (won && sub == 0) slot |= WON_BIT;
             }
         }
         if (inb && sub == 0) {

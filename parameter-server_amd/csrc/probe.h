@@ -19,15 +19,16 @@ __device__ __forceinline__ u64 shfl64(u64 v, u32 src) {
 
 
 struct Found {
-    u32 slot;
+    u32 slot;   // where the key is, or SLOT_NONE
     u32 row;
+    u32 empty;  // on a miss: the first empty slot of the bucket where the walk ended, or SLOT_NONE
 };
 
 // Four lanes (sub = 0..3 of group grp) look for `key`. Every lane of the wavefront must call
 // this; lanes whose `active` is false only take part in the ballots.
 __device__ __forceinline__ Found probe_find(const TableDev& t, u64 key, bool active, u32 grp,
                                             u32 sub) {
-    Found f{SLOT_NONE, ROW_NONE};
+    Found f{SLOT_NONE, ROW_NONE, SLOT_NONE};
     u32 b = (u32)hash64(key) & t.bucket_mask;
     bool done = !active;
     u32 steps = 0;
@@ -47,6 +48,7 @@ __device__ __forceinline__ Found probe_find(const TableDev& t, u64 key, bool act
                 f.row = row;
                 done = true;
             } else if (e4) {
+                f.empty = b * 4 + (u32)__ffs((int)e4) - 1u;
                 done = true;
             } else {
                 b = (b + 1) & t.bucket_mask;

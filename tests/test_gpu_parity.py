@@ -336,6 +336,47 @@ def test_dump_load_iterate_roundtrip(ps, orc, wl, opt, dim):
     t.close(), t2.close()
 
 
+def test_bulk_transfers_through_page_locked_buffers(ps, orc, wl):
+    """Dump into and Load from page-locked memory take the path without staging copies; the
+    records are the same as through pageable buffers (6 staging chunks here)."""
+    rng = np.random.default_rng(21)
+    dim, n = 128, 200000                       # 200000 x 520 B = 104 MB
+    t = ps.Table(dim, ps.OPT_SGD, lr=0.5, capacity=n)
+    keys = wl.table_keys_np(0, n, seed=8)
+    vals = rng.normal(0, 1, (n, dim)).astype(np.float32)
+    assert t.set(keys, vals) == 0
+    st, plain = t.dump()
+    st2, locked = t.dump(pinned=True)
+    assert st == 0 and st2 == 0
+    np.testing.assert_array_equal(plain, locked)
+    order = np.argsort(keys)
+    srt = np.sort(locked, order="key")
+    np.testing.assert_array_equal(srt["key"], keys[order])
+    np.testing.assert_array_equal(srt["value"], vals[order])
+    t2 = ps.Table(dim, ps.OPT_SGD, lr=0.5, capacity=n)
+    assert t2.load(locked, ps.LOAD_UNIQUE) == 0 and t2.size() == n
+    np.testing.assert_array_equal(np.sort(t2.dump()[1], order="key"), srt)
+    # a slice that starts inside the page-locked buffer is page-locked too
+    assert t2.clear() == 0 and t2.load(locked[1000:151000], ps.LOAD_UNIQUE) == 0 and t2.size() == 150000
+    t.close(), t2.close()
+
+
+def test_load_leaves_out_records_with_reserved_keys(ps, orc):
+    dim = 4
+    t = ps.Table(dim, capacity=100)
+    r = orc.Oracle(dim, capacity=100)
+    rec = np.zeros(10, dtype=ps.record_dtype(dim))
+    rec["key"] = np.arange(10, dtype=np.uint64) + 5
+    rec["key"][3] = 0xFFFFFFFFFFFFFFFF
+    rec["key"][7] = 0xFFFFFFFFFFFFFFFE
+    rec["value"] = np.arange(40, dtype=np.float32).reshape(10, dim)
+    assert t.load(rec) == ps.ERROR and r.load(rec) == orc.ERROR
+    assert "reserved" in t.last_error()
+    assert t.size() == 8 and r.size() == 8
+    np.testing.assert_array_equal(np.sort(t.dump()[1], order="key"), np.sort(r.dump()[1], order="key"))
+    t.close()
+
+
 def test_reserved_keys_and_stats(ps, orc, wl):
     t = ps.Table(4, capacity=20000, max_load_factor=0.8)
     bad = np.array([1, 0xFFFFFFFFFFFFFFFF], np.uint64)
