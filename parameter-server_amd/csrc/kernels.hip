@@ -130,7 +130,11 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
         bool inb = i < n;
         u64 key = inb ? keys[i] : KEY_EMPTY;
         bool active = inb && key < KEY_DELETED;
-        if (inb && !active && sub == 0) atomicAdd(&t.counters[CNT_BADKEY], 1u);
+        {  // one addition per wavefront: a batch full of them must not queue up on one address
+            const u64 bm = __ballot(inb && !active && sub == 0);
+            if (bm && lane == (u32)__ffsll((unsigned long long)bm) - 1u)
+                atomicAdd(&t.counters[CNT_BADKEY], (u32)__popcll(bm));
+        }
         u32 slot = SLOT_NONE;
         u32 row = ROW_NONE;
         bool dup = false;
@@ -253,7 +257,11 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
             slot_out[i] = slot;
             if (idx_out) idx_out[i] = (u32)i;
             if (row_out) row_out[i] = row;
-            if (count_dups && dup) atomicAdd(&t.counters[CNT_DUP], 1u);
+        }
+        if (count_dups) {
+            const u64 dm = __ballot(inb && sub == 0 && dup);
+            if (dm && lane == (u32)__ffsll((unsigned long long)dm) - 1u)
+                atomicAdd(&t.counters[CNT_DUP], (u32)__popcll(dm));
         }
     }
 }
@@ -921,29 +929,34 @@ __global__ __launch_bounds__(BLOCK) void unpack_records_kernel(const u32* __rest
     }
 }
 
-// distance, in buckets, between a stored key's home bucket and the bucket that holds it
+// distance, in buckets, between a stored key's home bucket and the bucket that holds it: four lanes
+// per key walk the chain, the counts are kept per workgroup in LDS and added to `hist` once per
+// workgroup and bin (additions to one address from all over the device are resolved one by one).
 __global__ __launch_bounds__(BLOCK) void probe_hist_kernel(TableDev t, u32 n_rows,
                                                             unsigned long long* hist) {
-    for (u64 r = (u64)blockIdx.x * BLOCK + threadIdx.x; r < n_rows; r += (u64)gridDim.x * BLOCK) {
-        u64 key = t.row_keys[r];
-        if (key >= KEY_DELETED) continue;
-        u32 b = (u32)hash64(key) & t.bucket_mask;
-        u32 dist = 0;
-        bool found = false;
-        while (!found && dist <= t.bucket_mask) {
-            for (u32 k = 0; k < 4 && !found; ++k) {
-                uint4 s = t.slots[(u64)b * 4 + k];
-                found = ((((u64)s.y) << 32) | s.x) == key;
-            }
-            if (!found) {
-                b = (b + 1) & t.bucket_mask;
-                ++dist;
-            }
+    __shared__ u32 h[16];
+    __shared__ u32 hmax;
+    if (threadIdx.x < 16) h[threadIdx.x] = 0;
+    if (threadIdx.x == 16) hmax = 0;
+    __syncthreads();
+    const u32 lane = threadIdx.x & 63u;
+    const u32 grp = lane >> 2, sub = lane & 3u;
+    const u64 wave = ((u64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
+    const u64 nwaves = ((u64)gridDim.x * BLOCK) >> 6;
+    for (u64 base = wave * KEYS_PER_ROUND; base < n_rows; base += nwaves * KEYS_PER_ROUND) {
+        const u64 r = base + grp;
+        const u64 key = r < n_rows ? t.row_keys[r] : KEY_EMPTY;
+        const bool active = key < KEY_DELETED;
+        const Found f = probe_find(t, key, active, grp, sub);
+        if (active && sub == 0 && f.slot != SLOT_NONE) {
+            const u32 dist = ((f.slot >> 2) - ((u32)hash64(key) & t.bucket_mask)) & t.bucket_mask;
+            atomicAdd(&h[dist < 15u ? dist : 15u], 1u);
+            atomicMax(&hmax, dist);
         }
-        if (!found) continue;
-        atomicAdd(&hist[dist < 15 ? dist : 15], 1ull);
-        atomicMax(&hist[16], (unsigned long long)dist);
     }
+    __syncthreads();
+    if (threadIdx.x < 16 && h[threadIdx.x]) atomicAdd(&hist[threadIdx.x], (unsigned long long)h[threadIdx.x]);
+    if (threadIdx.x == 16 && hmax) atomicMax(&hist[16], (unsigned long long)hmax);
 }
 
 inline u32 grid_for(u64 work_items, u32 per_block, u32 cap) {
@@ -1143,7 +1156,7 @@ hipError_t launch_unpack_records(const u32* records, size_t n, u32 stride_dw, u3
 hipError_t launch_probe_hist(const TableDev& t, u32 n_rows, unsigned long long* hist,
                              hipStream_t s) {
     if (n_rows == 0) return hipSuccess;
-    probe_hist_kernel<<<grid_for(n_rows, BLOCK, 65536), BLOCK, 0, s>>>(t, n_rows, hist);
+    probe_hist_kernel<<<grid_for(n_rows, KEYS_PER_ROUND * (BLOCK / 64) * 8, 16384), BLOCK, 0, s>>>(t, n_rows, hist);
     return hipGetLastError();
 }
 
