@@ -122,7 +122,8 @@ struct pshbm_table {
     hipEvent_t order_ev{};
     hipStream_t writer_stream = nullptr;      // stream of the last mutating call
     bool has_writer = false;
-    std::vector<hipStream_t> reader_streams;  // streams of the reading calls since
+    // streams, other than the writer's, that have waited for the last mutating call and pulled since
+    std::vector<hipStream_t> reader_streams;
 
     std::shared_mutex mu;
     uint64_t size_bound = 0;  // upper bound of the rows handed out
@@ -251,15 +252,19 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
 // (SparsePullOperator.h:188-192); a mutating call waits for the last mutating call and for every
 // reading call since (the exclusive side of the same lock, SparsePushOperator.h:220).
 int32_t begin_op(pshbm_table* t, hipStream_t s, bool reads_only = false) {
+    if (reads_only) {
+        if (!t->has_writer || t->writer_stream == s) return PSHBM_OK;  // nothing to wait for, or stream order
+        // one wait per reading stream and mutating call: later pulls on s are behind it already
+        if (std::find(t->reader_streams.begin(), t->reader_streams.end(), s) != t->reader_streams.end())
+            return PSHBM_OK;
+        HIP_TRY(t, hipEventRecord(t->order_ev, t->writer_stream));
+        HIP_TRY(t, hipStreamWaitEvent(s, t->order_ev, 0));
+        t->reader_streams.push_back(s);
+        return PSHBM_OK;
+    }
     if (t->has_writer && t->writer_stream != s) {
         HIP_TRY(t, hipEventRecord(t->order_ev, t->writer_stream));
         HIP_TRY(t, hipStreamWaitEvent(s, t->order_ev, 0));
-    }
-    if (reads_only) {
-        if (!(t->has_writer && t->writer_stream == s) &&
-            std::find(t->reader_streams.begin(), t->reader_streams.end(), s) == t->reader_streams.end())
-            t->reader_streams.push_back(s);
-        return PSHBM_OK;
     }
     for (hipStream_t r : t->reader_streams) {
         if (r == s) continue;
