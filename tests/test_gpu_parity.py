@@ -543,3 +543,39 @@ def test_erase_many_rounds_triggers_rebuild(ps, orc, wl):
         assert_same_table(t, r, exact=True)
     assert t.size() == r.size() == 12 * 99
     t.close()
+
+
+@pytest.mark.parametrize("opt,dim", [("ftrl", 16384), ("adagrad", 4097), ("sum", 16384)])
+def test_largest_rows(ps, orc, wl, opt, dim):
+    """The largest dim the library takes (16384: rows of up to 192 KB with FTRL state) and an odd one
+    just past a power of two: every entry point on a small table, against the oracle."""
+    rng = np.random.default_rng(dim)
+    n = 120
+    t, r = pair(ps, orc, dim, opt, capacity=400)
+    keys = wl.table_keys_np(0, n, seed=2)
+    vf = t.value_floats
+    vals = rng.integers(-3, 4, (n, vf)).astype(np.float32)
+    if opt != "sum":
+        vals[:, dim:] = np.abs(vals[:, dim:]) + 1.0
+    assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+    q = np.concatenate([keys[rng.integers(0, n, 150)], wl.fresh_keys_np(rng, 20)])
+    g = rng.integers(-2, 3, (q.size, dim)).astype(np.float32)
+    if opt != "sum":
+        q = np.unique(q)                      # inexact optimizers: distinct keys compare bit for bit
+        g = g[: q.size]
+    a, b = t.pull(q), r.pull(q)
+    np.testing.assert_array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+    np.testing.assert_array_equal(a[2], b[2])
+    assert t.push(q, g) == 0 and r.push(q, g) == 0
+    assert_same_table(t, r, exact=True)
+    a, b = t.for_each(), r.for_each()
+    assert a[:2] == b[:2]
+    np.testing.assert_allclose(a[2], b[2], rtol=1e-12, atol=1e-9)
+    where = [(-1, 6, (3, 1))]
+    assert t.erase_if(ps.predicate(*where)) == r.erase_if(orc.predicate(*where))
+    assert_same_table(t, r, exact=True)
+    st, rec = t.dump()
+    t2 = ps.Table(dim, capacity=400, **OPTS[opt])
+    assert t2.load(rec, ps.LOAD_UNIQUE) == 0
+    np.testing.assert_array_equal(np.sort(t2.dump()[1], order="key"), np.sort(rec, order="key"))
+    t.close(), t2.close()
