@@ -139,7 +139,8 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
  * store_push_value = one optimizer step with the summed gradient). grads is n x dim.
  * OUT_OF_MEMORY when the new keys do not fit: then the table is unchanged (the reference parks
  * such items in the shard's overflow vector, :257-259; a fixed-capacity table refuses the batch).
- * The *_dev form synchronizes only when the table is within n keys of its capacity. */
+ * The *_dev form synchronizes only when the table is within n keys of its capacity. A batch (and
+ * what is queued for one store) holds at most 2^30-1 keys; pulls, sets and erases 2^31-1. */
 int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, size_t n,
                    uint32_t flags);
 int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,

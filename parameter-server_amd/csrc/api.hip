@@ -21,6 +21,7 @@ namespace {
 
 constexpr size_t BULK_CHUNK_BYTES = 32u << 20;  // staging granule of load / dump
 constexpr uint32_t MAX_DIM = 16384;
+constexpr size_t MAX_PUSH_BATCH = (1u << 30) - 1;  // the sort's tile counters hold 30 bits
 
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
@@ -693,7 +694,7 @@ int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_gr
     if (!t) return PSHBM_INVALID_ID;
     if (n == 0) return PSHBM_OK;
     if (!d_keys || !d_grads) return fail(t, PSHBM_ERROR, "push: null buffer");
-    if (n > 0x7FFFFFFFull) return fail(t, PSHBM_ERROR, "push: batch larger than 2^31-1 keys");
+    if (n > MAX_PUSH_BATCH) return fail(t, PSHBM_ERROR, "push: batch larger than 2^30-1 keys");
     DeviceGuard g(t->device);
     std::unique_lock<std::shared_mutex> lk(t->mu);
     return push_locked(t, d_keys, d_grads, n, flags, static_cast<hipStream_t>(stream));
@@ -775,7 +776,7 @@ int32_t pshbm_queue_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_g
     DeviceGuard g(t->device);
     hipStream_t s = static_cast<hipStream_t>(stream);
     std::unique_lock<std::shared_mutex> lk(t->mu);
-    if (t->q_n + n > 0x7FFFFFFFull) return fail(t, PSHBM_ERROR, "queue: more than 2^31-1 keys queued");
+    if (t->q_n + n > MAX_PUSH_BATCH) return fail(t, PSHBM_ERROR, "queue: more than 2^30-1 keys queued");
     ST_TRY(begin_op(t, s));
     const size_t gb = (size_t)t->d.dim * 4;
     const size_t need = t->q_n + n;
