@@ -27,17 +27,22 @@ def _same(t, r):
     assert t.size() == r.size()
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(36))
 def test_random_operation_sequences(ps, orc, wl, seed):
+    """Seeds from 24 on run at a load factor of 0.9 of the slot array, where probe chains run over
+    several buckets and the markers of erased keys sit inside them."""
     rng = np.random.default_rng(1000 + seed)
     dim = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 31, 32, 64, 100, 128, 257]))
     opt = OPTS[seed % 4]
     exact_dups = opt["optimizer"] in (0, 1)
     cap = int(rng.integers(3000, 20000))
-    t = ps.Table(dim, capacity=cap, track_increment=True, **opt)
+    dense = seed >= 24
+    lf = 0.9 if dense else 0.0
+    t = ps.Table(dim, capacity=cap, track_increment=True, max_load_factor=lf, **opt)
     r = orc.Oracle(dim, capacity=cap, track_increment=True, **opt)
     vf = t.value_floats
-    universe = wl.table_keys_np(0, cap // 2, seed=seed + 50)
+    # a dense table is also kept nearly full: the key universe is 95 % of its capacity
+    universe = wl.table_keys_np(0, cap * 19 // 20 if dense else cap // 2, seed=seed + 50)
 
     def grads(n):
         return rng.integers(-4, 5, (n, dim)).astype(np.float32)
@@ -110,7 +115,7 @@ def test_random_operation_sequences(ps, orc, wl, seed):
             assert x == y and x[0] == 0
         elif op == "dump_load":
             st, rec = t.dump()
-            t2 = ps.Table(dim, capacity=cap, track_increment=True, **opt)
+            t2 = ps.Table(dim, capacity=cap, track_increment=True, max_load_factor=lf, **opt)
             assert t2.load(rec, ps.LOAD_UNIQUE) == 0
             t.close()
             t = t2
