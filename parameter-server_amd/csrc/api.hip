@@ -378,8 +378,9 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
         // a key inserted by this batch more than once: only the claiming occurrence got the row
         const SortLateKeys late{ROW_PENDING, slot, t->d.slots};
         HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_HIST,
-                     sort_begin(t->ws_sort.p, t->ws_sort.bytes, t->sort_parity++, row, n, t->row_bits,
+                     sort_begin(t->ws_sort.p, t->ws_sort.bytes, t->sort_parity, row, n, t->row_bits,
                                 &plan, s, insert ? &late : nullptr));
+        if (plan.uses_head) ++t->sort_parity;  // each such sort zeroes the other half for the next
         uint32_t *kin = row, *vin = idx, *kout = srow, *vout = sidx;
         for (uint32_t p = 0; p < plan.passes; ++p) {
             HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_PASS,

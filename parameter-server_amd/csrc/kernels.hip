@@ -1064,12 +1064,20 @@ hipError_t launch_segreduce(const TableDev& t, const u32* sorted_row, const u32*
     return hipGetLastError();
 }
 
+// A window lies wholly inside a run only if the run entered it from the window before, so window 0
+// never does: with fewer than two whole windows there is nothing for fixup_windows_kernel to add up,
+// and fixup_kernel (which is told so by n_windows = 0) looks at no window.
+inline u32 window_count(u32 n_chunks) {
+    return n_chunks < 2 * WINDOW ? 0u : (n_chunks + WINDOW - 1) / WINDOW;
+}
+
 hipError_t launch_fixup_windows(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
                                 const float* part_val, u32* win_row, float* win_val, hipStream_t s) {
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads, part_val) && vec4_ok(t, win_val);  // the layout launch_segreduce chose
     const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
-    const u32 n_windows = (g.n_chunks + WINDOW - 1) / WINDOW;
+    const u32 n_windows = window_count(g.n_chunks);
+    if (n_windows == 0) return hipSuccess;
     dim3 grid((n_windows + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per window
     if (v4)
         fixup_windows_kernel<float4><<<grid, BLOCK, 0, s>>>(
@@ -1087,7 +1095,7 @@ hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const u
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads, part_val) && vec4_ok(t, win_val);
     const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
-    const u32 n_windows = (g.n_chunks + WINDOW - 1) / WINDOW;
+    const u32 n_windows = window_count(g.n_chunks);
     dim3 grid((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per chunk
     if (v4)
         fixup_kernel<float4><<<grid, BLOCK, 0, s>>>(

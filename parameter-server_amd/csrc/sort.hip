@@ -9,7 +9,8 @@
 //      many pairs with digit b lie in earlier tiles (below);
 //   3. the pairs are first put in digit order in LDS, then written out by consecutive lanes, so
 //      that each run of equal digits is a contiguous, coalesced store.
-// How a tile learns what lies before it depends on the size of the input.
+// An input of one tile is sorted by one launch, all passes in LDS (sort_one_tile_kernel). Otherwise,
+// how a tile learns what lies before it depends on the size of the input.
 //   * Up to 256 tiles (2^20 pairs; one tile per compute unit, all resident at once) a pass is ONE
 //     launch: every tile publishes its counts, the last tile of every group of 16 tiles also
 //     publishes the group's count, and a tile adds up at most 15 tile words and 15 group words --
@@ -398,6 +399,117 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
     }
 }
 
+// An input of one tile: all digit passes in one launch. The pairs go from registers to their
+// places in LDS and back, pass after pass, ranked exactly as in sort_pass_kernel; only the last
+// pass writes to memory.
+template <u32 BITS>
+__global__ __launch_bounds__(SORT_BLOCK) void sort_one_tile_kernel(const u32* __restrict__ kin,
+                                                                    const u32* __restrict__ vin,
+                                                                    u32* __restrict__ kout,
+                                                                    u32* __restrict__ vout, u32 n,
+                                                                    u32 passes, SortLateKeys late) {
+    constexpr u32 RADIX = 1u << BITS;
+    __shared__ u32 pool[2 * SORT_TILE];
+    __shared__ u32 tile_start[RADIX];
+    __shared__ u32 sums[SORT_WAVES];
+    volatile u16* wcnt = reinterpret_cast<volatile u16*>(pool);  // [SORT_WAVES][RADIX]
+    u32* skey = pool;
+    u32* sval = pool + SORT_TILE;
+    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const u64 lt_mask = (1ull << lane) - 1ull;
+    const u32 lt_lo = (u32)lt_mask, lt_hi = (u32)(lt_mask >> 32);
+    u32 key[SORT_ITEMS], val[SORT_ITEMS], rnk[SORT_ITEMS];
+#pragma unroll
+    for (u32 j = 0; j < SORT_ITEMS; ++j) {
+        const u32 i = w * SORT_WAVE_SPAN + j * 64 + lane;
+        key[j] = i < n ? kin[i] : 0xFFFFFFFFu;
+        val[j] = i < n ? vin[i] : 0u;
+    }
+    if (late.table) {
+#pragma unroll
+        for (u32 j = 0; j < SORT_ITEMS; ++j) {
+            const u32 i = w * SORT_WAVE_SPAN + j * 64 + lane;
+            if (i < n && key[j] == late.marker) key[j] = late.table[late.index[i] & 0x7FFFFFFFu].z;
+        }
+    }
+    for (u32 p = 0; p < passes; ++p) {
+        const u32 shift = p * BITS;
+        if (p > 0) {  // the order the previous pass left in LDS
+            __syncthreads();
+#pragma unroll
+            for (u32 j = 0; j < SORT_ITEMS; ++j) {
+                const u32 i = w * SORT_WAVE_SPAN + j * 64 + lane;
+                key[j] = i < n ? skey[i] : 0xFFFFFFFFu;
+                val[j] = i < n ? sval[i] : 0u;
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (u32 x = 0; x < SORT_WAVES * RADIX / 2 / SORT_BLOCK; ++x) pool[x * SORT_BLOCK + tid] = 0;
+        __syncthreads();
+#pragma unroll
+        for (u32 j = 0; j < SORT_ITEMS; ++j) {
+            const bool valid = w * SORT_WAVE_SPAN + j * 64 + lane < n;
+            const u32 d = (key[j] >> shift) & (RADIX - 1u);
+            const u64 vm = __builtin_amdgcn_ballot_w64(valid);
+            u32 plo = (u32)vm, phi = (u32)(vm >> 32);
+#pragma unroll
+            for (u32 b = 0; b < BITS; ++b) {
+                const u32 bit = (d >> b) & 1u;
+                const u64 m = __builtin_amdgcn_ballot_w64(bit != 0u);
+                const u32 flip = bit - 1u;
+                plo &= (u32)m ^ flip;
+                phi &= (u32)(m >> 32) ^ flip;
+            }
+            const u32 before = (u32)__popc(plo & lt_lo) + (u32)__popc(phi & lt_hi);
+            const u32 npeers = (u32)__popc(plo) + (u32)__popc(phi);
+            u32 running = 0;
+            if (valid) {
+                running = wcnt[w * RADIX + d];
+                if (before == 0) wcnt[w * RADIX + d] = (u16)(running + npeers);
+            }
+            rnk[j] = running + before;
+        }
+        __syncthreads();
+        u32 tile_count = 0;
+        if (tid < RADIX) {
+            u32 run = 0;
+#pragma unroll
+            for (u32 x = 0; x < SORT_WAVES; ++x) {
+                const u32 c = wcnt[x * RADIX + tid];
+                wcnt[x * RADIX + tid] = (u16)run;
+                run += c;
+            }
+            tile_count = run;
+        }
+        const u32 local_start = scan_block_exclusive(tile_count, tid, sums);
+        if (tid < RADIX) tile_start[tid] = local_start;
+        __syncthreads();
+        u32 place[SORT_ITEMS];
+#pragma unroll
+        for (u32 j = 0; j < SORT_ITEMS; ++j) {
+            const u32 d = (key[j] >> shift) & (RADIX - 1u);
+            place[j] = tile_start[d] + wcnt[w * RADIX + d] + rnk[j];
+        }
+        __syncthreads();
+        if (p + 1 < passes) {
+#pragma unroll
+            for (u32 j = 0; j < SORT_ITEMS; ++j)
+                if (w * SORT_WAVE_SPAN + j * 64 + lane < n) {
+                    skey[place[j]] = key[j];
+                    sval[place[j]] = val[j];
+                }
+        } else {  // places of the last pass are positions of the output
+#pragma unroll
+            for (u32 j = 0; j < SORT_ITEMS; ++j)
+                if (w * SORT_WAVE_SPAN + j * 64 + lane < n) {
+                    kout[place[j]] = key[j];
+                    vout[place[j]] = val[j];
+                }
+        }
+    }
+}
+
 size_t tiles_of(size_t n) { return (n + SORT_TILE - 1) / SORT_TILE; }
 
 template <bool LOOKBACK>
@@ -458,7 +570,20 @@ hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, uint32_t* 
     plan->n = (u32)n;
     plan->n_tiles = n_tiles;
     plan->passes = passes;
+    plan->digit_passes = passes;
     plan->bits = bits;
+    plan->one_tile = n_tiles == 1;
+    plan->uses_head = !plan->one_tile;
+    plan->late = SortLateKeys{0u, nullptr, nullptr};
+    if (late) plan->late = *late;
+    if (plan->one_tile) {  // everything happens in the one sort_pass call
+        plan->passes = 1;
+        plan->lookback = false;
+        plan->totals = nullptr;
+        plan->status = nullptr;
+        plan->rows = 0;
+        return hipSuccess;
+    }
     plan->lookback = n_tiles <= LOOKBACK_TILES;
     plan->totals = head + HEAD_TOTALS;
     plan->status = words + OFF_ROWS;
@@ -479,6 +604,24 @@ hipError_t sort_pass(const SortPlan& plan, unsigned p, const uint32_t* kin, cons
                      uint32_t* kout, uint32_t* vout, uint32_t* err_flag, hipStream_t s) {
     if (plan.n == 0) return hipSuccess;
     if (p >= plan.passes) return hipErrorInvalidValue;
+    if (plan.one_tile) {
+        switch (plan.bits) {
+            case 8:
+                sort_one_tile_kernel<8><<<1, SORT_BLOCK, 0, s>>>(kin, vin, kout, vout, plan.n,
+                                                                 plan.digit_passes, plan.late);
+                break;
+            case 9:
+                sort_one_tile_kernel<9><<<1, SORT_BLOCK, 0, s>>>(kin, vin, kout, vout, plan.n,
+                                                                 plan.digit_passes, plan.late);
+                break;
+            case 10:
+                sort_one_tile_kernel<10><<<1, SORT_BLOCK, 0, s>>>(kin, vin, kout, vout, plan.n,
+                                                                  plan.digit_passes, plan.late);
+                break;
+            default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     const u32 shift = plan.bits * p;
     u32* totals = plan.totals + p * PASS_TOTALS;
     if (plan.lookback) {

@@ -208,19 +208,25 @@ size_t sort_pairs_temp_bytes(size_t n);
 size_t sort_pairs_head_bytes();
 // The same sort step by step (sort_begin counts, then sort_pass places digit p = 0 .. passes-1,
 // alternating between the two buffer pairs), for callers that time or interleave the launches.
-struct SortPlan {
-    uint32_t n, n_tiles, passes, bits;
-    bool lookback;  // one launch per pass (inputs of up to 2^20 pairs) or three
-    uint32_t* totals;
-    uint32_t* status;
-    size_t rows;
-};
-// late (may be null): every keys[i] equal to late->marker is first replaced, in `keys` too, by
-// late->table[late->index[i]].z.
+// late (may be null): every keys[i] equal to late->marker is first replaced (for inputs of more
+// than one tile in `keys` too) by late->table[late->index[i]].z.
 struct SortLateKeys {
     uint32_t marker;
     const uint32_t* index;
     const uint4* table;
+};
+struct SortPlan {
+    uint32_t n, n_tiles, bits;
+    uint32_t passes;        // sort_pass calls to make
+    uint32_t digit_passes;  // digit passes; all of them happen in one call when the input is one tile
+    bool one_tile;          // up to 4096 pairs: one launch sorts them in LDS; sort_begin launches
+                            // nothing, and the sort uses neither half of the head (`uses_head`)
+    bool uses_head;         // the caller alternates `parity` only over the sorts that do
+    bool lookback;          // otherwise: one launch per pass (up to 2^20 pairs) or three
+    uint32_t* totals;
+    uint32_t* status;
+    size_t rows;
+    SortLateKeys late;
 };
 hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys, size_t n,
                       unsigned end_bit, SortPlan* plan, hipStream_t s,
