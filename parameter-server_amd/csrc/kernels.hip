@@ -1095,6 +1095,7 @@ hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const u
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads, part_val) && vec4_ok(t, win_val);
     const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
+    if (g.n_chunks <= 1) return hipSuccess;  // no border, no run across one
     const u32 n_windows = window_count(g.n_chunks);
     dim3 grid((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per chunk
     if (v4)
