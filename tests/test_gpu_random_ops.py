@@ -35,7 +35,8 @@ def test_random_operation_sequences(ps, orc, wl, seed):
     dim = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 31, 32, 64, 100, 128, 257]))
     opt = OPTS[seed % 4]
     exact_dups = opt["optimizer"] in (0, 1)
-    cap = int(rng.integers(3000, 20000))
+    big = seed % 6 == 5                   # batches of several sort tiles (one tile = 4096 keys)
+    cap = int(rng.integers(60000, 150000)) if big else int(rng.integers(3000, 20000))
     dense = seed >= 24
     lf = 0.9 if dense else 0.0
     t = ps.Table(dim, capacity=cap, track_increment=True, max_load_factor=lf, **opt)
@@ -58,7 +59,7 @@ def test_random_operation_sequences(ps, orc, wl, seed):
         op = rng.choice(["push", "push", "push", "queue_store", "set", "pull", "pull_insert", "erase",
                          "erase_if", "for_each", "for_each_write", "dump_load", "increment",
                          "push_no_insert"])
-        n = int(rng.integers(1, 4000))
+        n = int(rng.integers(1, 40000 if big else 4000))
         if op in ("push", "push_no_insert"):
             q = batch(n)
             g = grads(q.size)
