@@ -22,6 +22,7 @@ namespace {
 constexpr size_t BULK_CHUNK_BYTES = 32u << 20;  // staging granule of load / dump
 constexpr uint32_t MAX_DIM = 16384;
 constexpr size_t MAX_PUSH_BATCH = (1u << 30) - 1;  // the sort's tile counters hold 30 bits
+constexpr size_t SMALL_HOST_BYTES = 1u << 20;       // host-pointer calls up to this size are staged
 
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
@@ -100,7 +101,10 @@ struct pshbm_table {
 
     // staging of the host-pointer entry points
     std::mutex st_mu;
-    DevBuf st_keys, st_vals, st_out, st_hit, st_raw;
+    DevBuf st_keys, st_vals, st_out, st_raw;
+    // small host-pointer calls go through this pinned buffer: one copy each way instead of the
+    // runtime's handling of pageable memory, which costs more than the kernel for a few KB
+    void* h_small = nullptr;
 
     // for-each / erase scratch: per-row flags, per-tile counts, row lists, reduction partials;
     // device and pinned copies of {erased, rows left, holes} and of the for-each result
@@ -419,6 +423,11 @@ int32_t set_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_values
     return PSHBM_OK;
 }
 
+int32_t ensure_small(pshbm_table* t) {
+    if (!t->h_small) HIP_TRY(t, hipHostMalloc(&t->h_small, SMALL_HOST_BYTES + 4096, hipHostMallocDefault));
+    return PSHBM_OK;
+}
+
 int32_t ensure_bulk(pshbm_table* t) {
     if (t->pin[0]) return PSHBM_OK;
     for (int k = 0; k < 2; ++k) {
@@ -434,7 +443,7 @@ void destroy_impl(pshbm_table* t) {
     DeviceGuard g(t->device);
     (void)hipDeviceSynchronize();
     DevBuf* bufs[] = {&t->ws_slot, &t->ws_row, &t->ws_idx,  &t->ws_srow, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
-                      &t->ws_pval, &t->ws_wrow, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_hit,  &t->st_raw,
+                      &t->ws_pval, &t->ws_wrow, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_raw,
                       &t->ms_dead, &t->ms_tiles, &t->ms_lists, &t->ms_fe,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
@@ -456,6 +465,7 @@ void destroy_impl(pshbm_table* t) {
     if (t->d_info) (void)hipFree(t->d_info);
     if (t->h_info) (void)hipHostFree(t->h_info);
     if (t->h_fe) (void)hipHostFree(t->h_fe);
+    if (t->h_small) (void)hipHostFree(t->h_small);
     if (t->order_ev) (void)hipEventDestroy(t->order_ev);
     for (hipEvent_t e : t->prof_ev) (void)hipEventDestroy(e);
     if (t->stream) (void)hipStreamDestroy(t->stream);
@@ -675,16 +685,29 @@ int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_ro
     if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "pull: reserved key in batch");
     DeviceGuard g(t->device);
     std::lock_guard<std::mutex> sl(t->st_mu);
-    const size_t out_bytes = n * (size_t)t->d.dim * 4;
-    ST_TRY(ensure(t, t->st_keys, n * 8));
-    ST_TRY(ensure(t, t->st_out, out_bytes));
-    ST_TRY(ensure(t, t->st_hit, n));
+    const size_t key_bytes = n * 8, out_bytes = n * (size_t)t->d.dim * 4;
+    ST_TRY(ensure(t, t->st_keys, key_bytes));
+    ST_TRY(ensure(t, t->st_out, out_bytes + n));  // the hit mask follows the rows
     hipStream_t s = t->stream;
-    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, n * 8, hipMemcpyHostToDevice, s));
-    ST_TRY(pshbm_pull_dev(t, static_cast<const uint64_t*>(t->st_keys.p), n,
-                          static_cast<float*>(t->st_out.p), static_cast<uint8_t*>(t->st_hit.p), flags, s));
-    HIP_TRY(t, hipMemcpyAsync(out_rows, t->st_out.p, out_bytes, hipMemcpyDeviceToHost, s));
-    if (hit) HIP_TRY(t, hipMemcpyAsync(hit, t->st_hit.p, n, hipMemcpyDeviceToHost, s));
+    float* d_rows = static_cast<float*>(t->st_out.p);
+    uint8_t* d_hit = static_cast<uint8_t*>(t->st_out.p) + out_bytes;
+    const size_t key_room = round_up(key_bytes, 256);
+    if (key_room + out_bytes + n <= SMALL_HOST_BYTES) {
+        ST_TRY(ensure_small(t));
+        char* h = static_cast<char*>(t->h_small);
+        std::memcpy(h, keys, key_bytes);
+        HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, h, key_bytes, hipMemcpyHostToDevice, s));
+        ST_TRY(pshbm_pull_dev(t, static_cast<const uint64_t*>(t->st_keys.p), n, d_rows, d_hit, flags, s));
+        HIP_TRY(t, hipMemcpyAsync(h + key_room, d_rows, out_bytes + n, hipMemcpyDeviceToHost, s));
+        HIP_TRY(t, hipStreamSynchronize(s));
+        std::memcpy(out_rows, h + key_room, out_bytes);
+        if (hit) std::memcpy(hit, h + key_room + out_bytes, n);
+        return PSHBM_OK;
+    }
+    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, key_bytes, hipMemcpyHostToDevice, s));
+    ST_TRY(pshbm_pull_dev(t, static_cast<const uint64_t*>(t->st_keys.p), n, d_rows, d_hit, flags, s));
+    HIP_TRY(t, hipMemcpyAsync(out_rows, d_rows, out_bytes, hipMemcpyDeviceToHost, s));
+    if (hit) HIP_TRY(t, hipMemcpyAsync(hit, d_hit, n, hipMemcpyDeviceToHost, s));
     HIP_TRY(t, hipStreamSynchronize(s));
     return PSHBM_OK;
 }
@@ -701,6 +724,28 @@ int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_gr
     return push_locked(t, d_keys, d_grads, n, flags, static_cast<hipStream_t>(stream));
 }
 
+// Keys and their n x `floats` values from host memory into st_keys / st_vals; small batches take
+// the pinned buffer and one copy. The caller holds st_mu.
+static int32_t stage_keys_values(pshbm_table* t, const uint64_t* keys, const float* vals, size_t n,
+                                 size_t floats, hipStream_t s) {
+    const size_t key_bytes = n * 8, val_bytes = n * floats * 4;
+    const size_t key_room = round_up(key_bytes, 256);
+    ST_TRY(ensure(t, t->st_keys, key_bytes));
+    ST_TRY(ensure(t, t->st_vals, val_bytes));
+    if (key_room + val_bytes <= SMALL_HOST_BYTES) {
+        ST_TRY(ensure_small(t));
+        char* h = static_cast<char*>(t->h_small);
+        std::memcpy(h, keys, key_bytes);
+        std::memcpy(h + key_room, vals, val_bytes);
+        HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, h, key_bytes, hipMemcpyHostToDevice, s));
+        HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, h + key_room, val_bytes, hipMemcpyHostToDevice, s));
+        return PSHBM_OK;
+    }
+    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, key_bytes, hipMemcpyHostToDevice, s));
+    HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, vals, val_bytes, hipMemcpyHostToDevice, s));
+    return PSHBM_OK;
+}
+
 int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, size_t n, uint32_t flags) {
     if (!t) return PSHBM_INVALID_ID;
     if (n == 0) return PSHBM_OK;
@@ -708,12 +753,8 @@ int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, siz
     if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "push: reserved key in batch");
     DeviceGuard g(t->device);
     std::lock_guard<std::mutex> sl(t->st_mu);
-    const size_t gbytes = n * (size_t)t->d.dim * 4;
-    ST_TRY(ensure(t, t->st_keys, n * 8));
-    ST_TRY(ensure(t, t->st_vals, gbytes));
     hipStream_t s = t->stream;
-    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, n * 8, hipMemcpyHostToDevice, s));
-    HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, grads, gbytes, hipMemcpyHostToDevice, s));
+    ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s));
     int32_t st = pshbm_push_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
                                 static_cast<const float*>(t->st_vals.p), n, flags, s);
     HIP_TRY(t, hipStreamSynchronize(s));
@@ -817,12 +858,8 @@ int32_t pshbm_queue(pshbm_table* t, const uint64_t* keys, const float* grads, si
     if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "queue: reserved key in batch");
     DeviceGuard g(t->device);
     std::lock_guard<std::mutex> sl(t->st_mu);
-    const size_t gbytes = n * (size_t)t->d.dim * 4;
-    ST_TRY(ensure(t, t->st_keys, n * 8));
-    ST_TRY(ensure(t, t->st_vals, gbytes));
     hipStream_t s = t->stream;
-    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, n * 8, hipMemcpyHostToDevice, s));
-    HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, grads, gbytes, hipMemcpyHostToDevice, s));
+    ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s));
     int32_t st = pshbm_queue_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
                                  static_cast<const float*>(t->st_vals.p), n, s);
     HIP_TRY(t, hipStreamSynchronize(s));
@@ -874,12 +911,8 @@ int32_t pshbm_set(pshbm_table* t, const uint64_t* keys, const float* values, siz
     if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "set: reserved key in batch");
     DeviceGuard g(t->device);
     std::lock_guard<std::mutex> sl(t->st_mu);
-    const size_t vbytes = n * (size_t)t->d.vf * 4;
-    ST_TRY(ensure(t, t->st_keys, n * 8));
-    ST_TRY(ensure(t, t->st_vals, vbytes));
     hipStream_t s = t->stream;
-    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, n * 8, hipMemcpyHostToDevice, s));
-    HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, values, vbytes, hipMemcpyHostToDevice, s));
+    ST_TRY(stage_keys_values(t, keys, values, n, t->d.vf, s));
     int32_t st = pshbm_set_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
                                static_cast<const float*>(t->st_vals.p), n, s);
     HIP_TRY(t, hipStreamSynchronize(s));
