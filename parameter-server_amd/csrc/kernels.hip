@@ -22,15 +22,6 @@ __device__ __forceinline__ float vadd(float a, float b) { return a + b; }
 __device__ __forceinline__ float4 vadd(float4 a, float4 b) {
     return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
 }
-__device__ __forceinline__ float vshfl(float v, u32 src) { return __shfl(v, (int)src); }
-__device__ __forceinline__ float4 vshfl(float4 v, u32 src) {
-    return make_float4(__shfl(v.x, (int)src), __shfl(v.y, (int)src), __shfl(v.z, (int)src),
-                       __shfl(v.w, (int)src));
-}
-__device__ __forceinline__ float vshfl_up(float v, u32 d) { return __shfl_up(v, d); }
-__device__ __forceinline__ float4 vshfl_up(float4 v, u32 d) {
-    return make_float4(__shfl_up(v.x, d), __shfl_up(v.y, d), __shfl_up(v.z, d), __shfl_up(v.w, d));
-}
 // n / d for n*d < 2^32 by one multiply: m = ceil(2^32 / d) (d == 1 handled by m = 2^32).
 __device__ __forceinline__ u32 div_small(u32 n, u64 m) { return (u32)(((u64)n * m) >> 32); }
 // n / d for any 64-bit n by one multiply-high: m = ceil(2^64 / d), d >= 2.
