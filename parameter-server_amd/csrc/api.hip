@@ -3,6 +3,7 @@
 #include "../../include/pshbm.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -101,10 +102,22 @@ struct pshbm_table {
 
     // staging of the host-pointer entry points
     std::mutex st_mu;
-    DevBuf st_keys, st_vals, st_out, st_raw;
+    DevBuf st_keys, st_vals, st_raw;
     // small host-pointer calls go through this pinned buffer: one copy each way instead of the
     // runtime's handling of pageable memory, which costs more than the kernel for a few KB
     void* h_small = nullptr;
+    // Host-pointer pulls of different threads share the table (SparsePullOperator.h:188-192): each
+    // takes one of these lanes -- a stream with its own staging -- so that their copies and
+    // kernels overlap instead of queueing behind one staging buffer.
+    struct PullLane {
+        std::mutex mu;
+        hipStream_t stream = nullptr;
+        DevBuf keys, out;
+        void* h_small = nullptr;
+    };
+    static constexpr unsigned PULL_LANES = 4;  // the reference's server runs 4 client-facing threads
+    PullLane lanes[PULL_LANES];
+    std::atomic<unsigned> next_lane{0};
 
     // for-each / erase scratch: per-row flags, per-tile counts, row lists, reduction partials;
     // device and pinned copies of {erased, rows left, holes} and of the for-each result
@@ -443,7 +456,7 @@ void destroy_impl(pshbm_table* t) {
     DeviceGuard g(t->device);
     (void)hipDeviceSynchronize();
     DevBuf* bufs[] = {&t->ws_slot, &t->ws_row, &t->ws_idx,  &t->ws_srow, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
-                      &t->ws_pval, &t->ws_wrow, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_out,  &t->st_raw,
+                      &t->ws_pval, &t->ws_wrow, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_raw,
                       &t->ms_dead, &t->ms_tiles, &t->ms_lists, &t->ms_fe,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
@@ -466,6 +479,12 @@ void destroy_impl(pshbm_table* t) {
     if (t->h_info) (void)hipHostFree(t->h_info);
     if (t->h_fe) (void)hipHostFree(t->h_fe);
     if (t->h_small) (void)hipHostFree(t->h_small);
+    for (pshbm_table::PullLane& l : t->lanes) {
+        if (l.keys.p) (void)hipFree(l.keys.p);
+        if (l.out.p) (void)hipFree(l.out.p);
+        if (l.h_small) (void)hipHostFree(l.h_small);
+        if (l.stream) (void)hipStreamDestroy(l.stream);
+    }
     if (t->order_ev) (void)hipEventDestroy(t->order_ev);
     for (hipEvent_t e : t->prof_ev) (void)hipEventDestroy(e);
     if (t->stream) (void)hipStreamDestroy(t->stream);
@@ -630,6 +649,7 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_hist), 17 * 8, hipHostMallocDefault));
     CREATE_TRY(hipStreamCreateWithFlags(&t->stream, hipStreamNonBlocking));
     CREATE_TRY(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));
+    for (pshbm_table::PullLane& l : t->lanes) CREATE_TRY(hipStreamCreateWithFlags(&l.stream, hipStreamNonBlocking));
     CREATE_TRY(hipEventCreateWithFlags(&t->order_ev, hipEventDisableTiming));
     CREATE_TRY(hipMemsetAsync(d.slots, 0xFF, t->slots_bytes, t->stream));
     CREATE_TRY(hipMemsetAsync(d.counters, 0, CNT_WORDS * 4, t->stream));
@@ -684,28 +704,47 @@ int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_ro
     if (!keys || !out_rows) return fail(t, PSHBM_ERROR, "pull: null buffer");
     if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "pull: reserved key in batch");
     DeviceGuard g(t->device);
-    std::lock_guard<std::mutex> sl(t->st_mu);
+    // a lane that is free, else the next one in turn
+    const unsigned first = t->next_lane.fetch_add(1, std::memory_order_relaxed) % pshbm_table::PULL_LANES;
+    pshbm_table::PullLane* lane = nullptr;
+    std::unique_lock<std::mutex> ll;
+    for (unsigned k = 0; k < pshbm_table::PULL_LANES && !lane; ++k) {
+        pshbm_table::PullLane& c = t->lanes[(first + k) % pshbm_table::PULL_LANES];
+        std::unique_lock<std::mutex> trial(c.mu, std::try_to_lock);
+        if (trial.owns_lock()) {
+            lane = &c;
+            ll = std::move(trial);
+        }
+    }
+    if (!lane) {
+        lane = &t->lanes[first];
+        ll = std::unique_lock<std::mutex>(lane->mu);
+    }
     const size_t key_bytes = n * 8, out_bytes = n * (size_t)t->d.dim * 4;
-    ST_TRY(ensure(t, t->st_keys, key_bytes));
-    ST_TRY(ensure(t, t->st_out, out_bytes + n));  // the hit mask follows the rows
-    hipStream_t s = t->stream;
-    float* d_rows = static_cast<float*>(t->st_out.p);
-    uint8_t* d_hit = static_cast<uint8_t*>(t->st_out.p) + out_bytes;
+    ST_TRY(ensure(t, lane->keys, key_bytes));
+    ST_TRY(ensure(t, lane->out, out_bytes + n));  // the hit mask follows the rows
+    hipStream_t s = lane->stream;
+    const uint64_t* d_keys = static_cast<const uint64_t*>(lane->keys.p);
+    float* d_rows = static_cast<float*>(lane->out.p);
+    uint8_t* d_hit = static_cast<uint8_t*>(lane->out.p) + out_bytes;
     const size_t key_room = round_up(key_bytes, 256);
     if (key_room + out_bytes + n <= SMALL_HOST_BYTES) {
-        ST_TRY(ensure_small(t));
-        char* h = static_cast<char*>(t->h_small);
+        if (!lane->h_small)
+            HIP_TRY(t, hipHostMalloc(&lane->h_small, SMALL_HOST_BYTES + 4096, hipHostMallocDefault));
+        // The kernel reads the keys from the pinned buffer and writes rows and hit mask into it:
+        // page-locked host memory is mapped into the device's address space, and for a few
+        // hundred KB the link's latency inside one kernel is cheaper than two copy commands.
+        char* h = static_cast<char*>(lane->h_small);
         std::memcpy(h, keys, key_bytes);
-        HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, h, key_bytes, hipMemcpyHostToDevice, s));
-        ST_TRY(pshbm_pull_dev(t, static_cast<const uint64_t*>(t->st_keys.p), n, d_rows, d_hit, flags, s));
-        HIP_TRY(t, hipMemcpyAsync(h + key_room, d_rows, out_bytes + n, hipMemcpyDeviceToHost, s));
+        ST_TRY(pshbm_pull_dev(t, reinterpret_cast<const uint64_t*>(h), n, reinterpret_cast<float*>(h + key_room),
+                              reinterpret_cast<uint8_t*>(h + key_room + out_bytes), flags, s));
         HIP_TRY(t, hipStreamSynchronize(s));
         std::memcpy(out_rows, h + key_room, out_bytes);
         if (hit) std::memcpy(hit, h + key_room + out_bytes, n);
         return PSHBM_OK;
     }
-    HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, key_bytes, hipMemcpyHostToDevice, s));
-    ST_TRY(pshbm_pull_dev(t, static_cast<const uint64_t*>(t->st_keys.p), n, d_rows, d_hit, flags, s));
+    HIP_TRY(t, hipMemcpyAsync(lane->keys.p, keys, key_bytes, hipMemcpyHostToDevice, s));
+    ST_TRY(pshbm_pull_dev(t, d_keys, n, d_rows, d_hit, flags, s));
     HIP_TRY(t, hipMemcpyAsync(out_rows, d_rows, out_bytes, hipMemcpyDeviceToHost, s));
     if (hit) HIP_TRY(t, hipMemcpyAsync(hit, d_hit, n, hipMemcpyDeviceToHost, s));
     HIP_TRY(t, hipStreamSynchronize(s));
@@ -724,25 +763,36 @@ int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_gr
     return push_locked(t, d_keys, d_grads, n, flags, static_cast<hipStream_t>(stream));
 }
 
-// Keys and their n x `floats` values from host memory into st_keys / st_vals; small batches take
-// the pinned buffer and one copy. The caller holds st_mu.
+// Keys and their n x `floats` values from host memory to where kernels on stream s can read them:
+// *dk / *dv. Larger batches are copied into st_keys / st_vals. Small ones are copied into the pinned
+// buffer and, when `mapped_ok`, read from there by the kernels themselves (page-locked memory is
+// mapped into the device's address space; the buffer is the caller's until the stream has been
+// waited for). The caller holds st_mu.
 static int32_t stage_keys_values(pshbm_table* t, const uint64_t* keys, const float* vals, size_t n,
-                                 size_t floats, hipStream_t s) {
+                                 size_t floats, hipStream_t s, bool mapped_ok, const uint64_t** dk,
+                                 const float** dv) {
     const size_t key_bytes = n * 8, val_bytes = n * floats * 4;
     const size_t key_room = round_up(key_bytes, 256);
-    ST_TRY(ensure(t, t->st_keys, key_bytes));
-    ST_TRY(ensure(t, t->st_vals, val_bytes));
-    if (key_room + val_bytes <= SMALL_HOST_BYTES) {
+    const bool small = key_room + val_bytes <= SMALL_HOST_BYTES;
+    if (small) {
         ST_TRY(ensure_small(t));
         char* h = static_cast<char*>(t->h_small);
         std::memcpy(h, keys, key_bytes);
         std::memcpy(h + key_room, vals, val_bytes);
-        HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, h, key_bytes, hipMemcpyHostToDevice, s));
-        HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, h + key_room, val_bytes, hipMemcpyHostToDevice, s));
-        return PSHBM_OK;
+        if (mapped_ok) {
+            *dk = reinterpret_cast<const uint64_t*>(h);
+            *dv = reinterpret_cast<const float*>(h + key_room);
+            return PSHBM_OK;
+        }
+        keys = reinterpret_cast<const uint64_t*>(h);
+        vals = reinterpret_cast<const float*>(h + key_room);
     }
+    ST_TRY(ensure(t, t->st_keys, key_bytes));
+    ST_TRY(ensure(t, t->st_vals, val_bytes));
     HIP_TRY(t, hipMemcpyAsync(t->st_keys.p, keys, key_bytes, hipMemcpyHostToDevice, s));
     HIP_TRY(t, hipMemcpyAsync(t->st_vals.p, vals, val_bytes, hipMemcpyHostToDevice, s));
+    *dk = static_cast<const uint64_t*>(t->st_keys.p);
+    *dv = static_cast<const float*>(t->st_vals.p);
     return PSHBM_OK;
 }
 
@@ -754,9 +804,10 @@ int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, siz
     DeviceGuard g(t->device);
     std::lock_guard<std::mutex> sl(t->st_mu);
     hipStream_t s = t->stream;
-    ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s));
-    int32_t st = pshbm_push_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
-                                static_cast<const float*>(t->st_vals.p), n, flags, s);
+    const uint64_t* dk = nullptr;
+    const float* dv = nullptr;
+    ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s, true, &dk, &dv));
+    int32_t st = pshbm_push_dev(t, dk, dv, n, flags, s);
     HIP_TRY(t, hipStreamSynchronize(s));
     return st;
 }
@@ -859,9 +910,10 @@ int32_t pshbm_queue(pshbm_table* t, const uint64_t* keys, const float* grads, si
     DeviceGuard g(t->device);
     std::lock_guard<std::mutex> sl(t->st_mu);
     hipStream_t s = t->stream;
-    ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s));
-    int32_t st = pshbm_queue_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
-                                 static_cast<const float*>(t->st_vals.p), n, s);
+    const uint64_t* dk = nullptr;
+    const float* dv = nullptr;
+    ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s, false, &dk, &dv));  // the queue copies device to device
+    int32_t st = pshbm_queue_dev(t, dk, dv, n, s);
     HIP_TRY(t, hipStreamSynchronize(s));
     return st;
 }
@@ -912,9 +964,10 @@ int32_t pshbm_set(pshbm_table* t, const uint64_t* keys, const float* values, siz
     DeviceGuard g(t->device);
     std::lock_guard<std::mutex> sl(t->st_mu);
     hipStream_t s = t->stream;
-    ST_TRY(stage_keys_values(t, keys, values, n, t->d.vf, s));
-    int32_t st = pshbm_set_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
-                               static_cast<const float*>(t->st_vals.p), n, s);
+    const uint64_t* dk = nullptr;
+    const float* dv = nullptr;
+    ST_TRY(stage_keys_values(t, keys, values, n, t->d.vf, s, true, &dk, &dv));
+    int32_t st = pshbm_set_dev(t, dk, dv, n, s);
     HIP_TRY(t, hipStreamSynchronize(s));
     return st;
 }
