@@ -824,12 +824,20 @@ static int32_t stage_pairs(pshbm_table* t, const void* pairs, size_t n, size_t s
         std::memcpy(&k, p + i * stride, 8);
         if (k >= KEY_DELETED) return fail(t, PSHBM_ERROR, "%s: reserved key in batch", what);
     }
-    ST_TRY(ensure(t, t->st_raw, n * stride));
     ST_TRY(ensure(t, t->st_keys, n * 8));
     ST_TRY(ensure(t, t->st_vals, n * (size_t)t->d.dim * 4));
     hipStream_t s = t->stream;
-    HIP_TRY(t, hipMemcpyAsync(t->st_raw.p, pairs, n * stride, hipMemcpyHostToDevice, s));
-    HIP_TRY(t, launch_unpack_records(static_cast<const uint32_t*>(t->st_raw.p), n,
+    const uint32_t* raw = nullptr;
+    if (n * stride <= SMALL_HOST_BYTES) {  // the split kernel reads the pairs from mapped pinned memory
+        ST_TRY(ensure_small(t));
+        std::memcpy(t->h_small, pairs, n * stride);
+        raw = static_cast<const uint32_t*>(t->h_small);
+    } else {
+        ST_TRY(ensure(t, t->st_raw, n * stride));
+        HIP_TRY(t, hipMemcpyAsync(t->st_raw.p, pairs, n * stride, hipMemcpyHostToDevice, s));
+        raw = static_cast<const uint32_t*>(t->st_raw.p);
+    }
+    HIP_TRY(t, launch_unpack_records(raw, n,
                                      (uint32_t)(stride / 4), t->d.dim,
                                      static_cast<uint64_t*>(t->st_keys.p),
                                      static_cast<float*>(t->st_vals.p), s));
