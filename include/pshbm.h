@@ -273,6 +273,14 @@ int32_t pshbm_erase_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, uint64
  * themselves once the markers fill an eighth of the slots. */
 int32_t pshbm_compact(pshbm_table* t);
 
+/* Grows the table to hold expected_max_items keys (no effect if it holds as many already): new
+ * arrays, the rows copied with their numbers, the hash array rebuilt from the stored keys. This is
+ * the rehash a growing hash map of the reference does by itself inside an insert (safe_insert,
+ * KVShardStorage.h:786-802, where a failed growth marks the storage unhealthy); here the operator
+ * decides when, typically on PSHBM_OUT_OF_MEMORY from a push. While it runs the device holds the old
+ * and the new arrays; OUT_OF_MEMORY leaves the table as it was. */
+int32_t pshbm_reserve(pshbm_table* t, uint64_t expected_max_items);
+
 /* ---- increment -----------------------------------------------------------------------------
  * The reference copies every value that a push or a store writes into a second storage, the
  * increment (safe_set(*incr_ht, ...), pico-ps/operator/SparsePushOperator.h:253-266,394-407), which

@@ -112,6 +112,7 @@ def lib():
         L.pso_for_each_write.argtypes = [vp, vp, vp, C.POINTER(C.c_uint64)]
         L.pso_erase_if.argtypes = [vp, vp, C.POINTER(C.c_uint64)]
         L.pso_erase.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_uint64)]
+        L.pso_reserve.argtypes = [vp, C.c_uint64]
         L.pso_increment_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pso_take_increment.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_size_t)]
         L.pso_clear.argtypes = [vp]
@@ -250,6 +251,9 @@ class Oracle:
 
     def compact(self):
         return OK
+
+    def reserve(self, capacity):
+        return lib().pso_reserve(self._h, capacity)
 
     def clear(self):
         return lib().pso_clear(self._h)

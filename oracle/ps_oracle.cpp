@@ -564,6 +564,15 @@ int32_t pso_erase(void* h, const uint64_t* keys, size_t n, uint64_t* erased) {
     return ST_OK;
 }
 
+// A growing hash map rehashes by itself (safe_insert, KVShardStorage.h:786-802); the fixed-capacity
+// model only raises its limit.
+int32_t pso_reserve(void* h, uint64_t capacity) {
+    Oracle& o = *static_cast<Oracle*>(h);
+    if (capacity > 0xFFFFFFF0ull) return ST_INVALID_CONFIG;
+    if (capacity > o.c.capacity) o.c.capacity = capacity;
+    return ST_OK;
+}
+
 // IncrementStorage::read_storage + the sync operator's walk of it (service/IncrementStorage.h:29-36,
 // operator/SyncOperator.h:185-266): the {key, value} records of the keys pushes wrote since the
 // last take, then the increment is empty. Too little room: ST_ERROR, *n_out = records needed.

@@ -31,7 +31,7 @@ SYMBOLS = [
     "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
     "pshbm_queue", "pshbm_queue_dev", "pshbm_queue_pairs", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
     "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
-    "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact",
+    "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
@@ -186,6 +186,7 @@ def lib():
         L.pshbm_erase.argtypes = [vp, vp, sz, C.POINTER(C.c_uint64)]
         L.pshbm_erase_dev.argtypes = [vp, vp, sz, C.POINTER(C.c_uint64), vp]
         L.pshbm_compact.argtypes = [vp]
+        L.pshbm_reserve.argtypes = [vp, C.c_uint64]
         L.pshbm_increment_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pshbm_take_increment.argtypes = [vp, vp, sz, C.POINTER(sz)]
         L.pshbm_clear.argtypes = [vp]
@@ -382,6 +383,10 @@ class Table:
 
     def compact(self):
         return lib().pshbm_compact(self._h)
+
+    def reserve(self, capacity):
+        """Grows the table to hold `capacity` keys; status."""
+        return lib().pshbm_reserve(self._h, capacity)
 
     def clear(self):
         return lib().pshbm_clear(self._h)

@@ -1302,6 +1302,84 @@ int32_t pshbm_take_increment(pshbm_table* t, void* records, size_t capacity_reco
     return dump_range(t, 0, marked, records, static_cast<const uint32_t*>(t->ms_lists.p));
 }
 
+int32_t pshbm_reserve(pshbm_table* t, uint64_t expected_max_items) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (expected_max_items > 0xFFFFFFF0ull)
+        return fail(t, PSHBM_INVALID_CONFIG, "reserve: at most 2^32-16 keys");
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    if (expected_max_items <= t->d.max_rows) return PSHBM_OK;
+    hipStream_t s = t->stream;
+    ST_TRY(begin_op(t, s));
+    ST_TRY(read_counters(t, s));  // waits for everything queued on the table so far
+    const uint32_t rows = t->h_counters[CNT_ROWS];
+    const uint64_t max_rows = expected_max_items;
+    uint64_t want_slots = (uint64_t)((double)max_rows / t->cfg.max_load_factor) + 1;
+    uint64_t nb = 16;
+    while (nb * 4 < want_slots) nb <<= 1;
+    if (nb * 4 > (1ull << 31)) return fail(t, PSHBM_INVALID_CONFIG, "reserve: the table would need more than 2^31 slots");
+    const size_t stride = t->d.stride_f;
+    const size_t slots_bytes = nb * 64, rows_bytes = max_rows * stride * 4, keys_bytes = max_rows * 8;
+    const size_t dirty_bytes = round_up(max_rows, 4);
+    uint4* n_slots = nullptr;
+    float* n_rows = nullptr;
+    uint64_t* n_keys = nullptr;
+    uint8_t* n_dirty = nullptr;
+    auto undo = [&](hipError_t e, const char* what) {
+        if (n_slots) (void)hipFree(n_slots);
+        if (n_rows) (void)hipFree(n_rows);
+        if (n_keys) (void)hipFree(n_keys);
+        if (n_dirty) (void)hipFree(n_dirty);
+        return hip_fail(t, e, what);
+    };
+    hipError_t e;
+    if ((e = hipMalloc(reinterpret_cast<void**>(&n_slots), slots_bytes)) != hipSuccess) return undo(e, "reserve: hash array");
+    if ((e = hipMalloc(reinterpret_cast<void**>(&n_rows), rows_bytes)) != hipSuccess) return undo(e, "reserve: rows");
+    if ((e = hipMalloc(reinterpret_cast<void**>(&n_keys), keys_bytes)) != hipSuccess) return undo(e, "reserve: row keys");
+    if (t->d.dirty && (e = hipMalloc(reinterpret_cast<void**>(&n_dirty), dirty_bytes)) != hipSuccess)
+        return undo(e, "reserve: marks");
+    // rows keep their numbers: the slab is copied as it is and the hash array rebuilt from row_keys
+    if ((e = hipMemsetAsync(n_slots, 0xFF, slots_bytes, s)) != hipSuccess) return undo(e, "reserve: fill");
+    if (rows) {
+        if ((e = hipMemcpyAsync(n_rows, t->d.rows, (size_t)rows * stride * 4, hipMemcpyDeviceToDevice, s)) != hipSuccess)
+            return undo(e, "reserve: copy rows");
+        if ((e = hipMemcpyAsync(n_keys, t->d.row_keys, (size_t)rows * 8, hipMemcpyDeviceToDevice, s)) != hipSuccess)
+            return undo(e, "reserve: copy keys");
+    }
+    if (n_dirty) {
+        if ((e = hipMemsetAsync(n_dirty, 0, dirty_bytes, s)) != hipSuccess) return undo(e, "reserve: marks");
+        if (rows && (e = hipMemcpyAsync(n_dirty, t->d.dirty, rows, hipMemcpyDeviceToDevice, s)) != hipSuccess)
+            return undo(e, "reserve: copy marks");
+    }
+    if ((e = hipStreamSynchronize(s)) != hipSuccess) return undo(e, "reserve: copy");
+    uint4* o_slots = t->d.slots;
+    float* o_rows = t->d.rows;
+    uint64_t* o_keys = t->d.row_keys;
+    uint8_t* o_dirty = t->d.dirty;
+    t->d.slots = n_slots;
+    t->d.rows = n_rows;
+    t->d.row_keys = n_keys;
+    t->d.dirty = n_dirty;
+    t->d.bucket_mask = (uint32_t)(nb - 1);
+    t->d.max_rows = (uint32_t)max_rows;
+    t->nbuckets = nb;
+    t->slots_bytes = slots_bytes;
+    t->rows_bytes = rows_bytes;
+    t->keys_bytes = keys_bytes;
+    t->cfg.expected_max_items = max_rows;
+    t->row_bits = 1;
+    while ((1ull << t->row_bits) <= max_rows) ++t->row_bits;
+    t->tombstones = 0;
+    (void)hipFree(o_slots);
+    (void)hipFree(o_rows);
+    (void)hipFree(o_keys);
+    if (o_dirty) (void)hipFree(o_dirty);
+    HIP_TRY(t, launch_reinsert(t->d, rows, s));
+    ST_TRY(read_counters(t, s));
+    if (t->h_counters[CNT_OVERFLOW]) return fail(t, PSHBM_FATAL, "reserve: the hash array overflowed");
+    return PSHBM_OK;
+}
+
 int32_t pshbm_clear(pshbm_table* t) {
     if (!t) return PSHBM_INVALID_ID;
     DeviceGuard g(t->device);

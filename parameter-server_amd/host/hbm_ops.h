@@ -31,8 +31,8 @@
 namespace pshbm_host {
 
 // op_config keys of an HBM table: dim, optimizer (sum|sgd|adagrad|ftrl), lr, init_acc, alpha, beta,
-// l1, l2, hbm_table.expected_max_items, hbm_table.max_load_factor, hbm_table.max_batch, read_only,
-// device. The learning rate lives in the operator config, as pico-ps/operator/Operator.h:55 expects.
+// l1, l2, hbm_table.expected_max_items, hbm_table.grow_limit, hbm_table.max_load_factor,
+// hbm_table.max_batch, hbm_table.track_increment, read_only, device. The learning rate lives in the operator config, as pico-ps/operator/Operator.h:55 expects.
 inline pshbm_config table_config(const Configure& c) {
     pshbm_config cfg{};
     cfg.struct_size = sizeof(cfg);
@@ -83,6 +83,7 @@ public:
             return false;
         }
         _shards[shard_id] = t;
+        _capacity[shard_id] = cfg.expected_max_items;
         _vf = pshbm_value_floats(cfg.dim, cfg.optimizer);
         _dim = cfg.dim;
         return true;
@@ -92,6 +93,22 @@ public:
         if (it == _shards.end()) return false;
         pshbm_destroy(it->second);
         _shards.erase(it);
+        return true;
+    }
+    // A hash map of the reference grows inside the insert that needs the room (safe_insert,
+    // KVShardStorage.h:786-802) until the memory limit makes it unhealthy; a table grows when an
+    // operator finds it full: twice the capacity at a time, up to op_config
+    // `hbm_table.grow_limit` keys (0, the default: never). False = no room to be had.
+    bool grow(int32_t shard_id) {
+        const uint64_t limit = (uint64_t)_config.number("hbm_table.grow_limit", 0);
+        pshbm_table* t = get(shard_id);
+        if (!t || _capacity[shard_id] >= limit) return false;
+        const uint64_t want = std::min<uint64_t>(limit, _capacity[shard_id] * 2);
+        if (pshbm_reserve(t, want) != PSHBM_OK) {
+            _error = pshbm_last_error(t);
+            return false;
+        }
+        _capacity[shard_id] = want;
         return true;
     }
     void clear() {  // KVShardStorage.h:902-908: every shard emptied, the shards stay
@@ -130,6 +147,7 @@ public:
 private:
     Configure _config;
     std::map<int32_t, pshbm_table*> _shards;
+    std::map<int32_t, uint64_t> _capacity;  // keys each shard's table holds at most
     uint32_t _dim = 0, _vf = 0;
     std::string _error;
 };
@@ -230,8 +248,10 @@ public:
     void apply_async_push_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, Storage* /*incr_storage*/,
                                   PSResponse& resp) {
         Status status;
-        for_each_block(rt, req, storage, [&](pshbm_table* t, const std::vector<char>& block, int32_t n, size_t stride) {
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        for_each_block(rt, req, storage, [&](int32_t shard_id, pshbm_table* t, const std::vector<char>& block, int32_t n, size_t stride) {
             int32_t rc = pshbm_push_pairs(t, block.data(), n, stride, 0);
+            while (rc == PSHBM_OUT_OF_MEMORY && st.grow(shard_id)) rc = pshbm_push_pairs(t, block.data(), n, stride, 0);
             if (rc == PSHBM_OUT_OF_MEMORY) status = Status::OOM(pshbm_last_error(t));
             else if (rc != PSHBM_OK) status = Status::Error(pshbm_last_error(t));
         });
@@ -244,7 +264,7 @@ public:
     // apply_sync_push_request, :278-320: blocks are queued, nothing is merged or applied yet.
     void apply_sync_push_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp) {
         Status status;
-        for_each_block(rt, req, storage, [&](pshbm_table* t, const std::vector<char>& block, int32_t n, size_t stride) {
+        for_each_block(rt, req, storage, [&](int32_t, pshbm_table* t, const std::vector<char>& block, int32_t n, size_t stride) {
             if (pshbm_queue_pairs(t, block.data(), n, stride) != PSHBM_OK) status = Status::Error(pshbm_last_error(t));
         });
         resp = PSResponse(req);
@@ -286,7 +306,7 @@ private:
                 std::vector<char> ar;
                 ps_deserialize(req.lazy(), ar);
                 PSHBM_SCHECK(ar.size() == (size_t)shard_items_num * stride, "push block size mismatch");
-                f(t, ar, shard_items_num, stride);
+                f(shard_id, t, ar, shard_items_num, stride);
             }
         }
     }

@@ -320,6 +320,55 @@ static void test_dense(const std::string& dir) {
     EXPECT(threw);
 }
 
+// A storage created for 64 keys takes 1000: the push that finds the table full grows it (twice the
+// capacity at a time, up to hbm_table.grow_limit) and is applied again; past the limit the response
+// carries Status::OOM, as the reference's does once its memory limit is reached
+// (pico-ps/operator/SparsePullOperator.h:245-253).
+static void test_growth() {
+    Configure op_config;
+    op_config.set("dim", 2);
+    op_config.set("optimizer", "sum");
+    op_config.set("hbm_table.expected_max_items", 64);
+    op_config.set("hbm_table.grow_limit", 700);
+    RuntimeInfo rt(0, {0, 1});
+    HbmStorageOperator storage_op(op_config);
+    std::unique_ptr<Storage> storage = storage_op.create_storage(rt, 0);
+    HbmSparsePushOperator push_op(op_config);
+    HbmSparsePullOperator pull_op(op_config);
+    std::vector<uint64_t> keys;
+    std::vector<float> args;
+    for (int k = 0; k < 1000; ++k) {
+        keys.push_back(k);
+        args.push_back((float)k);
+    }
+    PSResponse resp;
+    Status status;
+    PSRequest a = make_push_request(keys, args);  // 500 keys per shard: 64 -> 128 -> 256 -> 512
+    push_op.apply_async_push_request(rt, a, storage.get(), nullptr, resp);
+    resp >> status;
+    EXPECT(status.ok());
+    auto* hst = static_cast<HbmShardStorage*>(storage.get());
+    EXPECT(hst->shard_size(0) == 500 && hst->shard_size(1) == 500);
+    bool ok;
+    auto v = pull(pull_op, rt, storage.get(), keys, &ok);
+    EXPECT(ok);
+    for (size_t i = 0; i < keys.size(); ++i) EXPECT(v[i * 2] == (float)keys[i] && v[i * 2 + 1] == 1.0f);
+    // 800 more keys: 400 per shard do not fit under the limit of 700
+    std::vector<uint64_t> more;
+    std::vector<float> margs;
+    for (int k = 1000; k < 1800; ++k) {
+        more.push_back(k);
+        margs.push_back(1.0f);
+    }
+    PSRequest b = make_push_request(more, margs);
+    PSResponse resp2;
+    push_op.apply_async_push_request(rt, b, storage.get(), nullptr, resp2);
+    Status status2;
+    resp2 >> status2;
+    EXPECT(status2.IsOOM() && resp2.error_code() == RpcErrorCodeType::ELOGICERROR);
+    EXPECT(hst->shard_size(0) == 500 && hst->shard_size(1) == 500);
+}
+
 int main(int argc, char** argv) {
     const std::string dir = argc > 1 ? argv[1] : "/tmp";
     Configure op_config;
@@ -647,6 +696,7 @@ int main(int argc, char** argv) {
     }
 
     test_dense(dir);
+    test_growth();
     if (g_failed) {
         std::printf("FAILED: %d expectation(s)\n", g_failed);
         return 1;

@@ -579,3 +579,34 @@ def test_largest_rows(ps, orc, wl, opt, dim):
     assert t2.load(rec, ps.LOAD_UNIQUE) == 0
     np.testing.assert_array_equal(np.sort(t2.dump()[1], order="key"), np.sort(rec, order="key"))
     t.close(), t2.close()
+
+
+@pytest.mark.parametrize("opt,dim", [("sgd", 16), ("ftrl", 6), ("adagrad", 64)])
+def test_reserve_grows_a_full_table(ps, orc, wl, opt, dim):
+    """A table that refuses a batch for lack of room takes it after pshbm_reserve; keys, values,
+    marks and the order of the slab survive the move, erased slots' markers do not."""
+    rng = np.random.default_rng(77)
+    cap = 3000
+    t, r = pair(ps, orc, dim, opt, capacity=cap, track_increment=True)
+    keys = wl.table_keys_np(0, 20000, seed=4)
+    g = rng.integers(-3, 4, (20000, dim)).astype(np.float32)
+    assert t.push(keys[:2500], g[:2500]) == 0 and r.push(keys[:2500], g[:2500]) == 0
+    assert t.erase(keys[:400]) == r.erase(keys[:400])
+    before = t.dump()[1]
+    assert t.push(keys[2500:6000], g[2500:6000]) == ps.OUT_OF_MEMORY == r.push(keys[2500:6000], g[2500:6000])
+    np.testing.assert_array_equal(t.dump()[1], before)            # all or nothing
+    assert t.reserve(100) == 0 and t.stats().capacity == cap      # never shrinks
+    assert t.reserve(12000) == 0 and r.reserve(12000) == 0
+    s = t.stats()
+    assert s.capacity == 12000 and s.size == 2100 and sum(s.probe_hist) == 2100
+    np.testing.assert_array_equal(t.dump()[1], before)            # same slab, same order
+    assert t.push(keys[2500:6000], g[2500:6000]) == 0 and r.push(keys[2500:6000], g[2500:6000]) == 0
+    assert t.push(keys[:9000], g[:9000]) == 0 and r.push(keys[:9000], g[:9000]) == 0
+    assert_same_table(t, r, exact=True)
+    a, b = t.take_increment(), r.take_increment()
+    np.testing.assert_array_equal(np.sort(a[1], order="key"), np.sort(b[1], order="key"))
+    a, b = t.pull(keys[:12000]), r.pull(keys[:12000])
+    np.testing.assert_array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+    np.testing.assert_array_equal(a[2], b[2])
+    assert t.reserve(1 << 33) == ps.INVALID_CONFIG
+    t.close()

@@ -1,7 +1,7 @@
 """Random operation sequences on the HIP path and the oracle side by side (needs an MI355X).
 
 Each case draws a table shape (dim, optimizer) and a sequence of pulls, pushes, queued pushes and
-stores, sets, erases, erase-ifs, for-eachs, dump / load round trips and increment takes, with
+stores, sets, erases, erase-ifs, for-eachs, dump / load round trips, growth and increment takes, with
 gradients that are small integers (times a power of two for the optimizers with a learning rate)
 so that duplicate sums are exact and every value can be compared bit for bit after every step --
 except under FTRL and Adagrad, whose steps are not exact; those cases push distinct keys only.
@@ -58,7 +58,7 @@ def test_random_operation_sequences(ps, orc, wl, seed):
     for step in range(14):
         op = rng.choice(["push", "push", "push", "queue_store", "set", "pull", "pull_insert", "erase",
                          "erase_if", "for_each", "for_each_write", "dump_load", "increment",
-                         "push_no_insert"])
+                         "push_no_insert", "reserve"])
         n = int(rng.integers(1, 40000 if big else 4000))
         if op in ("push", "push_no_insert"):
             q = batch(n)
@@ -121,6 +121,9 @@ def test_random_operation_sequences(ps, orc, wl, seed):
             t.close()
             t = t2
             r.take_increment()                       # a fresh table has no marks
+        elif op == "reserve":
+            cap = cap + int(rng.integers(0, cap // 4 + 2))
+            assert t.reserve(cap) == 0 and r.reserve(cap) == 0
         elif op == "increment":
             a, b = t.take_increment(), r.take_increment()
             assert a[0] == b[0] == 0
