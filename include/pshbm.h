@@ -276,7 +276,7 @@ int32_t pshbm_compact(pshbm_table* t);
 /* Grows the table to hold expected_max_items keys (no effect if it holds as many already): new
  * arrays, the rows copied with their numbers, the hash array rebuilt from the stored keys. This is
  * the rehash a growing hash map of the reference does by itself inside an insert (safe_insert,
- * KVShardStorage.h:786-802, where a failed growth marks the storage unhealthy); here the operator
+ * KVShardStorage.h:791-801, where a failed growth marks the storage unhealthy); here the operator
  * decides when, typically on PSHBM_OUT_OF_MEMORY from a push. While it runs the device holds the old
  * and the new arrays; OUT_OF_MEMORY leaves the table as it was. */
 int32_t pshbm_reserve(pshbm_table* t, uint64_t expected_max_items);

@@ -564,7 +564,7 @@ int32_t pso_erase(void* h, const uint64_t* keys, size_t n, uint64_t* erased) {
     return ST_OK;
 }
 
-// A growing hash map rehashes by itself (safe_insert, KVShardStorage.h:786-802); the fixed-capacity
+// A growing hash map rehashes by itself (safe_insert, KVShardStorage.h:791-801); the fixed-capacity
 // model only raises its limit.
 int32_t pso_reserve(void* h, uint64_t capacity) {
     Oracle& o = *static_cast<Oracle*>(h);

@@ -96,7 +96,7 @@ public:
         return true;
     }
     // A hash map of the reference grows inside the insert that needs the room (safe_insert,
-    // KVShardStorage.h:786-802) until the memory limit makes it unhealthy; a table grows when an
+    // KVShardStorage.h:791-801) until the memory limit makes it unhealthy; a table grows when an
     // operator finds it full: twice the capacity at a time, up to op_config
     // `hbm_table.grow_limit` keys (0, the default: never). False = no room to be had.
     bool grow(int32_t shard_id) {
