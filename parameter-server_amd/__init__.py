@@ -36,7 +36,7 @@ SYMBOLS = [
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
-          "fixup_windows", "assign_rows"]
+          "fixup_windows", "assign_rows", "push_small"]
 
 
 class Config(C.Structure):

@@ -378,6 +378,12 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
     bool checked = false;
     uint32_t rows_before = 0;
     if (insert) ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
+    // A small batch is bound by launches: one workgroup does the whole push in one. (Not when the
+    // table is nearly full: undoing a batch that does not fit needs the separate steps.)
+    if (!unique && !checked && n <= push_small_max()) {
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_PUSH_SMALL, launch_push_small(t->d, d_keys, d_grads, n, insert, s));
+        return PSHBM_OK;
+    }
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
     uint32_t* idx = static_cast<uint32_t*>(t->ws_idx.p);
     // Everything after the probe works on row ids: they are dense, so the sort needs fewer bits

@@ -103,6 +103,113 @@ __global__ __launch_bounds__(BLOCK) void gather_slots_kernel(TableDev t,
 }
 
 // ---- locate / claim ------------------------------------------------------------------------
+struct Located {
+    u32 slot;  // slot of the key, SLOT_NONE if it is neither stored nor claimable
+    u32 row;   // its row; ROW_PENDING if the slot was claimed in this launch (by this call or another)
+    bool won;  // this call claimed the slot
+    bool dup;  // the key was there already, or another call of this launch claimed it
+};
+
+// Four lanes (sub = 0..3 of group grp) find `key` or claim a slot for it. Every lane of the
+// wavefront must call this; lanes whose `active` is false only take part in the ballots.
+// need_row: also fetch the row word where the key is found by the slow path.
+__device__ __forceinline__ Located find_or_claim(const TableDev& t, u64 key, bool active, u32 grp,
+                                                 u32 sub, bool need_row) {
+    Located r{SLOT_NONE, ROW_NONE, false, false};
+    // Most keys of a batch are stored already: look for them with ordinary cached loads first.
+    // What those loads show may be older than this launch, never wrong: a key that is seen is
+    // stored (slots only go from empty to a key), and a key that is not seen is dealt with below.
+    const Found f = probe_find(t, key, active, grp, sub);
+    if (f.slot != SLOT_NONE) {
+        r.slot = f.slot;
+        r.row = f.row < t.max_rows ? f.row : ROW_PENDING;
+        r.dup = true;
+    }
+    bool done = !active || f.slot != SLOT_NONE;
+    u32 b = (u32)hash64(key) & t.bucket_mask;
+    u32 steps = 0;
+    // A key that is not seen goes straight for the first slot that looked empty. The view may be
+    // old, but only in one direction (slots go from empty to a key and stay), so the first slot
+    // that is truly empty is not before this one, and a copy of the key that another group stored
+    // during this launch is either seen, or in this slot, or behind a slot that looked empty and
+    // is not -- the compare-and-swap tells which: it finds the slot empty (claimed), holding the
+    // key (a repeat), or holding another key (then the bucket is looked at again, with loads that
+    // bypass the caches).
+    if (__ballot(!done)) {
+        const bool try_it = !done && f.empty != SLOT_NONE;
+        u64 old = 0;
+        if (try_it && sub == 0)
+            old = atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[f.empty]),
+                            (unsigned long long)KEY_EMPTY, (unsigned long long)key);
+        const u64 oldb = shfl64(old, grp * 4);
+        if (try_it) {
+            b = f.empty >> 2;  // the buckets before it are full and stay full
+            if (oldb == KEY_EMPTY || oldb == key) {
+                r.slot = f.empty;
+                r.row = ROW_PENDING;
+                r.won = oldb == KEY_EMPTY;
+                r.dup = !r.won;
+                done = true;
+            }
+        }
+    }
+    while (__ballot(!done)) {
+        u64 skey = 0;
+        u32 srow = ROW_NONE;
+        // Coherent at the device level: a slot claimed by another compute unit during this
+        // launch must be seen, so the loads bypass the per-CU cache.
+        if (!done) {
+            uint4* sp = &t.slots[(u64)b * 4 + sub];
+            skey = __hip_atomic_load(reinterpret_cast<u64*>(sp), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (need_row)
+                srow = __hip_atomic_load(reinterpret_cast<u32*>(sp) + 2, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+        }
+        const bool match = !done && skey == key;
+        const bool empty = !done && skey == KEY_EMPTY;
+        const u32 m4 = (u32)(__ballot(match) >> (grp * 4)) & 0xFu;
+        const u32 e4 = (u32)(__ballot(empty) >> (grp * 4)) & 0xFu;
+        const u32 tgt = e4 ? (u32)__ffs((int)e4) - 1u : 0u;
+        const bool do_cas = !done && !m4 && e4 && sub == tgt;
+        u64 old = 0;
+        if (do_cas)
+            old = atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[(u64)b * 4 + tgt]),
+                            (unsigned long long)KEY_EMPTY, (unsigned long long)key);
+        const u64 oldb = shfl64(old, grp * 4 + tgt);
+        const u32 msub = m4 ? (u32)__ffs((int)m4) - 1u : 0u;
+        const u32 mrow = __shfl(srow, (int)(grp * 4 + msub));
+        if (!done) {
+            if (m4) {
+                r.slot = b * 4 + msub;
+                // a key that another group claimed in this launch has no row yet
+                r.row = mrow < t.max_rows ? mrow : ROW_PENDING;
+                r.dup = true;
+                done = true;
+            } else if (e4) {
+                if (oldb == KEY_EMPTY) {
+                    r.slot = b * 4 + tgt;
+                    r.row = ROW_PENDING;
+                    r.won = true;
+                    done = true;
+                } else if (oldb == key) {  // the same key, claimed by another group
+                    r.slot = b * 4 + tgt;
+                    r.row = ROW_PENDING;
+                    r.dup = true;
+                    done = true;
+                }
+                // otherwise another key took the slot: look at this bucket again
+            } else {
+                b = (b + 1) & t.bucket_mask;
+                if (++steps > t.bucket_mask) {
+                    done = true;
+                    if (sub == 0) t.counters[CNT_OVERFLOW] = 1u;
+                }
+            }
+        }
+    }
+    return r;
+}
+
 template <bool kInsert>
 __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __restrict__ keys,
                                                         u32 n, u32* __restrict__ slot_out,
@@ -135,100 +242,10 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
             row = f.row;
             dup = f.slot != SLOT_NONE;
         } else {
-            // Most keys of a batch are stored already: look for them with ordinary cached loads
-            // first. What those loads show may be older than this launch, never wrong: a key that
-            // is seen is stored (slots only go from empty to a key), and a key that is not seen
-            // is looked for again below, with loads that bypass the caches.
-            Found f = probe_find(t, key, active, grp, sub);
-            if (f.slot != SLOT_NONE) {
-                slot = f.slot;
-                row = f.row < t.max_rows ? f.row : ROW_PENDING;
-                dup = true;
-            }
-            bool won = false;
-            bool done = !active || f.slot != SLOT_NONE;
-            u32 b = (u32)hash64(key) & t.bucket_mask;
-            u32 steps = 0;
-            // A key that is not seen goes straight for the first slot that looked empty. The view
-            // may be old, but only in one direction (slots go from empty to a key and stay), so the
-            // first slot that is truly empty is not before this one, and a copy of the key that
-            // another group stored during this launch is either seen, or in this slot, or behind
-            // a slot that looked empty and is not -- the compare-and-swap tells which: it finds
-            // the slot empty (claimed), holding the key (a repeat), or holding another key (then
-            // the bucket is looked at again, with loads that bypass the caches).
-            if (__ballot(!done)) {
-                const bool try_it = !done && f.empty != SLOT_NONE;
-                u64 old = 0;
-                if (try_it && sub == 0)
-                    old = atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[f.empty]),
-                                    (unsigned long long)KEY_EMPTY, (unsigned long long)key);
-                const u64 oldb = shfl64(old, grp * 4);
-                if (try_it) {
-                    b = f.empty >> 2;  // the buckets before it are full and stay full
-                    if (oldb == KEY_EMPTY || oldb == key) {
-                        slot = f.empty;
-                        row = ROW_PENDING;
-                        won = oldb == KEY_EMPTY;
-                        dup = !won;
-                        done = true;
-                    }
-                }
-            }
-            while (__ballot(!done)) {
-                u64 skey = 0;
-                u32 srow = ROW_NONE;
-                // Coherent at the device level: a slot claimed by another compute unit during
-                // this launch must be seen, so the loads bypass the per-CU cache.
-                if (!done) {
-                    uint4* sp = &t.slots[(u64)b * 4 + sub];
-                    skey = __hip_atomic_load(reinterpret_cast<u64*>(sp), __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT);
-                    if (row_out)
-                        srow = __hip_atomic_load(reinterpret_cast<u32*>(sp) + 2, __ATOMIC_RELAXED,
-                                                 __HIP_MEMORY_SCOPE_AGENT);
-                }
-                bool match = !done && skey == key;
-                bool empty = !done && skey == KEY_EMPTY;
-                u32 m4 = (u32)(__ballot(match) >> (grp * 4)) & 0xFu;
-                u32 e4 = (u32)(__ballot(empty) >> (grp * 4)) & 0xFu;
-                u32 tgt = e4 ? (u32)__ffs((int)e4) - 1u : 0u;
-                bool do_cas = !done && !m4 && e4 && sub == tgt;
-                u64 old = 0;
-                if (do_cas)
-                    old = atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[(u64)b * 4 + tgt]),
-                                    (unsigned long long)KEY_EMPTY, (unsigned long long)key);
-                u64 oldb = shfl64(old, grp * 4 + tgt);
-                const u32 msub = m4 ? (u32)__ffs((int)m4) - 1u : 0u;
-                const u32 mrow = __shfl(srow, (int)(grp * 4 + msub));
-                if (!done) {
-                    if (m4) {
-                        slot = b * 4 + msub;
-                        // a key that another group claimed in this launch has no row yet
-                        row = mrow < t.max_rows ? mrow : ROW_PENDING;
-                        dup = true;
-                        done = true;
-                    } else if (e4) {
-                        if (oldb == KEY_EMPTY) {
-                            slot = b * 4 + tgt;
-                            row = ROW_PENDING;
-                            won = true;
-                            done = true;
-                        } else if (oldb == key) {  // the same key, claimed by another group
-                            slot = b * 4 + tgt;
-                            row = ROW_PENDING;
-                            dup = true;
-                            done = true;
-                        }
-                        // otherwise another key took the slot: look at this bucket again
-                    } else {
-                        b = (b + 1) & t.bucket_mask;
-                        if (++steps > t.bucket_mask) {
-                            done = true;
-                            if (sub == 0) t.counters[CNT_OVERFLOW] = 1u;
-                        }
-                    }
-                }
-            }
+            const Located l = find_or_claim(t, key, active, grp, sub, row_out != nullptr);
+            slot = l.slot;
+            row = l.row;
+            dup = l.dup;
             // The group that claimed the slot only marks it and counts itself in its 1024-key
             // block: rows are handed out afterwards by assign_rows_kernel. (One shared row counter
             // bumped from here costs a device-scope atomic on one address per wavefront, which
@@ -237,11 +254,11 @@ __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __
             // after the other, about 120 ns each, and the 1024 keys of a block are probed at about
             // the same time. The 16 keys of a round lie in one block: one addition per wavefront.)
             static_assert(ASSIGN_KEYS % KEYS_PER_ROUND == 0, "a round's keys share a block");
-            const u64 wm = __ballot(won && sub == 0);
+            const u64 wm = __ballot(l.won && sub == 0);
             if (wm) {
                 if (lane == (u32)__ffsll((unsigned long long)wm) - 1u)
                     atomicAdd(&won_count[base / ASSIGN_KEYS], (u32)__popcll(wm));
-                if (won && sub == 0) slot |= WON_BIT;
+                if (l.won && sub == 0) slot |= WON_BIT;
             }
         }
         if (inb && sub == 0) {
@@ -841,6 +858,192 @@ __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* _
     if (lane_on && g == 0) finalize<T>(t, h.z, col, units, acc);
 }
 
+// ---- a whole push in one launch, for batches of up to 1024 keys --------------------------------
+// Small batches are bound by launches, not by work, so one workgroup of 1024 threads does what the
+// chain of kernels above does: (1) four lanes per key find the key or claim a slot for it;
+// (2) thread i numbers key i's claim (a prefix sum over the workgroup), the new rows are
+// initialised and the later occurrences of a new key read its row from its slot; (3) thread i
+// ranks pair (row, i) among all pairs by comparing with every other one (n <= 1024: about a
+// thousand LDS reads) and puts it at its place -- the pairs are then sorted by row, equal rows in
+// batch order; (4) the starts of the runs of equal rows are listed; (5) groups of lanes, one lane
+// per 4 or 16 bytes of a gradient row, add up a run each in batch order and take the optimizer
+// step. A run of more than SMALL_LONG rows is added by all groups together: strided partial sums,
+// then added in group order.
+constexpr u32 SMALL_PUSH = 1024, SMALL_LONG = 32;
+
+__device__ __forceinline__ u32 block_scan_1024(u32 v, u32 tid, u32* wave_sums, u32* total) {
+    const u32 lane = tid & 63u, w = tid >> 6;
+    u32 incl = v;
+    for (u32 off = 1; off < 64; off <<= 1) {
+        const u32 o = __shfl_up(incl, off);
+        if (lane >= off) incl += o;
+    }
+    if (lane == 63) wave_sums[w] = incl;
+    __syncthreads();
+    u32 before = 0, all = 0;
+    for (u32 x = 0; x < SMALL_PUSH / 64; ++x) {
+        const u32 c = wave_sums[x];
+        if (x < w) before += c;
+        all += c;
+    }
+    *total = all;
+    __syncthreads();  // wave_sums may be used again
+    return before + incl - v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(SMALL_PUSH) void push_small_kernel(TableDev t, const u64* __restrict__ keys,
+                                                                const T* __restrict__ grads, u32 n,
+                                                                int insert, u32 units) {
+    __shared__ u32 s_slot[SMALL_PUSH], s_row[SMALL_PUSH];   // per key, batch order
+    __shared__ u32 q_row[SMALL_PUSH], q_idx[SMALL_PUSH];    // pairs sorted by (row, batch index)
+    __shared__ u32 heads[SMALL_PUSH + 1];                   // starts of the runs; heads[nruns] = their end
+    __shared__ u32 longs[SMALL_PUSH / SMALL_LONG + 1];      // runs added by the whole workgroup
+    __shared__ u32 new_rows[SMALL_PUSH];
+    __shared__ u32 wave_sums[SMALL_PUSH / 64];
+    __shared__ u32 n_long;
+    __shared__ T part[SMALL_PUSH];
+    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const u32 grp = lane >> 2, sub = lane & 3u;
+    const u32 entry = t.counters[CNT_ROWS];
+    if (tid == 0) n_long = 0;
+
+    // 1. find or claim: 256 keys per round
+    for (u32 r0 = 0; r0 < n; r0 += SMALL_PUSH / 4) {
+        const u32 i = r0 + w * KEYS_PER_ROUND + grp;
+        const bool inb = i < n;
+        const u64 key = inb ? keys[i] : KEY_EMPTY;
+        const bool active = inb && key < KEY_DELETED;
+        const u64 bm = __ballot(inb && !active && sub == 0);
+        if (bm && lane == (u32)__ffsll((unsigned long long)bm) - 1u)
+            atomicAdd(&t.counters[CNT_BADKEY], (u32)__popcll(bm));
+        u32 slot = SLOT_NONE, row = ROW_NONE;
+        if (insert) {
+            const Located l = find_or_claim(t, key, active, grp, sub, true);
+            slot = l.slot;
+            row = l.row;
+            if (l.won) slot |= WON_BIT;
+        } else {
+            const Found f = probe_find(t, key, active, grp, sub);
+            slot = f.slot;
+            row = f.row;
+        }
+        if (inb && sub == 0) {
+            s_slot[i] = slot;
+            s_row[i] = row;
+        }
+    }
+    __syncthreads();
+
+    // 2. rows for the claims, in batch order
+    const bool won = tid < n && s_slot[tid] != SLOT_NONE && (s_slot[tid] & WON_BIT);
+    u32 n_won = 0;
+    const u32 rank = block_scan_1024(won ? 1u : 0u, tid, wave_sums, &n_won);
+    if (won) {
+        const u32 rid = entry + rank;
+        const u32 slot = s_slot[tid] & ~WON_BIT;
+        s_slot[tid] = slot;
+        if (rid < t.max_rows) {
+            reinterpret_cast<u32*>(&t.slots[slot])[2] = rid;
+            t.row_keys[rid] = keys[tid];
+            s_row[tid] = rid;
+            new_rows[rank] = rid;
+        } else {  // does not fit (the host rules this out before it chooses this kernel)
+            s_row[tid] = ROW_NONE;
+            new_rows[rank] = ROW_NONE;
+        }
+    }
+    if (tid == 0 && insert) {
+        t.counters[CNT_ENTRY] = entry;
+        t.counters[CNT_ROWS] = entry + n_won;
+        if (entry + n_won > t.max_rows) t.counters[CNT_OVERFLOW] = 1u;
+    }
+    __threadfence();
+    __syncthreads();
+    if (n_won) {
+        // a later occurrence of a key claimed by this batch: the row is in the slot now
+        if (tid < n && s_row[tid] == ROW_PENDING)
+            s_row[tid] = __hip_atomic_load(reinterpret_cast<u32*>(&t.slots[s_slot[tid]]) + 2, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+        // fresh rows: zero weights, initial optimizer state
+        const u32 per = t.stride_f;
+        for (u32 e = tid; e < n_won * per; e += SMALL_PUSH) {
+            const u32 k = e / per, f = e - k * per;
+            const u32 rid = new_rows[k];
+            if (rid != ROW_NONE) t.rows[(u64)rid * per + f] = init_float(t, f);
+        }
+        __threadfence();
+        __syncthreads();
+    }
+
+    // 3. place of pair (row, i) among the pairs: those with a smaller row, or the same row earlier
+    if (tid < n) {
+        const u32 mine = s_row[tid];
+        u32 pos = 0;
+        for (u32 j = 0; j < n; ++j) {
+            const u32 o = s_row[j];
+            pos += (o < mine || (o == mine && j < tid)) ? 1u : 0u;
+        }
+        q_row[pos] = mine;
+        q_idx[pos] = tid;
+    }
+    __syncthreads();
+
+    // 4. run starts; keys that are not stored (ROW_NONE, the largest value) come last and form no run
+    const bool real = tid < n && q_row[tid] < t.max_rows;
+    const bool head = real && (tid == 0 || q_row[tid - 1] != q_row[tid]);
+    u32 nruns = 0, nreal = 0;
+    const u32 hpos = block_scan_1024(head ? 1u : 0u, tid, wave_sums, &nruns);
+    (void)block_scan_1024(real ? 1u : 0u, tid, wave_sums, &nreal);
+    if (head) heads[hpos] = tid;
+    if (tid == 0) heads[nruns] = nreal;
+    __syncthreads();
+    if (tid < nruns && heads[tid + 1] - heads[tid] > SMALL_LONG) longs[atomicAdd(&n_long, 1u)] = tid;
+    __syncthreads();
+
+    // 5. sums and optimizer steps, 64 columns (of T) at a time
+    for (u32 col0 = 0; col0 < units; col0 += 64) {
+        const u32 lp = (units - col0) < 64u ? (units - col0) : 64u;  // lanes per row
+        const u32 G = SMALL_PUSH / lp;                               // lane groups
+        const u32 g = tid / lp, c = tid - g * lp;
+        const u32 col = col0 + c;
+        if (g < G) {
+            for (u32 j = g; j < nruns; j += G) {
+                const u32 st = heads[j], en = heads[j + 1];
+                if (en - st > SMALL_LONG) continue;
+                T a0 = vzero(T()), a1 = vzero(T());
+                u32 q = st;
+                for (; q + 1 < en; q += 2) {  // two loads in flight; the order of additions is fixed
+                    const T v0 = grads[(u64)q_idx[q] * units + col];
+                    const T v1 = grads[(u64)q_idx[q + 1] * units + col];
+                    a0 = vadd(a0, v0);
+                    a1 = vadd(a1, v1);
+                }
+                if (q < en) a0 = vadd(a0, grads[(u64)q_idx[q] * units + col]);
+                finalize<T>(t, q_row[st], col, units, vadd(a0, a1));
+            }
+        }
+        const u32 nl = n_long;
+        for (u32 x = 0; x < nl; ++x) {  // workgroup-uniform
+            const u32 j = longs[x];  // in no particular order: the runs are of different rows
+            const u32 st = heads[j], en = heads[j + 1];
+            T a = vzero(T());
+            if (g < G)
+                for (u32 q = st + g; q < en; q += G) a = vadd(a, grads[(u64)q_idx[q] * units + col]);
+            __syncthreads();
+            if (g < G) part[g * lp + c] = a;
+            __syncthreads();
+            if (g == 0) {
+                T sum = vzero(T());
+                const u32 used = (en - st) < G ? (en - st) : G;
+                for (u32 y = 0; y < used; ++y) sum = vadd(sum, part[y * lp + c]);
+                finalize<T>(t, q_row[st], col, units, sum);
+            }
+        }
+        __syncthreads();
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void update_unique_kernel(TableDev t,
                                                                const u32* __restrict__ row_idx,
@@ -1096,6 +1299,20 @@ hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const u
     else
         fixup_kernel<float><<<grid, BLOCK, 0, s>>>(t, part_hdr, part_val, win_row, win_val, g.units,
                                                    g.lp, g.p, g.n_chunks, n_windows);
+    return hipGetLastError();
+}
+
+size_t push_small_max() { return SMALL_PUSH; }
+
+hipError_t launch_push_small(const TableDev& t, const u64* keys, const float* grads, size_t n, bool insert,
+                             hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    if (n > SMALL_PUSH) return hipErrorInvalidValue;
+    if (vec4_ok(t, grads))
+        push_small_kernel<float4><<<1, SMALL_PUSH, 0, s>>>(t, keys, reinterpret_cast<const float4*>(grads),
+                                                          (u32)n, insert ? 1 : 0, t.dim / 4);
+    else
+        push_small_kernel<float><<<1, SMALL_PUSH, 0, s>>>(t, keys, grads, (u32)n, insert ? 1 : 0, t.dim);
     return hipGetLastError();
 }
 

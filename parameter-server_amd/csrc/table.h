@@ -141,6 +141,12 @@ hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const u
                         const float* part_val, const uint32_t* win_row, const float* win_val,
                         hipStream_t s);
 
+// A whole push (probe and claim, rows for new keys, aggregation, update) of up to push_small_max()
+// keys in one launch of one workgroup. The caller has made sure that the new keys fit.
+size_t push_small_max();
+hipError_t launch_push_small(const TableDev& t, const uint64_t* keys, const float* grads, size_t n,
+                             bool insert, hipStream_t s);
+
 // One optimizer step per located key, no aggregation (keys distinct); rows[i] = row of key i.
 hipError_t launch_update_unique(const TableDev& t, const uint32_t* rows, size_t n,
                                 const float* grads, hipStream_t s);
