@@ -610,3 +610,28 @@ def test_reserve_grows_a_full_table(ps, orc, wl, opt, dim):
     np.testing.assert_array_equal(a[2], b[2])
     assert t.reserve(1 << 33) == ps.INVALID_CONFIG
     t.close()
+
+
+@pytest.mark.parametrize("dim", [1, 4, 16, 100, 260])
+@pytest.mark.parametrize("n", [1, 33, 257, 1000, 1024])
+def test_one_launch_push_heavy_repeats(ps, orc, dim, n):
+    """Batches of up to 1024 keys take the one-launch push: a few keys repeated hundreds of times
+    (runs added by the whole workgroup), keys that are new and repeated inside the batch, keys not
+    stored under PUSH_NO_INSERT; integer gradients, so the sums are exact in any order."""
+    rng = np.random.default_rng(dim * 1000 + n)
+    t, r = pair(ps, orc, dim, "sum", capacity=5000)
+    base = np.arange(1, 41, dtype=np.uint64) * 7919
+    assert t.set(base[:20], np.ones((20, dim), np.float32)) == 0
+    assert r.set(base[:20], np.ones((20, dim), np.float32)) == 0
+    for it in range(4):
+        hot = base[rng.integers(0, 3, n)]                         # three keys take most of the batch
+        cold = base[rng.integers(0, 40, n)]                       # stored and new ones
+        fresh = rng.integers(1 << 40, 1 << 41, n).astype(np.uint64)
+        pick = rng.random(n)
+        q = np.where(pick < 0.6, hot, np.where(pick < 0.9, cold, fresh)).astype(np.uint64)
+        q[rng.integers(0, n)] = q[0]                              # at least one repeat of a maybe-new key
+        g = rng.integers(-4, 5, (n, dim)).astype(np.float32)
+        flags = ps.PUSH_NO_INSERT if it == 2 else 0
+        assert t.push(q, g, flags) == 0 and r.push(q, g, flags) == 0
+        assert_same_table(t, r, exact=True)
+    t.close()
