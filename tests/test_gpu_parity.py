@@ -203,9 +203,10 @@ def assert_push_parity(gpu, seq, exact, multiplicity):
 
 @pytest.mark.parametrize("opt", ["sgd", "adagrad", "ftrl"])
 @pytest.mark.parametrize("dim,s", [(16, 1.05), (64, 1.2), (8, 1.1), (128, 1.1)])
-def test_push_zipf_within_tolerance(ps, orc, wl, opt, dim, s):
+@pytest.mark.parametrize("batch", [30000, 900])       # 900: the one-launch push
+def test_push_zipf_within_tolerance(ps, orc, wl, opt, dim, s, batch):
     rng = np.random.default_rng(11)
-    n_table, batch = 20000, 30000
+    n_table = 20000
     t, r = pair(ps, orc, dim, opt, capacity=n_table + 4000)
     x = orc.Oracle(dim, capacity=n_table + 4000, **OPTS[opt])   # exactly rounded aggregation
     keys = wl.table_keys_np(0, n_table, seed=2)
