@@ -320,7 +320,7 @@ int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out);
 #define PSHBM_PHASE_SORT_PASS 7     /* radix sort of (row, index): one digit pass */
 #define PSHBM_PHASE_FIXUP_WINDOWS 8 /* window sums of runs that span many chunks */
 #define PSHBM_PHASE_ASSIGN_ROWS 9   /* rows for the slots an inserting operation claimed */
-#define PSHBM_PHASE_PUSH_SMALL 10   /* a whole push of up to 1024 keys in one launch */
+#define PSHBM_PHASE_PUSH_SMALL 10   /* a whole push of a small batch in one launch */
 #define PSHBM_PHASES 12
 typedef struct pshbm_profile {
     double ms[PSHBM_PHASES];

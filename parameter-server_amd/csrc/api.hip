@@ -108,10 +108,13 @@ struct pshbm_table {
     void* h_small = nullptr;
     // Host-pointer pulls of different threads share the table (SparsePullOperator.h:188-192): each
     // takes one of these lanes -- a stream with its own staging -- so that their copies and
-    // kernels overlap instead of queueing behind one staging buffer.
+    // kernels overlap instead of queueing behind one staging buffer. Small host-pointer pushes
+    // take a lane for its pinned buffer only: their kernels run on the table's stream one after
+    // the other, but a thread waits for its own batch while the next thread's is already queued.
     struct PullLane {
         std::mutex mu;
         hipStream_t stream = nullptr;
+        hipEvent_t done = nullptr;  // small pushes: their work on the table's stream has finished
         DevBuf keys, out;
         void* h_small = nullptr;
     };
@@ -490,6 +493,7 @@ void destroy_impl(pshbm_table* t) {
         if (l.out.p) (void)hipFree(l.out.p);
         if (l.h_small) (void)hipHostFree(l.h_small);
         if (l.stream) (void)hipStreamDestroy(l.stream);
+        if (l.done) (void)hipEventDestroy(l.done);
     }
     if (t->order_ev) (void)hipEventDestroy(t->order_ev);
     for (hipEvent_t e : t->prof_ev) (void)hipEventDestroy(e);
@@ -655,7 +659,10 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_hist), 17 * 8, hipHostMallocDefault));
     CREATE_TRY(hipStreamCreateWithFlags(&t->stream, hipStreamNonBlocking));
     CREATE_TRY(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));
-    for (pshbm_table::PullLane& l : t->lanes) CREATE_TRY(hipStreamCreateWithFlags(&l.stream, hipStreamNonBlocking));
+    for (pshbm_table::PullLane& l : t->lanes) {
+        CREATE_TRY(hipStreamCreateWithFlags(&l.stream, hipStreamNonBlocking));
+        CREATE_TRY(hipEventCreateWithFlags(&l.done, hipEventDisableTiming));
+    }
     CREATE_TRY(hipEventCreateWithFlags(&t->order_ev, hipEventDisableTiming));
     CREATE_TRY(hipMemsetAsync(d.slots, 0xFF, t->slots_bytes, t->stream));
     CREATE_TRY(hipMemsetAsync(d.counters, 0, CNT_WORDS * 4, t->stream));
@@ -703,6 +710,27 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     return PSHBM_OK;
 }
 
+// A lane that is free, else the next one in turn; held until `lock` goes.
+static pshbm_table::PullLane* take_lane(pshbm_table* t, std::unique_lock<std::mutex>& lock) {
+    const unsigned first = t->next_lane.fetch_add(1, std::memory_order_relaxed) % pshbm_table::PULL_LANES;
+    for (unsigned k = 0; k < pshbm_table::PULL_LANES; ++k) {
+        pshbm_table::PullLane& c = t->lanes[(first + k) % pshbm_table::PULL_LANES];
+        std::unique_lock<std::mutex> trial(c.mu, std::try_to_lock);
+        if (trial.owns_lock()) {
+            lock = std::move(trial);
+            return &c;
+        }
+    }
+    lock = std::unique_lock<std::mutex>(t->lanes[first].mu);
+    return &t->lanes[first];
+}
+
+static int32_t lane_pinned(pshbm_table* t, pshbm_table::PullLane* lane) {
+    if (!lane->h_small)
+        HIP_TRY(t, hipHostMalloc(&lane->h_small, SMALL_HOST_BYTES + 4096, hipHostMallocDefault));
+    return PSHBM_OK;
+}
+
 int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_rows, uint8_t* hit,
                    uint32_t flags) {
     if (!t) return PSHBM_INVALID_ID;
@@ -710,22 +738,8 @@ int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_ro
     if (!keys || !out_rows) return fail(t, PSHBM_ERROR, "pull: null buffer");
     if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "pull: reserved key in batch");
     DeviceGuard g(t->device);
-    // a lane that is free, else the next one in turn
-    const unsigned first = t->next_lane.fetch_add(1, std::memory_order_relaxed) % pshbm_table::PULL_LANES;
-    pshbm_table::PullLane* lane = nullptr;
     std::unique_lock<std::mutex> ll;
-    for (unsigned k = 0; k < pshbm_table::PULL_LANES && !lane; ++k) {
-        pshbm_table::PullLane& c = t->lanes[(first + k) % pshbm_table::PULL_LANES];
-        std::unique_lock<std::mutex> trial(c.mu, std::try_to_lock);
-        if (trial.owns_lock()) {
-            lane = &c;
-            ll = std::move(trial);
-        }
-    }
-    if (!lane) {
-        lane = &t->lanes[first];
-        ll = std::unique_lock<std::mutex>(lane->mu);
-    }
+    pshbm_table::PullLane* lane = take_lane(t, ll);
     const size_t key_bytes = n * 8, out_bytes = n * (size_t)t->d.dim * 4;
     ST_TRY(ensure(t, lane->keys, key_bytes));
     ST_TRY(ensure(t, lane->out, out_bytes + n));  // the hit mask follows the rows
@@ -735,8 +749,7 @@ int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_ro
     uint8_t* d_hit = static_cast<uint8_t*>(lane->out.p) + out_bytes;
     const size_t key_room = round_up(key_bytes, 256);
     if (key_room + out_bytes + n <= SMALL_HOST_BYTES) {
-        if (!lane->h_small)
-            HIP_TRY(t, hipHostMalloc(&lane->h_small, SMALL_HOST_BYTES + 4096, hipHostMallocDefault));
+        ST_TRY(lane_pinned(t, lane));
         // The kernel reads the keys from the pinned buffer and writes rows and hit mask into it:
         // page-locked host memory is mapped into the device's address space, and for a few
         // hundred KB the link's latency inside one kernel is cheaper than two copy commands.
@@ -808,8 +821,25 @@ int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, siz
     if (!keys || !grads) return fail(t, PSHBM_ERROR, "push: null buffer");
     if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "push: reserved key in batch");
     DeviceGuard g(t->device);
-    std::lock_guard<std::mutex> sl(t->st_mu);
     hipStream_t s = t->stream;
+    const size_t key_bytes = n * 8, val_bytes = n * (size_t)t->d.dim * 4;
+    const size_t key_room = round_up(key_bytes, 256);
+    if (key_room + val_bytes <= SMALL_HOST_BYTES) {
+        // the kernels read the batch from a lane's pinned buffer; the thread waits for its own
+        // batch only, so the next thread's push is queued behind it meanwhile
+        std::unique_lock<std::mutex> ll;
+        pshbm_table::PullLane* lane = take_lane(t, ll);
+        ST_TRY(lane_pinned(t, lane));
+        char* h = static_cast<char*>(lane->h_small);
+        std::memcpy(h, keys, key_bytes);
+        std::memcpy(h + key_room, grads, val_bytes);
+        int32_t st = pshbm_push_dev(t, reinterpret_cast<const uint64_t*>(h),
+                                    reinterpret_cast<const float*>(h + key_room), n, flags, s);
+        HIP_TRY(t, hipEventRecord(lane->done, s));
+        HIP_TRY(t, hipEventSynchronize(lane->done));
+        return st;
+    }
+    std::lock_guard<std::mutex> sl(t->st_mu);
     const uint64_t* dk = nullptr;
     const float* dv = nullptr;
     ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s, true, &dk, &dv));
@@ -854,6 +884,28 @@ int32_t pshbm_push_pairs(pshbm_table* t, const void* pairs, size_t n, size_t str
     if (!t) return PSHBM_INVALID_ID;
     if (n == 0) return PSHBM_OK;
     DeviceGuard g(t->device);
+    const size_t key_room = round_up(n * 8, 256), val_bytes = n * (size_t)t->d.dim * 4;
+    if (pairs && stride >= 8 + (size_t)t->d.dim * 4 && stride % 4 == 0 && key_room + val_bytes <= SMALL_HOST_BYTES) {
+        // a small block is split into keys and gradients on its way into a lane's pinned buffer
+        std::unique_lock<std::mutex> ll;
+        pshbm_table::PullLane* lane = take_lane(t, ll);
+        ST_TRY(lane_pinned(t, lane));
+        char* h = static_cast<char*>(lane->h_small);
+        const char* p = static_cast<const char*>(pairs);
+        const size_t row_bytes = (size_t)t->d.dim * 4;
+        for (size_t i = 0; i < n; ++i) {
+            uint64_t k;
+            std::memcpy(&k, p + i * stride, 8);
+            if (k >= KEY_DELETED) return fail(t, PSHBM_ERROR, "push_pairs: reserved key in batch");
+            std::memcpy(h + i * 8, &k, 8);
+            std::memcpy(h + key_room + i * row_bytes, p + i * stride + 8, row_bytes);
+        }
+        int32_t st = pshbm_push_dev(t, reinterpret_cast<const uint64_t*>(h),
+                                    reinterpret_cast<const float*>(h + key_room), n, flags, t->stream);
+        HIP_TRY(t, hipEventRecord(lane->done, t->stream));
+        HIP_TRY(t, hipEventSynchronize(lane->done));
+        return st;
+    }
     std::lock_guard<std::mutex> sl(t->st_mu);
     ST_TRY(stage_pairs(t, pairs, n, stride, "push_pairs"));
     int32_t st = pshbm_push_dev(t, static_cast<const uint64_t*>(t->st_keys.p),

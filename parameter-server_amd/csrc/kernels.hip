@@ -858,7 +858,7 @@ __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* _
     if (lane_on && g == 0) finalize<T>(t, h.z, col, units, acc);
 }
 
-// ---- a whole push in one launch, for batches of up to 1024 keys --------------------------------
+// ---- a whole push in one launch, for small batches (the kernel takes up to 1024 keys) -----------
 // Small batches are bound by launches, not by work, so one workgroup of 1024 threads does what the
 // chain of kernels above does: (1) four lanes per key find the key or claim a slot for it;
 // (2) thread i numbers key i's claim (a prefix sum over the workgroup), the new rows are
@@ -895,7 +895,8 @@ template <typename T>
 __global__ __launch_bounds__(SMALL_PUSH) void push_small_kernel(TableDev t, const u64* __restrict__ keys,
                                                                 const T* __restrict__ grads, u32 n,
                                                                 int insert, u32 units) {
-    __shared__ u32 s_slot[SMALL_PUSH], s_row[SMALL_PUSH];   // per key, batch order
+    __shared__ u32 s_slot[SMALL_PUSH];                       // per key, batch order
+    __shared__ __align__(16) u32 s_row[SMALL_PUSH];
     __shared__ u32 q_row[SMALL_PUSH], q_idx[SMALL_PUSH];    // pairs sorted by (row, batch index)
     __shared__ u32 heads[SMALL_PUSH + 1];                   // starts of the runs; heads[nruns] = their end
     __shared__ u32 longs[SMALL_PUSH / SMALL_LONG + 1];      // runs added by the whole workgroup
@@ -977,12 +978,20 @@ __global__ __launch_bounds__(SMALL_PUSH) void push_small_kernel(TableDev t, cons
     }
 
     // 3. place of pair (row, i) among the pairs: those with a smaller row, or the same row earlier
+    // (four rows per LDS read; the entries past n hold ROW_NONE and count for nobody)
+    if (tid >= n) s_row[tid] = ROW_NONE;
+    __syncthreads();
     if (tid < n) {
         const u32 mine = s_row[tid];
+        const uint4* rows4 = reinterpret_cast<const uint4*>(s_row);
         u32 pos = 0;
-        for (u32 j = 0; j < n; ++j) {
-            const u32 o = s_row[j];
-            pos += (o < mine || (o == mine && j < tid)) ? 1u : 0u;
+#pragma unroll 4
+        for (u32 j = 0; j < n; j += 4) {
+            const uint4 o = rows4[j >> 2];
+            pos += (o.x < mine || (o.x == mine && j < tid)) ? 1u : 0u;
+            pos += (o.y < mine || (o.y == mine && j + 1 < tid)) ? 1u : 0u;
+            pos += (o.z < mine || (o.z == mine && j + 2 < tid)) ? 1u : 0u;
+            pos += (o.w < mine || (o.w == mine && j + 3 < tid)) ? 1u : 0u;
         }
         q_row[pos] = mine;
         q_idx[pos] = tid;
@@ -1302,7 +1311,10 @@ hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const u
     return hipGetLastError();
 }
 
-size_t push_small_max() { return SMALL_PUSH; }
+// One workgroup takes its keys 256 at a time, so its time grows with the batch where the chain of
+// kernels spreads over the device: the one launch wins up to about 512 keys (256 keys: 15 µs
+// against 29, 512: 25 against 30, 1024: 55 against 30).
+size_t push_small_max() { return SMALL_PUSH / 2; }
 
 hipError_t launch_push_small(const TableDev& t, const u64* keys, const float* grads, size_t n, bool insert,
                              hipStream_t s) {
