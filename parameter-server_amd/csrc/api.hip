@@ -784,27 +784,21 @@ int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_gr
 
 // Keys and their n x `floats` values from host memory to where kernels on stream s can read them:
 // *dk / *dv. Larger batches are copied into st_keys / st_vals. Small ones are copied into the pinned
-// buffer and, when `mapped_ok`, read from there by the kernels themselves (page-locked memory is
-// mapped into the device's address space; the buffer is the caller's until the stream has been
-// waited for). The caller holds st_mu.
+// buffer and read from there by the kernels themselves (page-locked memory is mapped into the
+// device's address space; the buffer is in use until the stream has been waited for). The caller
+// holds st_mu.
 static int32_t stage_keys_values(pshbm_table* t, const uint64_t* keys, const float* vals, size_t n,
-                                 size_t floats, hipStream_t s, bool mapped_ok, const uint64_t** dk,
-                                 const float** dv) {
+                                 size_t floats, hipStream_t s, const uint64_t** dk, const float** dv) {
     const size_t key_bytes = n * 8, val_bytes = n * floats * 4;
     const size_t key_room = round_up(key_bytes, 256);
-    const bool small = key_room + val_bytes <= SMALL_HOST_BYTES;
-    if (small) {
+    if (key_room + val_bytes <= SMALL_HOST_BYTES) {
         ST_TRY(ensure_small(t));
         char* h = static_cast<char*>(t->h_small);
         std::memcpy(h, keys, key_bytes);
         std::memcpy(h + key_room, vals, val_bytes);
-        if (mapped_ok) {
-            *dk = reinterpret_cast<const uint64_t*>(h);
-            *dv = reinterpret_cast<const float*>(h + key_room);
-            return PSHBM_OK;
-        }
-        keys = reinterpret_cast<const uint64_t*>(h);
-        vals = reinterpret_cast<const float*>(h + key_room);
+        *dk = reinterpret_cast<const uint64_t*>(h);
+        *dv = reinterpret_cast<const float*>(h + key_room);
+        return PSHBM_OK;
     }
     ST_TRY(ensure(t, t->st_keys, key_bytes));
     ST_TRY(ensure(t, t->st_vals, val_bytes));
@@ -842,7 +836,7 @@ int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, siz
     std::lock_guard<std::mutex> sl(t->st_mu);
     const uint64_t* dk = nullptr;
     const float* dv = nullptr;
-    ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s, true, &dk, &dv));
+    ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s, &dk, &dv));
     int32_t st = pshbm_push_dev(t, dk, dv, n, flags, s);
     HIP_TRY(t, hipStreamSynchronize(s));
     return st;
@@ -880,6 +874,21 @@ static int32_t stage_pairs(pshbm_table* t, const void* pairs, size_t n, size_t s
     return PSHBM_OK;
 }
 
+// n wire pairs {uint64 key, dim floats} split into a key array and a gradient array on the host.
+static int32_t split_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride, char* keys_out,
+                           char* grads_out, const char* what) {
+    const char* p = static_cast<const char*>(pairs);
+    const size_t row_bytes = (size_t)t->d.dim * 4;
+    for (size_t i = 0; i < n; ++i) {
+        uint64_t k;
+        std::memcpy(&k, p + i * stride, 8);
+        if (k >= KEY_DELETED) return fail(t, PSHBM_ERROR, "%s: reserved key in batch", what);
+        std::memcpy(keys_out + i * 8, &k, 8);
+        std::memcpy(grads_out + i * row_bytes, p + i * stride + 8, row_bytes);
+    }
+    return PSHBM_OK;
+}
+
 int32_t pshbm_push_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride, uint32_t flags) {
     if (!t) return PSHBM_INVALID_ID;
     if (n == 0) return PSHBM_OK;
@@ -891,16 +900,9 @@ int32_t pshbm_push_pairs(pshbm_table* t, const void* pairs, size_t n, size_t str
         pshbm_table::PullLane* lane = take_lane(t, ll);
         ST_TRY(lane_pinned(t, lane));
         char* h = static_cast<char*>(lane->h_small);
-        const char* p = static_cast<const char*>(pairs);
-        const size_t row_bytes = (size_t)t->d.dim * 4;
-        for (size_t i = 0; i < n; ++i) {
-            uint64_t k;
-            std::memcpy(&k, p + i * stride, 8);
-            if (k >= KEY_DELETED) return fail(t, PSHBM_ERROR, "push_pairs: reserved key in batch");
-            std::memcpy(h + i * 8, &k, 8);
-            std::memcpy(h + key_room + i * row_bytes, p + i * stride + 8, row_bytes);
-        }
-        int32_t st = pshbm_push_dev(t, reinterpret_cast<const uint64_t*>(h),
+        int32_t st = split_pairs(t, pairs, n, stride, h, h + key_room, "push_pairs");
+        if (st != PSHBM_OK) return st;
+        st = pshbm_push_dev(t, reinterpret_cast<const uint64_t*>(h),
                                     reinterpret_cast<const float*>(h + key_room), n, flags, t->stream);
         HIP_TRY(t, hipEventRecord(lane->done, t->stream));
         HIP_TRY(t, hipEventSynchronize(lane->done));
@@ -918,6 +920,20 @@ int32_t pshbm_queue_pairs(pshbm_table* t, const void* pairs, size_t n, size_t st
     if (!t) return PSHBM_INVALID_ID;
     if (n == 0) return PSHBM_OK;
     DeviceGuard g(t->device);
+    const size_t key_room = round_up(n * 8, 256), val_bytes = n * (size_t)t->d.dim * 4;
+    if (pairs && stride >= 8 + (size_t)t->d.dim * 4 && stride % 4 == 0 && key_room + val_bytes <= SMALL_HOST_BYTES) {
+        std::unique_lock<std::mutex> ll;
+        pshbm_table::PullLane* lane = take_lane(t, ll);
+        ST_TRY(lane_pinned(t, lane));
+        char* h = static_cast<char*>(lane->h_small);
+        int32_t st = split_pairs(t, pairs, n, stride, h, h + key_room, "queue_pairs");
+        if (st != PSHBM_OK) return st;
+        st = pshbm_queue_dev(t, reinterpret_cast<const uint64_t*>(h), reinterpret_cast<const float*>(h + key_room), n,
+                             t->stream);
+        HIP_TRY(t, hipEventRecord(lane->done, t->stream));
+        HIP_TRY(t, hipEventSynchronize(lane->done));
+        return st;
+    }
     std::lock_guard<std::mutex> sl(t->st_mu);
     ST_TRY(stage_pairs(t, pairs, n, stride, "queue_pairs"));
     int32_t st = pshbm_queue_dev(t, static_cast<const uint64_t*>(t->st_keys.p),
@@ -960,10 +976,11 @@ int32_t pshbm_queue_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_g
         t->q_keys = nk;
         t->q_grads = ng;
     }
+    // (the host-pointer entry points hand their pinned or pageable buffers straight to these copies)
     HIP_TRY(t, hipMemcpyAsync(static_cast<uint64_t*>(t->q_keys.p) + t->q_n, d_keys, n * 8,
-                              hipMemcpyDeviceToDevice, s));
+                              hipMemcpyDefault, s));
     HIP_TRY(t, hipMemcpyAsync(static_cast<char*>(t->q_grads.p) + t->q_n * gb, d_grads, n * gb,
-                              hipMemcpyDeviceToDevice, s));
+                              hipMemcpyDefault, s));
     t->q_n += n;
     return PSHBM_OK;
 }
@@ -974,12 +991,24 @@ int32_t pshbm_queue(pshbm_table* t, const uint64_t* keys, const float* grads, si
     if (!keys || !grads) return fail(t, PSHBM_ERROR, "queue: null buffer");
     if (has_reserved_key(keys, n)) return fail(t, PSHBM_ERROR, "queue: reserved key in batch");
     DeviceGuard g(t->device);
-    std::lock_guard<std::mutex> sl(t->st_mu);
     hipStream_t s = t->stream;
-    const uint64_t* dk = nullptr;
-    const float* dv = nullptr;
-    ST_TRY(stage_keys_values(t, keys, grads, n, t->d.dim, s, false, &dk, &dv));  // the queue copies device to device
-    int32_t st = pshbm_queue_dev(t, dk, dv, n, s);
+    const size_t key_bytes = n * 8, val_bytes = n * (size_t)t->d.dim * 4;
+    const size_t key_room = round_up(key_bytes, 256);
+    if (key_room + val_bytes <= SMALL_HOST_BYTES) {  // through a lane's pinned buffer, as a small push
+        std::unique_lock<std::mutex> ll;
+        pshbm_table::PullLane* lane = take_lane(t, ll);
+        ST_TRY(lane_pinned(t, lane));
+        char* h = static_cast<char*>(lane->h_small);
+        std::memcpy(h, keys, key_bytes);
+        std::memcpy(h + key_room, grads, val_bytes);
+        int32_t st = pshbm_queue_dev(t, reinterpret_cast<const uint64_t*>(h),
+                                     reinterpret_cast<const float*>(h + key_room), n, s);
+        HIP_TRY(t, hipEventRecord(lane->done, s));
+        HIP_TRY(t, hipEventSynchronize(lane->done));
+        return st;
+    }
+    std::lock_guard<std::mutex> sl(t->st_mu);
+    int32_t st = pshbm_queue_dev(t, keys, grads, n, s);  // copied from the caller's memory into the queue
     HIP_TRY(t, hipStreamSynchronize(s));
     return st;
 }
@@ -1032,7 +1061,7 @@ int32_t pshbm_set(pshbm_table* t, const uint64_t* keys, const float* values, siz
     hipStream_t s = t->stream;
     const uint64_t* dk = nullptr;
     const float* dv = nullptr;
-    ST_TRY(stage_keys_values(t, keys, values, n, t->d.vf, s, true, &dk, &dv));
+    ST_TRY(stage_keys_values(t, keys, values, n, t->d.vf, s, &dk, &dv));
     int32_t st = pshbm_set_dev(t, dk, dv, n, s);
     HIP_TRY(t, hipStreamSynchronize(s));
     return st;
