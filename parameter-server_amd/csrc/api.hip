@@ -741,12 +741,7 @@ int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_ro
     std::unique_lock<std::mutex> ll;
     pshbm_table::PullLane* lane = take_lane(t, ll);
     const size_t key_bytes = n * 8, out_bytes = n * (size_t)t->d.dim * 4;
-    ST_TRY(ensure(t, lane->keys, key_bytes));
-    ST_TRY(ensure(t, lane->out, out_bytes + n));  // the hit mask follows the rows
     hipStream_t s = lane->stream;
-    const uint64_t* d_keys = static_cast<const uint64_t*>(lane->keys.p);
-    float* d_rows = static_cast<float*>(lane->out.p);
-    uint8_t* d_hit = static_cast<uint8_t*>(lane->out.p) + out_bytes;
     const size_t key_room = round_up(key_bytes, 256);
     if (key_room + out_bytes + n <= SMALL_HOST_BYTES) {
         ST_TRY(lane_pinned(t, lane));
@@ -762,6 +757,11 @@ int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_ro
         if (hit) std::memcpy(hit, h + key_room + out_bytes, n);
         return PSHBM_OK;
     }
+    ST_TRY(ensure(t, lane->keys, key_bytes));
+    ST_TRY(ensure(t, lane->out, out_bytes + n));  // the hit mask follows the rows
+    const uint64_t* d_keys = static_cast<const uint64_t*>(lane->keys.p);
+    float* d_rows = static_cast<float*>(lane->out.p);
+    uint8_t* d_hit = static_cast<uint8_t*>(lane->out.p) + out_bytes;
     HIP_TRY(t, hipMemcpyAsync(lane->keys.p, keys, key_bytes, hipMemcpyHostToDevice, s));
     ST_TRY(pshbm_pull_dev(t, d_keys, n, d_rows, d_hit, flags, s));
     HIP_TRY(t, hipMemcpyAsync(out_rows, d_rows, out_bytes, hipMemcpyDeviceToHost, s));
@@ -842,8 +842,8 @@ int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, siz
     return st;
 }
 
-// Copies n wire pairs {uint64 key, dim floats} to the device and splits them into the staged key
-// and gradient arrays (st_keys, st_vals). The caller holds st_mu.
+// Copies n wire pairs {uint64 key, dim floats} to the device and splits them there into the staged
+// key and gradient arrays (st_keys, st_vals): the path of large blocks. The caller holds st_mu.
 static int32_t stage_pairs(pshbm_table* t, const void* pairs, size_t n, size_t stride, const char* what) {
     if (!pairs) return fail(t, PSHBM_ERROR, "%s: null buffer", what);
     const size_t used = 8 + (size_t)t->d.dim * 4;
@@ -857,17 +857,9 @@ static int32_t stage_pairs(pshbm_table* t, const void* pairs, size_t n, size_t s
     ST_TRY(ensure(t, t->st_keys, n * 8));
     ST_TRY(ensure(t, t->st_vals, n * (size_t)t->d.dim * 4));
     hipStream_t s = t->stream;
-    const uint32_t* raw = nullptr;
-    if (n * stride <= SMALL_HOST_BYTES) {  // the split kernel reads the pairs from mapped pinned memory
-        ST_TRY(ensure_small(t));
-        std::memcpy(t->h_small, pairs, n * stride);
-        raw = static_cast<const uint32_t*>(t->h_small);
-    } else {
-        ST_TRY(ensure(t, t->st_raw, n * stride));
-        HIP_TRY(t, hipMemcpyAsync(t->st_raw.p, pairs, n * stride, hipMemcpyHostToDevice, s));
-        raw = static_cast<const uint32_t*>(t->st_raw.p);
-    }
-    HIP_TRY(t, launch_unpack_records(raw, n,
+    ST_TRY(ensure(t, t->st_raw, n * stride));
+    HIP_TRY(t, hipMemcpyAsync(t->st_raw.p, pairs, n * stride, hipMemcpyHostToDevice, s));
+    HIP_TRY(t, launch_unpack_records(static_cast<const uint32_t*>(t->st_raw.p), n,
                                      (uint32_t)(stride / 4), t->d.dim,
                                      static_cast<uint64_t*>(t->st_keys.p),
                                      static_cast<float*>(t->st_vals.p), s));
