@@ -291,14 +291,26 @@ def test_sync_push_and_store(ps, orc, wl):
     t.close()
 
 
-def test_push_pairs_wire_layout(ps, orc):
+@pytest.mark.parametrize("n", [300, 60000])     # a block split on the host; one split on the device (2.5 MB)
+def test_push_pairs_wire_layout(ps, orc, n):
     rng = np.random.default_rng(8)
-    t, r = pair(ps, orc, 6, "sgd", capacity=1000)
-    pairs = np.zeros(300, dtype=np.dtype([("key", "<u8"), ("value", "<f4", (6,))]))
-    pairs["key"] = rng.permutation(1000)[:300]
-    pairs["value"] = rng.normal(0, 1, (300, 6))
+    t, r = pair(ps, orc, 6, "sgd", capacity=4 * n)
+    dt = np.dtype([("key", "<u8"), ("value", "<f4", (6,))])
+    pairs = np.zeros(n, dtype=dt)
+    pairs["key"] = rng.permutation(3 * n)[:n] + 1
+    pairs["value"] = rng.normal(0, 1, (n, 6))
     assert t.push_pairs(pairs) == 0 and r.push(pairs["key"], pairs["value"]) == 0
     assert_same_table(t, r, exact=True)
+    # the sync path takes the same blocks; padded pairs (a stride beyond the value) are allowed
+    wide = np.zeros(n, dtype=np.dtype([("key", "<u8"), ("value", "<f4", (6,)), ("pad", "<u4", (3,))]))
+    wide["key"], wide["value"] = pairs["key"], pairs["value"]
+    assert t.queue_pairs(pairs) == 0 and t.queue_pairs(wide) == 0 and t.queued() == 2 * n
+    assert r.queue(pairs["key"], pairs["value"]) == 0 and r.queue(pairs["key"], pairs["value"]) == 0
+    assert t.store() == 0 and r.store() == 0
+    assert_same_table(t, r, exact=False)
+    bad = pairs[:10].copy()
+    bad["key"][4] = 0xFFFFFFFFFFFFFFFF
+    assert t.push_pairs(bad) == ps.ERROR and t.queue_pairs(bad) == ps.ERROR and t.queued() == 0
     t.close()
 
 
