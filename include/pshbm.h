@@ -273,6 +273,19 @@ int32_t pshbm_erase_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, uint64
  * themselves once the markers fill an eighth of the slots. */
 int32_t pshbm_compact(pshbm_table* t);
 
+/* The optimizer's hyperparameters for the pushes and stores that follow. In the reference they
+ * belong to the push operator, not to the storage ("the learning rate of a push",
+ * pico-ps/operator/Operator.h:53-57), and a newly registered operator may bring new ones to a table
+ * that keeps its contents; this is also how a learning-rate schedule reaches the table. The
+ * optimizer itself and dim cannot change. INVALID_CONFIG on a bad struct_size or FTRL alpha <= 0. */
+typedef struct pshbm_hyperparameters {
+    uint32_t struct_size;        /* sizeof(pshbm_hyperparameters) */
+    float lr;                    /* SGD, ADAGRAD */
+    float init_acc;              /* ADAGRAD accumulator of keys inserted from now on */
+    float alpha, beta, l1, l2;   /* FTRL */
+} pshbm_hyperparameters;
+int32_t pshbm_set_hyperparameters(pshbm_table* t, const pshbm_hyperparameters* hp);
+
 /* Grows the table to hold expected_max_items keys (no effect if it holds as many already): new
  * arrays, the rows copied with their numbers, the hash array rebuilt from the stored keys. This is
  * the rehash a growing hash map of the reference does by itself inside an insert (safe_insert,

@@ -113,6 +113,7 @@ def lib():
         L.pso_erase_if.argtypes = [vp, vp, C.POINTER(C.c_uint64)]
         L.pso_erase.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_uint64)]
         L.pso_reserve.argtypes = [vp, C.c_uint64]
+        L.pso_set_hyperparameters.argtypes = [vp] + [C.c_float] * 6
         L.pso_increment_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pso_take_increment.argtypes = [vp, vp, C.c_size_t, C.POINTER(C.c_size_t)]
         L.pso_clear.argtypes = [vp]
@@ -251,6 +252,9 @@ class Oracle:
 
     def compact(self):
         return OK
+
+    def set_hyperparameters(self, lr=0.0, init_acc=0.0, alpha=0.0, beta=0.0, l1=0.0, l2=0.0):
+        return lib().pso_set_hyperparameters(self._h, lr, init_acc, alpha, beta, l1, l2)
 
     def reserve(self, capacity):
         return lib().pso_reserve(self._h, capacity)

@@ -564,6 +564,20 @@ int32_t pso_erase(void* h, const uint64_t* keys, size_t n, uint64_t* erased) {
     return ST_OK;
 }
 
+// The hyperparameters belong to the push operator (Operator.h:53-57); a new operator brings new ones.
+int32_t pso_set_hyperparameters(void* h, float lr, float init_acc, float alpha, float beta, float l1,
+                                float l2) {
+    Oracle& o = *static_cast<Oracle*>(h);
+    if (o.c.optimizer == OPT_FTRL && !(alpha > 0.0f)) return ST_INVALID_CONFIG;
+    o.c.lr = lr;
+    o.c.init_acc = init_acc;
+    o.c.alpha = alpha;
+    o.c.beta = beta;
+    o.c.l1 = l1;
+    o.c.l2 = l2;
+    return ST_OK;
+}
+
 // A growing hash map rehashes by itself (safe_insert, KVShardStorage.h:791-801); the fixed-capacity
 // model only raises its limit.
 int32_t pso_reserve(void* h, uint64_t capacity) {

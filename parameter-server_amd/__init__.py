@@ -31,7 +31,7 @@ SYMBOLS = [
     "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
     "pshbm_queue", "pshbm_queue_dev", "pshbm_queue_pairs", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
     "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
-    "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve",
+    "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve", "pshbm_set_hyperparameters",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
@@ -57,6 +57,18 @@ class Config(C.Structure):
         ("max_batch", C.c_uint64),
         ("track_increment", C.c_int32),
         ("reserved", C.c_int32),
+    ]
+
+
+class Hyperparameters(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("lr", C.c_float),
+        ("init_acc", C.c_float),
+        ("alpha", C.c_float),
+        ("beta", C.c_float),
+        ("l1", C.c_float),
+        ("l2", C.c_float),
     ]
 
 
@@ -187,6 +199,7 @@ def lib():
         L.pshbm_erase_dev.argtypes = [vp, vp, sz, C.POINTER(C.c_uint64), vp]
         L.pshbm_compact.argtypes = [vp]
         L.pshbm_reserve.argtypes = [vp, C.c_uint64]
+        L.pshbm_set_hyperparameters.argtypes = [vp, C.POINTER(Hyperparameters)]
         L.pshbm_increment_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pshbm_take_increment.argtypes = [vp, vp, sz, C.POINTER(sz)]
         L.pshbm_clear.argtypes = [vp]
@@ -383,6 +396,11 @@ class Table:
 
     def compact(self):
         return lib().pshbm_compact(self._h)
+
+    def set_hyperparameters(self, lr=0.0, init_acc=0.0, alpha=0.0, beta=0.0, l1=0.0, l2=0.0):
+        """The optimizer's hyperparameters for the pushes and stores that follow; status."""
+        hp = Hyperparameters(C.sizeof(Hyperparameters), lr, init_acc, alpha, beta, l1, l2)
+        return lib().pshbm_set_hyperparameters(self._h, C.byref(hp))
 
     def reserve(self, capacity):
         """Grows the table to hold `capacity` keys; status."""

@@ -1381,6 +1381,24 @@ int32_t pshbm_take_increment(pshbm_table* t, void* records, size_t capacity_reco
     return dump_range(t, 0, marked, records, static_cast<const uint32_t*>(t->ms_lists.p));
 }
 
+int32_t pshbm_set_hyperparameters(pshbm_table* t, const pshbm_hyperparameters* hp) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (!hp || hp->struct_size != sizeof(pshbm_hyperparameters))
+        return fail(t, PSHBM_INVALID_CONFIG, "set_hyperparameters: struct_size");
+    if (t->cfg.optimizer == PSHBM_OPT_FTRL && !(hp->alpha > 0.0f))
+        return fail(t, PSHBM_INVALID_CONFIG, "set_hyperparameters: FTRL needs alpha > 0");
+    // kernels take the parameters by value at launch: calls already queued keep the old ones
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    t->cfg.lr = hp->lr;
+    t->cfg.init_acc = hp->init_acc;
+    t->cfg.alpha = hp->alpha;
+    t->cfg.beta = hp->beta;
+    t->cfg.l1 = hp->l1;
+    t->cfg.l2 = hp->l2;
+    t->d.opt = OptParams{t->cfg.optimizer, hp->lr, hp->init_acc, hp->alpha, hp->beta, hp->l1, hp->l2};
+    return PSHBM_OK;
+}
+
 int32_t pshbm_reserve(pshbm_table* t, uint64_t expected_max_items) {
     if (!t) return PSHBM_INVALID_ID;
     if (expected_max_items > 0xFFFFFFF0ull)

@@ -111,6 +111,17 @@ public:
         _capacity[shard_id] = want;
         return true;
     }
+    // The hyperparameters of the push operator that is about to touch the shard (they live in the
+    // operator's config, pico-ps/operator/Operator.h:53-57): handed to the table when they differ
+    // from the ones it has. Operators with different hyperparameters must not push to one table at
+    // the same time (the reference advises against changing a registered operator's config at all).
+    void use_hyperparameters(int32_t shard_id, const pshbm_hyperparameters& hp) {
+        auto it = _hp.find(shard_id);
+        if (it != _hp.end() && std::memcmp(&it->second, &hp, sizeof hp) == 0) return;
+        PSHBM_SCHECK(pshbm_set_hyperparameters(get(shard_id), &hp) == PSHBM_OK,
+                     std::string("bad hyperparameters: ") + pshbm_last_error(nullptr));
+        _hp[shard_id] = hp;
+    }
     void clear() {  // KVShardStorage.h:902-908: every shard emptied, the shards stay
         for (auto& p : _shards) pshbm_clear(p.second);
     }
@@ -148,6 +159,7 @@ private:
     Configure _config;
     std::map<int32_t, pshbm_table*> _shards;
     std::map<int32_t, uint64_t> _capacity;  // keys each shard's table holds at most
+    std::map<int32_t, pshbm_hyperparameters> _hp;  // what each shard's table was last given
     uint32_t _dim = 0, _vf = 0;
     std::string _error;
 };
@@ -237,9 +249,18 @@ private:
 
 // Server halves of the sparse push. A push block is n raw std::pair<KEY, PUSH_VALUE> records, here
 // {uint64 key, dim floats} (SparsePushOperator.h:164-179, 245-247).
+// lr, init_acc, alpha, beta, l1, l2 of an operator's config, if it names any of them
+inline bool operator_hyperparameters(const Configure& c, pshbm_hyperparameters* hp) {
+    const pshbm_config cfg = table_config(c);
+    *hp = pshbm_hyperparameters{sizeof(pshbm_hyperparameters), cfg.lr, cfg.init_acc, cfg.alpha, cfg.beta, cfg.l1, cfg.l2};
+    for (const char* k : {"lr", "init_acc", "alpha", "beta", "l1", "l2"})
+        if (c.has(k)) return true;
+    return false;
+}
+
 class HbmSparsePushOperator {
 public:
-    explicit HbmSparsePushOperator(const Configure&) {}
+    explicit HbmSparsePushOperator(const Configure& config) : _has_hp(operator_hyperparameters(config, &_hp)) {}
 
     // apply_async_push_request, SparsePushOperator.h:197-276. Differences, both documented in
     // include/pshbm.h: equal keys inside one block are summed (the reference's client never sends
@@ -250,6 +271,7 @@ public:
         Status status;
         auto& st = *static_cast<HbmShardStorage*>(storage);
         for_each_block(rt, req, storage, [&](int32_t shard_id, pshbm_table* t, const std::vector<char>& block, int32_t n, size_t stride) {
+            if (_has_hp) st.use_hyperparameters(shard_id, _hp);
             int32_t rc = pshbm_push_pairs(t, block.data(), n, stride, 0);
             while (rc == PSHBM_OUT_OF_MEMORY && st.grow(shard_id)) rc = pshbm_push_pairs(t, block.data(), n, stride, 0);
             if (rc == PSHBM_OUT_OF_MEMORY) status = Status::OOM(pshbm_last_error(t));
@@ -282,12 +304,16 @@ public:
         resp << Status();
         send_response(std::move(resp));
         if (delta_storage == nullptr) return;  // :336-341
+        if (_has_hp) static_cast<HbmShardStorage*>(storage)->use_hyperparameters(shard_id, _hp);
         pshbm_store(static_cast<HbmShardStorage*>(storage)->get(shard_id), 0);
     }
 
     std::unique_ptr<Storage> create_delta_storage(RuntimeInfo&) { return std::make_unique<HbmDeltaStorage>(); }  // :425-427
 
 private:
+    pshbm_hyperparameters _hp{};
+    bool _has_hp;
+
     template <class F>
     static void for_each_block(RuntimeInfo& rt, PSRequest& req, Storage* storage, F&& f) {
         int32_t shards_num, merge_num;

@@ -369,6 +369,40 @@ static void test_growth() {
     EXPECT(hst->shard_size(0) == 500 && hst->shard_size(1) == 500);
 }
 
+// The learning rate belongs to the push operator (pico-ps/operator/Operator.h:53-57): two operators
+// registered with different rates push to one storage, each with its own.
+static void test_operator_hyperparameters() {
+    Configure storage_config;
+    storage_config.set("dim", 2);
+    storage_config.set("optimizer", "sgd");
+    storage_config.set("lr", 0.5);
+    storage_config.set("hbm_table.expected_max_items", 100);
+    RuntimeInfo rt(0, {0, 1});
+    HbmStorageOperator storage_op(storage_config);
+    std::unique_ptr<Storage> storage = storage_op.create_storage(rt, 0);
+    Configure slow = storage_config;
+    slow.set("lr", 0.25);
+    HbmSparsePushOperator push_fast(storage_config), push_slow(slow);
+    HbmSparsePullOperator pull_op(storage_config);
+    const std::vector<uint64_t> keys{10, 11, 12, 13};
+    const std::vector<float> args{1.0f, 1.0f, 1.0f, 1.0f};  // gradient [arg, 1]
+    auto push = [&](HbmSparsePushOperator& op) {
+        PSRequest req = make_push_request(keys, args);
+        PSResponse resp;
+        Status status;
+        op.apply_async_push_request(rt, req, storage.get(), nullptr, resp);
+        resp >> status;
+        EXPECT(status.ok());
+    };
+    push(push_fast);   // w = -0.5
+    push(push_slow);   // w = -0.75
+    push(push_fast);   // w = -1.25
+    bool ok;
+    auto v = pull(pull_op, rt, storage.get(), keys, &ok);
+    EXPECT(ok);
+    for (size_t i = 0; i < keys.size(); ++i) EXPECT(v[i * 2] == -1.25f && v[i * 2 + 1] == -1.25f);
+}
+
 int main(int argc, char** argv) {
     const std::string dir = argc > 1 ? argv[1] : "/tmp";
     Configure op_config;
@@ -697,6 +731,7 @@ int main(int argc, char** argv) {
 
     test_dense(dir);
     test_growth();
+    test_operator_hyperparameters();
     if (g_failed) {
         std::printf("FAILED: %d expectation(s)\n", g_failed);
         return 1;

@@ -649,3 +649,27 @@ def test_one_launch_push_heavy_repeats(ps, orc, dim, n):
         assert t.push(q, g, flags) == 0 and r.push(q, g, flags) == 0
         assert_same_table(t, r, exact=True)
     t.close()
+
+
+@pytest.mark.parametrize("opt", ["sgd", "adagrad", "ftrl"])
+def test_hyperparameters_change_between_pushes(ps, orc, wl, opt):
+    """A learning-rate schedule (or a newly registered push operator, pico-ps/operator/Operator.h:53-57):
+    the pushes after pshbm_set_hyperparameters take the new values, keys inserted afterwards the new
+    initial accumulator; distinct keys per batch, so every value compares bit for bit."""
+    rng = np.random.default_rng(3)
+    dim = 12
+    t, r = pair(ps, orc, dim, opt, capacity=6000)
+    keys = wl.table_keys_np(0, 5000, seed=6)
+    schedules = [dict(lr=0.5, init_acc=0.25, alpha=0.1, beta=0.5, l1=1e-3, l2=1e-2),
+                 dict(lr=0.03125, init_acc=1.0, alpha=0.7, beta=2.0, l1=0.0, l2=0.0)]
+    for it in range(4):
+        q = keys[rng.permutation(5000)[: 400 + 700 * it]]          # one-launch and chained pushes
+        g = rng.normal(0, 0.1, (q.size, dim)).astype(np.float32)
+        assert t.push(q, g) == 0 and r.push(q, g) == 0
+        if it < 2:
+            hp = schedules[it]
+            assert t.set_hyperparameters(**hp) == 0 and r.set_hyperparameters(**hp) == 0
+    assert_same_table(t, r, exact=True)
+    if opt == "ftrl":
+        assert t.set_hyperparameters(alpha=0.0) == ps.INVALID_CONFIG
+    t.close()
