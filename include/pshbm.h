@@ -79,7 +79,9 @@ typedef struct pshbm_config {
     uint64_t max_batch;          /* workspace is pre-sized for batches of this many keys;
                                     larger batches grow it (which allocates and synchronizes) */
     int32_t track_increment;     /* remember which keys pushes touch, for pshbm_take_increment */
-    int32_t reserved;
+    float init_range;            /* weights of a key that is inserted by a push or a pull: 0 = zeros;
+                                    r > 0 = uniform in [-r, r), drawn from a hash of (key, column)
+                                    (see "Initial weights" below). Fixed for the table's life. */
 } pshbm_config;
 
 typedef struct pshbm_stats {
@@ -117,12 +119,24 @@ int32_t pshbm_destroy(pshbm_table* t);
  * on several threads at once; valid until the same thread's next failing call. */
 const char* pshbm_last_error(const pshbm_table* t);
 
+/* Initial weights. The reference leaves the value of a new key to the operator's init_store_value
+ * (pico-ps/operator/SparsePullOperator.h:307-310, SparsePushOperator.h:250-251), which models
+ * usually fill with small random numbers. With init_range = r > 0 column c of key k starts at
+ *     h = fmix64(k ^ ((c + 1) * 0x9E3779B97F4A7C15))      (fmix64: MurmurHash3's 64-bit finalizer)
+ *     w = ((float)(h >> 40) * 2^-23 - 1) * r               (each operation rounded to fp32)
+ * a pure function of (key, column): a pull that does not insert answers the same weights that a
+ * later insertion of the key stores, every shard and every replica agrees on them without
+ * exchanging anything, and a restored table continues as the dumped one would have. Optimizer
+ * state starts as without init_range. pshbm_init_weight gives the same number on the host. */
+float pshbm_init_weight(float init_range, uint64_t key, uint32_t column);
+
 /* Floats per stored value (weights + optimizer state) for a dim and optimizer; 0 if invalid. */
 uint32_t pshbm_value_floats(uint32_t dim, int32_t optimizer);
 
 /* Sparse pull. Replaces the per-key loop of SparseTablePullOperator::apply_request
  * (pico-ps/operator/SparsePullOperator.h:208-228): for key i, out_rows[i*dim .. +dim) is the
- * stored weights (fetch_pull_value) or zeros on a miss (init_store_value's value_type(), :307-310);
+ * stored weights (fetch_pull_value) or, on a miss, the weights a new key starts with
+ * (init_store_value, :217,307-310: zeros, or the table's initial weights when init_range > 0);
  * hit[i] (may be NULL) is lock_find's return against the table as it was when the call began.
  * With PSHBM_PULL_INSERT_ON_MISS (ignored on a read_only table) each distinct missing key is
  * inserted with a fresh row. OUT_OF_MEMORY when the insertions do not fit (:245-253): then no key

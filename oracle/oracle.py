@@ -33,6 +33,7 @@ class _Config(C.Structure):
         ("capacity", C.c_uint64),
         ("read_only", C.c_int32),
         ("track_increment", C.c_int32),
+        ("init_range", C.c_float),
     ]
 
 
@@ -96,6 +97,8 @@ def lib():
         L.pso_value_floats.restype = C.c_uint32
         L.pso_value_floats.argtypes = [C.c_uint32, C.c_int32]
         L.pso_create.argtypes = [C.POINTER(_Config), C.POINTER(vp)]
+        L.pso_init_weight.restype = C.c_float
+        L.pso_init_weight.argtypes = [C.c_float, C.c_uint64, C.c_uint32]
         L.pso_destroy.argtypes = [vp]
         L.pso_pull.argtypes = [vp, u64p, C.c_size_t, f32p, u8p, C.c_uint32]
         L.pso_aggregate.argtypes = [C.c_uint32, u64p, f32p, C.c_size_t, u64p, f32p,
@@ -137,16 +140,21 @@ def record_dtype(value_floats):
     return np.dtype([("key", "<u8"), ("value", "<f4", (value_floats,))])
 
 
+def init_weight(init_range, key, column):
+    """Weight `column` of a new key of a table that draws initial weights in [-init_range, init_range)."""
+    return lib().pso_init_weight(init_range, key, column)
+
+
 class Oracle:
     """One shard of the reference's KV storage with the operator loops on top (CPU, scalar)."""
 
     def __init__(self, dim, optimizer=OPT_SUM, lr=0.0, init_acc=0.0, alpha=0.0, beta=0.0, l1=0.0,
-                 l2=0.0, capacity=1 << 20, read_only=False, track_increment=False):
+                 l2=0.0, capacity=1 << 20, read_only=False, track_increment=False, init_range=0.0):
         self.dim = dim
         self.optimizer = optimizer
         self.value_floats = lib().pso_value_floats(dim, optimizer)
         cfg = _Config(dim, optimizer, lr, init_acc, alpha, beta, l1, l2, capacity, int(read_only),
-                      int(track_increment))
+                      int(track_increment), init_range)
         self._h = C.c_void_p()
         st = lib().pso_create(C.byref(cfg), C.byref(self._h))
         if st != OK:

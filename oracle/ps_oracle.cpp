@@ -41,6 +41,12 @@
 //       hook SparsePushOperator.h:448). The formulas are this repository's definition; they are
 //       pinned by hand-computed single-key cases, a float64 re-evaluation and algebraic special
 //       cases in tests/test_oracle_optimizers.py.
+//   Initial weights of a new key (init_weight below, when init_range > 0)
+//       PARITY UNPINNED BY THE REFERENCE: the value a pull or push inserts is the user hook
+//       init_store_value (SparsePullOperator.h:307-310, SparsePushOperator.h:250-251), for which
+//       pico-ps ships only zeros. The formula is this repository's; it is pinned by MurmurHash3's
+//       published finalizer vectors, an integer-only Python restatement, the exact bounds and the
+//       first two moments of the uniform distribution (tests/test_initial_weights.py).
 //   Capacity handling (PSO_OUT_OF_MEMORY, all-or-nothing per batch)
 //       this repository's decision for a fixed-capacity table; the reference instead parks the
 //       items in an overflow vector (SparsePushOperator.h:257-259). Documented, not pinned.
@@ -74,6 +80,7 @@ struct Config {
     uint64_t capacity;
     int32_t read_only;
     int32_t track_increment;
+    float init_range;
 };
 
 struct Oracle {
@@ -104,10 +111,28 @@ uint32_t value_floats(uint32_t dim, int32_t opt) {
 
 bool reserved(uint64_t k) { return k == KEY_EMPTY || k == KEY_DELETED; }
 
-// value_type() of a key that a pull or push inserts: zero weights, fresh optimizer state.
-void init_value(const Config& c, float* v) {
+// MurmurHash3's 64-bit finalizer (Appleby, MurmurHash3.cpp, public domain).
+uint64_t fmix64(uint64_t k) {
+    k ^= k >> 33;
+    k *= 0xff51afd7ed558ccdull;
+    k ^= k >> 33;
+    k *= 0xc4ceb9fe1a85ec53ull;
+    k ^= k >> 33;
+    return k;
+}
+
+// Weight j of a new key when the table draws initial weights: the top 24 bits of a hash of
+// (key, column) as a number in [-1, 1) (exact in fp32), times the range (one rounding).
+float init_weight(float range, uint64_t key, uint32_t j) {
+    const uint64_t h = fmix64(key ^ ((uint64_t)(j + 1u) * 0x9E3779B97F4A7C15ull));
+    const float unit = (float)(uint32_t)(h >> 40) * (1.0f / 8388608.0f) - 1.0f;
+    return unit * range;
+}
+
+// value_type() of a key that a pull or push inserts: zero (or drawn) weights, fresh optimizer state.
+void init_value(const Config& c, uint64_t key, float* v) {
     const uint32_t d = c.dim;
-    for (uint32_t j = 0; j < d; ++j) v[j] = 0.0f;
+    for (uint32_t j = 0; j < d; ++j) v[j] = c.init_range != 0.0f ? init_weight(c.init_range, key, j) : 0.0f;
     if (c.optimizer == OPT_ADAGRAD)
         for (uint32_t j = 0; j < d; ++j) v[d + j] = c.init_acc;
     if (c.optimizer == OPT_FTRL)
@@ -218,7 +243,7 @@ int32_t apply_unique(Oracle& o, const std::vector<uint64_t>& ukeys, const std::v
         if (it == o.map.end()) {
             if (!insert) continue;  // init_store_value returned false: item dropped (:250-251)
             r = append_row(o, ukeys[u]);
-            init_value(o.c, &o.rows[(size_t)r * o.vf]);
+            init_value(o.c, ukeys[u], &o.rows[(size_t)r * o.vf]);
         } else {
             r = it->second;
         }
@@ -239,19 +264,22 @@ struct pso_config {
     uint64_t capacity;
     int32_t read_only;
     int32_t track_increment;
+    float init_range;
 };
+
+float pso_init_weight(float range, uint64_t key, uint32_t column) { return init_weight(range, key, column); }
 
 uint32_t pso_value_floats(uint32_t dim, int32_t opt) { return value_floats(dim, opt); }
 
 // create_shard, KVShardStorage.h:910-925
 int32_t pso_create(const pso_config* cfg, void** out) {
     if (!cfg || !out || cfg->dim == 0 || value_floats(cfg->dim, cfg->optimizer) == 0 ||
-        cfg->capacity == 0)
+        cfg->capacity == 0 || !(cfg->init_range >= 0.0f && cfg->init_range <= 3.0e38f))
         return ST_INVALID_CONFIG;
     auto* o = new Oracle();
     o->c = Config{cfg->dim, cfg->optimizer, cfg->lr,  cfg->init_acc,  cfg->alpha,
                   cfg->beta, cfg->l1,       cfg->l2,  cfg->capacity,  cfg->read_only,
-                  cfg->track_increment};
+                  cfg->track_increment, cfg->init_range};
     o->vf = value_floats(cfg->dim, cfg->optimizer);
     *out = o;
     return ST_OK;
@@ -285,7 +313,7 @@ int32_t pso_pull(void* h, const uint64_t* keys, size_t n, float* out_rows, uint8
             src = &o.rows[(size_t)it->second * o.vf];
             if (hit) hit[i] = it->second < rows_at_entry;  // mask against the table at entry
         } else {
-            init_value(o.c, store_val.data());  // init_store_value, :217
+            init_value(o.c, keys[i], store_val.data());  // init_store_value, :217
             src = store_val.data();
             if (hit) hit[i] = 0;
             if (insert) {  // safe_insert, :224

@@ -27,7 +27,7 @@ LOAD_UNIQUE = 1
 
 # every symbol include/pshbm.h declares
 SYMBOLS = [
-    "pshbm_create", "pshbm_destroy", "pshbm_last_error", "pshbm_value_floats",
+    "pshbm_create", "pshbm_destroy", "pshbm_last_error", "pshbm_value_floats", "pshbm_init_weight",
     "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
     "pshbm_queue", "pshbm_queue_dev", "pshbm_queue_pairs", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
     "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
@@ -56,7 +56,7 @@ class Config(C.Structure):
         ("read_only", C.c_int32),
         ("max_batch", C.c_uint64),
         ("track_increment", C.c_int32),
-        ("reserved", C.c_int32),
+        ("init_range", C.c_float),
     ]
 
 
@@ -176,6 +176,8 @@ def lib():
         L.pshbm_last_error.restype = C.c_char_p
         L.pshbm_value_floats.argtypes = [u32, i32]
         L.pshbm_value_floats.restype = u32
+        L.pshbm_init_weight.argtypes = [C.c_float, C.c_uint64, u32]
+        L.pshbm_init_weight.restype = C.c_float
         L.pshbm_pull.argtypes = [vp, vp, sz, vp, vp, u32]
         L.pshbm_pull_dev.argtypes = [vp, vp, sz, vp, vp, u32, vp]
         L.pshbm_push.argtypes = [vp, vp, vp, sz, u32]
@@ -221,6 +223,11 @@ def value_floats(dim, optimizer):
     return lib().pshbm_value_floats(dim, optimizer)
 
 
+def init_weight(init_range, key, column):
+    """Weight `column` that a table with this init_range gives a new key (host side of the kernels' formula)."""
+    return lib().pshbm_init_weight(init_range, key, column)
+
+
 def record_dtype(vf):
     """Layout of one Load/Dump record: uint64 key then the value's floats, packed."""
     return np.dtype([("key", "<u8"), ("value", "<f4", (vf,))])
@@ -256,12 +263,12 @@ class Table:
 
     def __init__(self, dim, optimizer=OPT_SUM, lr=0.0, init_acc=0.0, alpha=0.0, beta=0.0, l1=0.0,
                  l2=0.0, capacity=1 << 20, max_load_factor=0.0, read_only=False, max_batch=0,
-                 device=0, track_increment=False):
+                 device=0, track_increment=False, init_range=0.0):
         self.dim = dim
         self.optimizer = optimizer
         self._h = C.c_void_p()
         cfg = Config(C.sizeof(Config), device, dim, optimizer, lr, init_acc, alpha, beta, l1, l2,
-                     capacity, max_load_factor, int(read_only), max_batch, int(track_increment), 0)
+                     capacity, max_load_factor, int(read_only), max_batch, int(track_increment), init_range)
         st = lib().pshbm_create(C.byref(cfg), C.byref(self._h))
         if st != OK:
             raise PshbmError(st, (lib().pshbm_last_error(None) or b"").decode())

@@ -580,6 +580,10 @@ uint32_t pshbm_value_floats(uint32_t dim, int32_t optimizer) {
 
 const char* pshbm_last_error(const pshbm_table*) { return g_error.c_str(); }
 
+float pshbm_init_weight(float init_range, uint64_t key, uint32_t column) {
+    return init_weight(init_range, key, column);
+}
+
 int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     if (!cfg || !out) return PSHBM_INVALID_CONFIG;
     *out = nullptr;
@@ -596,6 +600,7 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     float lf = cfg->max_load_factor == 0.0f ? 0.5f : cfg->max_load_factor;
     if (!(lf > 0.0f && lf <= 0.9f)) return bad("max_load_factor must be in (0, 0.9]");
     if (cfg->optimizer == PSHBM_OPT_FTRL && !(cfg->alpha > 0.0f)) return bad("FTRL needs alpha > 0");
+    if (!(cfg->init_range >= 0.0f && cfg->init_range <= 3.0e38f)) return bad("init_range must be finite and >= 0");
 
     int ndev = 0;
     hipError_t e = hipGetDeviceCount(&ndev);
@@ -630,7 +635,8 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     d.dim = cfg->dim;
     d.vf = vf;
     d.stride_f = (uint32_t)round_up(vf, 4);
-    d.opt = OptParams{cfg->optimizer, cfg->lr, cfg->init_acc, cfg->alpha, cfg->beta, cfg->l1, cfg->l2};
+    d.opt = OptParams{cfg->optimizer, cfg->lr, cfg->init_acc, cfg->alpha, cfg->beta, cfg->l1, cfg->l2,
+                      cfg->init_range};
     t->slots_bytes = nb * 64;
     t->rows_bytes = max_rows * d.stride_f * 4;
     t->keys_bytes = max_rows * 8;
@@ -706,7 +712,7 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
     ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, nullptr, true, true, false, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
-    HIP_TRY_PROF(t, s, PSHBM_PHASE_GATHER, launch_gather_slots(t->d, slot, n, d_out_rows, d_hit, s));
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_GATHER, launch_gather_slots(t->d, d_keys, slot, n, d_out_rows, d_hit, s));
     return PSHBM_OK;
 }
 
@@ -1395,7 +1401,8 @@ int32_t pshbm_set_hyperparameters(pshbm_table* t, const pshbm_hyperparameters* h
     t->cfg.beta = hp->beta;
     t->cfg.l1 = hp->l1;
     t->cfg.l2 = hp->l2;
-    t->d.opt = OptParams{t->cfg.optimizer, hp->lr, hp->init_acc, hp->alpha, hp->beta, hp->l1, hp->l2};
+    t->d.opt = OptParams{t->cfg.optimizer, hp->lr, hp->init_acc, hp->alpha, hp->beta, hp->l1, hp->l2,
+                         t->cfg.init_range};
     return PSHBM_OK;
 }
 

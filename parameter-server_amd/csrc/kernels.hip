@@ -30,16 +30,28 @@ __device__ __forceinline__ u64 div_big(u64 n, u64 m, u32 d) { return d == 1 ? n 
 inline u64 magic32(u32 d) { return ((1ull << 32) + d - 1) / d; }
 inline u64 magic64(u32 d) { return d <= 1 ? 0 : (~0ull / d) + 1; }
 
-__device__ __forceinline__ float init_float(const TableDev& t, u32 f) {
-    return (t.opt.kind == 2 /*ADAGRAD*/ && f >= t.dim) ? t.opt.init_acc : 0.0f;
+// float f of the value a key starts with: weights, then optimizer state
+__device__ __forceinline__ float init_float(const TableDev& t, u64 key, u32 f) {
+    if (f < t.dim) return t.opt.init_range != 0.0f ? init_weight(t.opt.init_range, key, f) : 0.0f;
+    return t.opt.kind == 2 /*ADAGRAD*/ ? t.opt.init_acc : 0.0f;
+}
+// the weights a pull answers for a key that is not stored (init_store_value + fetch_pull_value of
+// pico-ps/operator/SparsePullOperator.h:217,226), column unit c of T
+__device__ __forceinline__ float init_pulled(const TableDev& t, u64 key, u32 c, float) {
+    return init_weight(t.opt.init_range, key, c);
+}
+__device__ __forceinline__ float4 init_pulled(const TableDev& t, u64 key, u32 c, float4) {
+    return make_float4(init_weight(t.opt.init_range, key, c * 4), init_weight(t.opt.init_range, key, c * 4 + 1),
+                       init_weight(t.opt.init_range, key, c * 4 + 2), init_weight(t.opt.init_range, key, c * 4 + 3));
 }
 
 // ---- row gather into the packed response -----------------------------------------------------
-// `row` holds, in the lanes of group k, the row of key base + k (ROW_NONE = miss -> zeros).
+// `row` holds, in the lanes of group k, the row of key base + k (ROW_NONE = miss -> the weights a
+// new key would start with: zeros, or init_weight() when the table draws them).
 template <typename T>
 __device__ __forceinline__ void gather_round(const TableDev& t, u32 row, u64 base, u32 cnt,
                                              T* __restrict__ out, u32 units, u32 stride_units,
-                                             u64 m32, u32 lane) {
+                                             u64 m32, u32 lane, const u64* __restrict__ keys) {
     const T* rows = reinterpret_cast<const T*>(t.rows);
     const u32 total = cnt * units;
     for (u32 j0 = 0; j0 < total; j0 += 64) {
@@ -50,7 +62,12 @@ __device__ __forceinline__ void gather_round(const TableDev& t, u32 row, u64 bas
         u32 r = __shfl(row, (int)(k * 4));
         if (on) {
             T v = vzero(T());
-            if (r != ROW_NONE) v = rows[(u64)r * stride_units + c];
+            if (r != ROW_NONE) {
+                v = rows[(u64)r * stride_units + c];
+            } else if (t.opt.init_range != 0.0f) {
+                const u64 key = keys[base + k];
+                if (key < KEY_DELETED) v = init_pulled(t, key, c, T());
+            }
             out[base * units + j] = v;
         }
     }
@@ -73,12 +90,13 @@ __global__ __launch_bounds__(BLOCK) void pull_kernel(TableDev t, const u64* __re
         Found f = probe_find(t, key, active, grp, sub);
         if (hit && inb && sub == 0) hit[i] = f.row != ROW_NONE;
         u32 cnt = (u32)((n - base) < KEYS_PER_ROUND ? (n - base) : KEYS_PER_ROUND);
-        gather_round<T>(t, f.row, base, cnt, out, units, stride_units, m32, lane);
+        gather_round<T>(t, f.row, base, cnt, out, units, stride_units, m32, lane, keys);
     }
 }
 
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void gather_slots_kernel(TableDev t,
+                                                              const u64* __restrict__ keys,
                                                               const u32* __restrict__ slot_idx,
                                                               u32 n, T* __restrict__ out,
                                                               uint8_t* __restrict__ hit, u32 units,
@@ -98,7 +116,7 @@ __global__ __launch_bounds__(BLOCK) void gather_slots_kernel(TableDev t,
             if (hit && sub == 0) hit[i] = row < entry_rows;
         }
         u32 cnt = (u32)((n - base) < KEYS_PER_ROUND ? (n - base) : KEYS_PER_ROUND);
-        gather_round<T>(t, row, base, cnt, out, units, stride_units, m32, lane);
+        gather_round<T>(t, row, base, cnt, out, units, stride_units, m32, lane, keys);
     }
 }
 
@@ -351,8 +369,8 @@ __global__ __launch_bounds__(BLOCK) void assign_rows_kernel(TableDev t, const u6
             float4* r4 = reinterpret_cast<float4*>(t.rows + (u64)rid * t.stride_f);
             for (u32 c = 0; c < t.stride_f / 4; ++c) {
                 const u32 f = c * 4;
-                r4[c] = make_float4(init_float(t, f), init_float(t, f + 1), init_float(t, f + 2),
-                                    init_float(t, f + 3));
+                r4[c] = make_float4(init_float(t, keys[i], f), init_float(t, keys[i], f + 1),
+                                    init_float(t, keys[i], f + 2), init_float(t, keys[i], f + 3));
             }
         }
     }
@@ -900,7 +918,7 @@ __global__ __launch_bounds__(SMALL_PUSH) void push_small_kernel(TableDev t, cons
     __shared__ u32 q_row[SMALL_PUSH], q_idx[SMALL_PUSH];    // pairs sorted by (row, batch index)
     __shared__ u32 heads[SMALL_PUSH + 1];                   // starts of the runs; heads[nruns] = their end
     __shared__ u32 longs[SMALL_PUSH / SMALL_LONG + 1];      // runs added by the whole workgroup
-    __shared__ u32 new_rows[SMALL_PUSH];
+    __shared__ u32 new_idx[SMALL_PUSH];  // batch index of the k-th key inserted by this call
     __shared__ u32 wave_sums[SMALL_PUSH / 64];
     __shared__ u32 n_long;
     __shared__ T part[SMALL_PUSH];
@@ -948,11 +966,10 @@ __global__ __launch_bounds__(SMALL_PUSH) void push_small_kernel(TableDev t, cons
             reinterpret_cast<u32*>(&t.slots[slot])[2] = rid;
             t.row_keys[rid] = keys[tid];
             s_row[tid] = rid;
-            new_rows[rank] = rid;
         } else {  // does not fit (the host rules this out before it chooses this kernel)
             s_row[tid] = ROW_NONE;
-            new_rows[rank] = ROW_NONE;
         }
+        new_idx[rank] = tid;
     }
     if (tid == 0 && insert) {
         t.counters[CNT_ENTRY] = entry;
@@ -966,12 +983,13 @@ __global__ __launch_bounds__(SMALL_PUSH) void push_small_kernel(TableDev t, cons
         if (tid < n && s_row[tid] == ROW_PENDING)
             s_row[tid] = __hip_atomic_load(reinterpret_cast<u32*>(&t.slots[s_slot[tid]]) + 2, __ATOMIC_RELAXED,
                                            __HIP_MEMORY_SCOPE_AGENT);
-        // fresh rows: zero weights, initial optimizer state
+        // fresh rows: initial weights, initial optimizer state
         const u32 per = t.stride_f;
         for (u32 e = tid; e < n_won * per; e += SMALL_PUSH) {
             const u32 k = e / per, f = e - k * per;
-            const u32 rid = new_rows[k];
-            if (rid != ROW_NONE) t.rows[(u64)rid * per + f] = init_float(t, f);
+            const u32 i = new_idx[k];
+            const u32 rid = s_row[i];
+            if (rid != ROW_NONE) t.rows[(u64)rid * per + f] = init_float(t, keys[i], f);
         }
         __threadfence();
         __syncthreads();
@@ -1198,17 +1216,17 @@ hipError_t launch_pull(const TableDev& t, const u64* keys, size_t n, float* out,
     return hipGetLastError();
 }
 
-hipError_t launch_gather_slots(const TableDev& t, const u32* slot_idx, size_t n, float* out,
+hipError_t launch_gather_slots(const TableDev& t, const u64* keys, const u32* slot_idx, size_t n, float* out,
                                uint8_t* hit, hipStream_t s) {
     if (n == 0) return hipSuccess;
     const u32 grid = grid_for(n, KEYS_PER_ROUND * (BLOCK / 64), 16384);
     if (vec4_ok(t, out)) {
         u32 units = t.dim / 4;
-        gather_slots_kernel<float4><<<grid, BLOCK, 0, s>>>(t, slot_idx, (u32)n,
+        gather_slots_kernel<float4><<<grid, BLOCK, 0, s>>>(t, keys, slot_idx, (u32)n,
                                                            reinterpret_cast<float4*>(out), hit,
                                                            units, t.stride_f / 4, magic32(units));
     } else {
-        gather_slots_kernel<float><<<grid, BLOCK, 0, s>>>(t, slot_idx, (u32)n, out, hit, t.dim,
+        gather_slots_kernel<float><<<grid, BLOCK, 0, s>>>(t, keys, slot_idx, (u32)n, out, hit, t.dim,
                                                           t.stride_f, magic32(t.dim));
     }
     return hipGetLastError();

@@ -39,6 +39,7 @@ enum {
 struct OptParams {
     int32_t kind;  // PSHBM_OPT_*
     float lr, init_acc, alpha, beta, l1, l2;
+    float init_range;  // weights of a new key: 0, or uniform in [-init_range, init_range) by init_weight()
 };
 
 struct TableDev {
@@ -62,6 +63,16 @@ __host__ __device__ inline uint64_t hash64(uint64_t h) {
     h *= 0xc4ceb9fe1a85ec53ull;
     h ^= h >> 33;
     return h;
+}
+
+// Weight `col` of a key that is inserted, when the table draws initial weights: a pure function
+// of key and column (24 bits of a hash, mapped to [-1, 1) exactly, times the range with one
+// rounding), so that every path -- and the CPU restatement -- gives the key the same weights.
+__host__ __device__ inline float init_weight(float range, uint64_t key, uint32_t col) {
+    const uint64_t h = hash64(key ^ ((uint64_t)(col + 1u) * 0x9E3779B97F4A7C15ull));
+    const float u = (float)(uint32_t)(h >> 40);
+    const float x = u * 1.1920928955078125e-07f - 1.0f;
+    return x * range;
 }
 
 // Segment-reduce geometry shared by the kernels and the host that sizes their scratch.
@@ -115,7 +126,7 @@ hipError_t launch_assign_rows(const TableDev& t, const uint64_t* keys, size_t n,
                               size_t won_words, bool init_rows, hipStream_t s);
 
 // Gather through located slots (pull with insertion); hit = row existed when the pull began.
-hipError_t launch_gather_slots(const TableDev& t, const uint32_t* slot_idx, size_t n, float* out,
+hipError_t launch_gather_slots(const TableDev& t, const uint64_t* keys, const uint32_t* slot_idx, size_t n, float* out,
                                uint8_t* hit, hipStream_t s);
 
 // Undo of a batch of claims: every located slot whose row is >= first_new_row (or unset) is

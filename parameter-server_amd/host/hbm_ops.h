@@ -32,7 +32,7 @@ namespace pshbm_host {
 
 // op_config keys of an HBM table: dim, optimizer (sum|sgd|adagrad|ftrl), lr, init_acc, alpha, beta,
 // l1, l2, hbm_table.expected_max_items, hbm_table.grow_limit, hbm_table.max_load_factor,
-// hbm_table.max_batch, hbm_table.track_increment, read_only, device. The learning rate lives in the operator config, as pico-ps/operator/Operator.h:55 expects.
+// hbm_table.max_batch, hbm_table.track_increment, hbm_table.init_range, read_only, device. The learning rate lives in the operator config, as pico-ps/operator/Operator.h:55 expects.
 inline pshbm_config table_config(const Configure& c) {
     pshbm_config cfg{};
     cfg.struct_size = sizeof(cfg);
@@ -52,6 +52,7 @@ inline pshbm_config table_config(const Configure& c) {
     cfg.max_batch = (uint64_t)c.number("hbm_table.max_batch", 0);
     cfg.read_only = (int32_t)c.number("read_only", 0);
     cfg.track_increment = (int32_t)c.number("hbm_table.track_increment", 0);
+    cfg.init_range = (float)c.number("hbm_table.init_range", 0.0);
     return cfg;
 }
 

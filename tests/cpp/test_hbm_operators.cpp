@@ -403,6 +403,44 @@ static void test_operator_hyperparameters() {
     for (size_t i = 0; i < keys.size(); ++i) EXPECT(v[i * 2] == -1.25f && v[i * 2 + 1] == -1.25f);
 }
 
+// hbm_table.init_range: a pull that misses answers the weights an insertion would store; a push
+// of a new key takes its step from them (init_store_value, SparsePullOperator.h:217,307-310).
+static void test_initial_weights() {
+    Configure cfg;
+    cfg.set("dim", 2);
+    cfg.set("optimizer", "sgd");
+    cfg.set("lr", 0.5);
+    cfg.set("hbm_table.expected_max_items", 100);
+    cfg.set("hbm_table.init_range", 0.125);
+    RuntimeInfo rt(0, {0, 1});
+    HbmStorageOperator storage_op(cfg);
+    std::unique_ptr<Storage> storage = storage_op.create_storage(rt, 0);
+    HbmSparsePushOperator push_op(cfg);
+    HbmSparsePullOperator pull_op(cfg);
+    const std::vector<uint64_t> keys{7, 8, 9};
+    bool ok;
+    auto v = pull(pull_op, rt, storage.get(), keys, &ok);
+    EXPECT(ok);
+    for (size_t i = 0; i < keys.size(); ++i)
+        for (uint32_t c = 0; c < 2; ++c) {
+            const float w = pshbm_init_weight(0.125f, keys[i], c);
+            EXPECT(v[i * 2 + c] == w && w >= -0.125f && w < 0.125f);
+        }
+    EXPECT(v[0] != v[1] && v[0] != v[2]);
+    PSRequest req = make_push_request(keys, std::vector<float>{2.0f, 2.0f, 2.0f});  // gradient [arg, 1]
+    PSResponse resp;
+    Status status;
+    push_op.apply_async_push_request(rt, req, storage.get(), nullptr, resp);
+    resp >> status;
+    EXPECT(status.ok());
+    v = pull(pull_op, rt, storage.get(), keys, &ok);
+    EXPECT(ok);
+    for (size_t i = 0; i < keys.size(); ++i) {
+        EXPECT(v[i * 2] == pshbm_init_weight(0.125f, keys[i], 0) - 1.0f);
+        EXPECT(v[i * 2 + 1] == pshbm_init_weight(0.125f, keys[i], 1) - 0.5f);
+    }
+}
+
 int main(int argc, char** argv) {
     const std::string dir = argc > 1 ? argv[1] : "/tmp";
     Configure op_config;
@@ -732,6 +770,7 @@ int main(int argc, char** argv) {
     test_dense(dir);
     test_growth();
     test_operator_hyperparameters();
+    test_initial_weights();
     if (g_failed) {
         std::printf("FAILED: %d expectation(s)\n", g_failed);
         return 1;

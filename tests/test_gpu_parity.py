@@ -673,3 +673,53 @@ def test_hyperparameters_change_between_pushes(ps, orc, wl, opt):
     if opt == "ftrl":
         assert t.set_hyperparameters(alpha=0.0) == ps.INVALID_CONFIG
     t.close()
+
+
+@pytest.mark.parametrize("opt", ["sum", "sgd", "adagrad", "ftrl"])
+@pytest.mark.parametrize("dim", [5, 8, 128])
+@pytest.mark.parametrize("n", [300, 20000])      # the one-launch push; the chain of kernels
+def test_initial_weights_of_new_keys(ps, orc, wl, opt, dim, n):
+    """init_range > 0: a miss answers the weights an insertion would store, a push and an inserting
+    pull store them, bit for bit the oracle's (a pure function of key and column)."""
+    rng = np.random.default_rng(17)
+    rg = 0.05
+    t, r = pair(ps, orc, dim, opt, capacity=4 * n + 64, init_range=rg)
+    keys = wl.fresh_keys_np(rng, 3 * n)
+    a, b = t.pull(keys[:n]), r.pull(keys[:n])                  # nothing stored: every key misses
+    assert a[0] == b[0] == 0 and not a[2].any() and t.size() == 0
+    np.testing.assert_array_equal(a[1], b[1])
+    assert np.abs(a[1]).max() <= rg and a[1].std() > rg / 4
+    spot = rng.integers(0, n, 5)
+    for i in spot:
+        assert a[1][i, dim - 1] == np.float32(ps.init_weight(rg, int(keys[i]), dim - 1))
+    g = rng.normal(0, 1e-2, (n, dim)).astype(np.float32)
+    assert t.push(keys[:n], g) == 0 and r.push(keys[:n], g) == 0     # distinct keys: bit-exact
+    assert_same_table(t, r, exact=True)
+    q = np.concatenate([keys[: n // 2], keys[n: n + n // 4], keys[n: n + n // 4]])  # stored, new twice
+    rng.shuffle(q)
+    g = rng.normal(0, 1e-2, (q.size, dim)).astype(np.float32)
+    assert t.push(q, g) == 0 and r.push(q, g) == 0
+    assert_same_table(t, r, exact=False)
+    assert t.set(*(lambda d: (d["key"], d["value"]))(sorted_dump(r))) == 0
+    q = np.concatenate([keys[2 * n:], keys[:n // 3], keys[2 * n: 2 * n + 7]])
+    rng.shuffle(q)
+    a, b = t.pull(q, ps.PULL_INSERT_ON_MISS), r.pull(q, orc.PULL_INSERT_ON_MISS)
+    assert a[0] == b[0] == 0
+    np.testing.assert_array_equal(a[1], b[1])
+    np.testing.assert_array_equal(a[2], b[2])
+    assert_same_table(t, r, exact=True)
+    assert t.size() == r.size() == n + n // 4 + n
+    # the hyperparameters may change, the range stays
+    if opt != "sum":
+        o = dict(OPTS[opt]); o.pop("optimizer")
+        assert t.set_hyperparameters(**o) == 0
+        extra = wl.fresh_keys_np(rng, 40)
+        a, b = t.pull(extra), r.pull(extra)
+        np.testing.assert_array_equal(a[1], b[1])
+    t.close()
+
+
+def test_initial_weights_config_is_validated(ps):
+    for bad in (-0.5, float("inf"), float("nan")):
+        with pytest.raises(ps.PshbmError):
+            ps.Table(4, capacity=16, init_range=bad)
