@@ -195,8 +195,9 @@ int32_t pshbm_set_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_val
  * pass through a pair of pinned staging buffers. Replaces BaseKVTextFileLoadOperator::restore
  * (pico-ps/operator/LoadOperator.h:164-213) once the file is decoded; with PSHBM_LOAD_UNIQUE a key
  * that is already present (or repeated) fails with PSHBM_ERROR the way restore aborts on it
- * (:194,210), and the records loaded before the failing block stay. A record with a reserved key
- * is left out and the call returns PSHBM_ERROR after loading the others. */
+ * (:194,210), and the records loaded before the failing block stay. Without the flag a key that
+ * is present is overwritten, and of several records with one key any one may win. A record with a
+ * reserved key is left out and the call returns PSHBM_ERROR after loading the others. */
 int32_t pshbm_load(pshbm_table* t, const void* records, size_t n, uint32_t flags);
 
 /* Bulk dump of every (key, value) as the same records, in row-slab order, the same way (written by
