@@ -357,6 +357,19 @@ typedef struct pshbm_profile {
 int32_t pshbm_profile_enable(pshbm_table* t, int32_t on);
 int32_t pshbm_profile_read(pshbm_table* t, pshbm_profile* out);
 
+/* Budget of device memory for everything this library allocates on `device` in this process:
+ * tables, their growth (pshbm_reserve holds the old and the new arrays while it copies) and the
+ * per-batch workspaces. A call that would pass it fails with PSHBM_OUT_OF_MEMORY and changes
+ * nothing, exactly as when the device itself is full. bytes = 0 lifts the limit; a limit below what
+ * is in use only refuses further allocations. Stands where ShardStorageMemory::initialize's hard
+ * limit stands for host memory (pico-ps/storage/Storage.h:261-289, Storage.cpp:93-98: past it
+ * allocations throw, the storage turns unhealthy and operators answer Status::OOM); it lets a shard
+ * share the GPU with a learner's own buffers predictably. No GPU call is made. */
+int32_t pshbm_set_memory_limit(int32_t device, uint64_t bytes);
+/* Device bytes the library holds on `device` right now, and the limit (0 = none); either pointer
+ * may be NULL. The per-table figure is pshbm_memory_usage. */
+int32_t pshbm_device_memory(int32_t device, uint64_t* in_use, uint64_t* limit);
+
 /* Pinned host memory for request/response buffers of the host-pointer entry points. */
 int32_t pshbm_host_alloc(void** p, size_t bytes);
 int32_t pshbm_host_free(void* p);

@@ -31,7 +31,7 @@ SYMBOLS = [
     "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
     "pshbm_queue", "pshbm_queue_dev", "pshbm_queue_pairs", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
     "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
-    "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve", "pshbm_set_hyperparameters",
+    "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve", "pshbm_set_hyperparameters", "pshbm_set_memory_limit", "pshbm_device_memory",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
 ]
@@ -208,6 +208,8 @@ def lib():
         L.pshbm_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pshbm_memory_usage.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pshbm_get_stats.argtypes = [vp, C.POINTER(Stats)]
+        L.pshbm_set_memory_limit.argtypes = [i32, C.c_uint64]
+        L.pshbm_device_memory.argtypes = [i32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
         L.pshbm_host_alloc.argtypes = [C.POINTER(vp), sz]
         L.pshbm_host_free.argtypes = [vp]
         L.pshbm_profile_enable.argtypes = [vp, i32]
@@ -221,6 +223,22 @@ def lib():
 
 def value_floats(dim, optimizer):
     return lib().pshbm_value_floats(dim, optimizer)
+
+
+def set_memory_limit(device, nbytes):
+    """Budget of device memory for everything the library allocates on `device` (0 = none)."""
+    st = lib().pshbm_set_memory_limit(device, nbytes)
+    if st != OK:
+        raise PshbmError(st, "set_memory_limit: bad device")
+
+
+def device_memory(device=0):
+    """(bytes the library holds on the device, limit or 0)."""
+    a, b = C.c_uint64(), C.c_uint64()
+    st = lib().pshbm_device_memory(device, C.byref(a), C.byref(b))
+    if st != OK:
+        raise PshbmError(st, "device_memory: bad device")
+    return a.value, b.value
 
 
 def init_weight(init_range, key, column):

@@ -12,6 +12,7 @@
 #include <shared_mutex>
 #include <string>
 #include <thread>
+#include <unordered_map>
 #include <vector>
 
 #include "table.h"
@@ -78,6 +79,54 @@ void copy_parallel(void* dst, const void* src, size_t bytes) {
     }
     std::memcpy(dst, src, std::min(per, bytes));
     for (std::thread& w : workers) w.join();
+}
+
+// Device memory held by the tables of this process, per device, against an optional limit: the
+// role of ShardStorageMemory's hard limit (pico-ps/storage/Storage.h:261-289, Storage.cpp:93-98),
+// with the device's memory in the place of the host's. Every device allocation of the library goes
+// through dev_malloc / dev_free.
+constexpr int MAX_DEVICES = 64;
+struct DeviceBudget {
+    std::mutex mu;
+    uint64_t in_use = 0, limit = 0;  // limit 0: none
+    std::unordered_map<void*, size_t> sizes;
+};
+DeviceBudget g_budget[MAX_DEVICES];
+thread_local bool g_over_limit = false;  // the calling thread's last dev_malloc failed on the limit
+
+hipError_t dev_malloc(int device, void** p, size_t bytes) {
+    g_over_limit = false;
+    DeviceBudget& b = g_budget[device];
+    {
+        std::lock_guard<std::mutex> lk(b.mu);
+        if (b.limit && b.in_use + bytes > b.limit) {
+            g_over_limit = true;
+            return hipErrorOutOfMemory;
+        }
+        b.in_use += bytes;  // booked first, so that concurrent calls cannot pass the limit together
+    }
+    hipError_t e = ::hipMalloc(p, bytes);
+    std::lock_guard<std::mutex> lk(b.mu);
+    if (e != hipSuccess) {
+        b.in_use -= bytes;
+        return e;
+    }
+    b.sizes[*p] = bytes;
+    return hipSuccess;
+}
+
+hipError_t dev_free(int device, void* p) {
+    if (!p) return hipSuccess;
+    DeviceBudget& b = g_budget[device];
+    {
+        std::lock_guard<std::mutex> lk(b.mu);
+        auto it = b.sizes.find(p);
+        if (it != b.sizes.end()) {
+            b.in_use -= it->second;
+            b.sizes.erase(it);
+        }
+    }
+    return ::hipFree(p);
 }
 
 }  // namespace
@@ -184,6 +233,10 @@ int32_t fail(pshbm_table*, int32_t code, const char* fmt, ...) {
 
 int32_t hip_fail(pshbm_table* t, hipError_t e, const char* what) {
     int32_t code = (e == hipErrorOutOfMemory) ? PSHBM_OUT_OF_MEMORY : PSHBM_ERROR;
+    if (e == hipErrorOutOfMemory && g_over_limit) {
+        g_over_limit = false;
+        return fail(t, code, "%s: over the device memory limit (pshbm_set_memory_limit)", what);
+    }
     return fail(t, code, "%s: %s", what, hipGetErrorString(e));
 }
 
@@ -229,12 +282,12 @@ int32_t ensure(pshbm_table* t, DevBuf& b, size_t bytes) {
     if (bytes <= b.bytes) return PSHBM_OK;
     if (b.p) {
         HIP_TRY(t, hipDeviceSynchronize());
-        HIP_TRY(t, hipFree(b.p));
+        HIP_TRY(t, dev_free(t->device, b.p));
         b.p = nullptr;
         b.bytes = 0;
     }
     size_t want = round_up(bytes + bytes / 4, 256);
-    HIP_TRY(t, hipMalloc(&b.p, want));
+    HIP_TRY(t, dev_malloc(t->device, &b.p, want));
     b.bytes = want;
     return PSHBM_OK;
 }
@@ -454,7 +507,7 @@ int32_t ensure_bulk(pshbm_table* t) {
     if (t->pin[0]) return PSHBM_OK;
     for (int k = 0; k < 2; ++k) {
         HIP_TRY(t, hipHostMalloc(&t->pin[k], BULK_CHUNK_BYTES, hipHostMallocDefault));
-        HIP_TRY(t, hipMalloc(&t->dbuf[k], BULK_CHUNK_BYTES));
+        HIP_TRY(t, dev_malloc(t->device, &t->dbuf[k], BULK_CHUNK_BYTES));
         HIP_TRY(t, hipEventCreateWithFlags(&t->ev_copy[k], hipEventDisableTiming));
         HIP_TRY(t, hipEventCreateWithFlags(&t->ev_done[k], hipEventDisableTiming));
     }
@@ -469,28 +522,28 @@ void destroy_impl(pshbm_table* t) {
                       &t->ms_dead, &t->ms_tiles, &t->ms_lists, &t->ms_fe,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
-        if (b->p) (void)hipFree(b->p);
+        if (b->p) (void)dev_free(t->device, b->p);
     for (int k = 0; k < 2; ++k) {
         if (t->pin[k]) (void)hipHostFree(t->pin[k]);
-        if (t->dbuf[k]) (void)hipFree(t->dbuf[k]);
+        if (t->dbuf[k]) (void)dev_free(t->device, t->dbuf[k]);
         if (t->ev_copy[k]) (void)hipEventDestroy(t->ev_copy[k]);
         if (t->ev_done[k]) (void)hipEventDestroy(t->ev_done[k]);
     }
-    if (t->d.slots) (void)hipFree(t->d.slots);
-    if (t->d.rows) (void)hipFree(t->d.rows);
-    if (t->d.row_keys) (void)hipFree(t->d.row_keys);
-    if (t->d.counters) (void)hipFree(t->d.counters);
-    if (t->d.dirty) (void)hipFree(t->d.dirty);
-    if (t->d_hist) (void)hipFree(t->d_hist);
+    if (t->d.slots) (void)dev_free(t->device, t->d.slots);
+    if (t->d.rows) (void)dev_free(t->device, t->d.rows);
+    if (t->d.row_keys) (void)dev_free(t->device, t->d.row_keys);
+    if (t->d.counters) (void)dev_free(t->device, t->d.counters);
+    if (t->d.dirty) (void)dev_free(t->device, t->d.dirty);
+    if (t->d_hist) (void)dev_free(t->device, t->d_hist);
     if (t->h_counters) (void)hipHostFree(t->h_counters);
     if (t->h_hist) (void)hipHostFree(t->h_hist);
-    if (t->d_info) (void)hipFree(t->d_info);
+    if (t->d_info) (void)dev_free(t->device, t->d_info);
     if (t->h_info) (void)hipHostFree(t->h_info);
     if (t->h_fe) (void)hipHostFree(t->h_fe);
     if (t->h_small) (void)hipHostFree(t->h_small);
     for (pshbm_table::PullLane& l : t->lanes) {
-        if (l.keys.p) (void)hipFree(l.keys.p);
-        if (l.out.p) (void)hipFree(l.out.p);
+        if (l.keys.p) (void)dev_free(t->device, l.keys.p);
+        if (l.out.p) (void)dev_free(t->device, l.out.p);
         if (l.h_small) (void)hipHostFree(l.h_small);
         if (l.stream) (void)hipStreamDestroy(l.stream);
         if (l.done) (void)hipEventDestroy(l.done);
@@ -523,7 +576,7 @@ int32_t check_predicate(pshbm_table* t, const pshbm_predicate* w, pshbm_predicat
 }
 
 int32_t ensure_maint(pshbm_table* t) {
-    if (!t->d_info) HIP_TRY(t, hipMalloc(reinterpret_cast<void**>(&t->d_info), 4 * sizeof(uint32_t)));
+    if (!t->d_info) HIP_TRY(t, dev_malloc(t->device, reinterpret_cast<void**>(&t->d_info), 4 * sizeof(uint32_t)));
     if (!t->h_info) HIP_TRY(t, hipHostMalloc(reinterpret_cast<void**>(&t->h_info), 4 * sizeof(uint32_t), hipHostMallocDefault));
     if (!t->h_fe)
         HIP_TRY(t, hipHostMalloc(reinterpret_cast<void**>(&t->h_fe), ((size_t)t->d.vf + 1) * sizeof(double), hipHostMallocDefault));
@@ -608,7 +661,7 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
         g_error = std::string("no HIP device: ") + hipGetErrorString(e);
         return PSHBM_ERROR;
     }
-    if (cfg->device < 0 || cfg->device >= ndev) return bad("device ordinal out of range");
+    if (cfg->device < 0 || cfg->device >= ndev || cfg->device >= MAX_DEVICES) return bad("device ordinal out of range");
 
     pshbm_table* t = new (std::nothrow) pshbm_table();
     if (!t) return PSHBM_OUT_OF_MEMORY;
@@ -642,7 +695,10 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     t->keys_bytes = max_rows * 8;
 
     auto bail = [&](hipError_t err, const char* what) {
-        g_error = std::string(what) + ": " + hipGetErrorString(err);
+        const bool limit = err == hipErrorOutOfMemory && g_over_limit;
+        g_error = std::string(what) + ": " +
+                  (limit ? "over the device memory limit (pshbm_set_memory_limit)" : hipGetErrorString(err));
+        g_over_limit = false;
         int32_t code = err == hipErrorOutOfMemory ? PSHBM_OUT_OF_MEMORY : PSHBM_ERROR;
         destroy_impl(t);
         return code;
@@ -652,15 +708,15 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
         hipError_t e__ = (expr);                      \
         if (e__ != hipSuccess) return bail(e__, #expr); \
     } while (0)
-    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.slots), t->slots_bytes));
-    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.rows), t->rows_bytes));
-    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.row_keys), t->keys_bytes));
-    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.counters), CNT_WORDS * 4));
+    CREATE_TRY(dev_malloc(t->device, reinterpret_cast<void**>(&d.slots), t->slots_bytes));
+    CREATE_TRY(dev_malloc(t->device, reinterpret_cast<void**>(&d.rows), t->rows_bytes));
+    CREATE_TRY(dev_malloc(t->device, reinterpret_cast<void**>(&d.row_keys), t->keys_bytes));
+    CREATE_TRY(dev_malloc(t->device, reinterpret_cast<void**>(&d.counters), CNT_WORDS * 4));
     if (cfg->track_increment) {
-        CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&d.dirty), round_up(max_rows, 4)));
+        CREATE_TRY(dev_malloc(t->device, reinterpret_cast<void**>(&d.dirty), round_up(max_rows, 4)));
         CREATE_TRY(hipMemset(d.dirty, 0, round_up(max_rows, 4)));
     }
-    CREATE_TRY(hipMalloc(reinterpret_cast<void**>(&t->d_hist), 17 * 8));
+    CREATE_TRY(dev_malloc(t->device, reinterpret_cast<void**>(&t->d_hist), 17 * 8));
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_counters), CNT_WORDS * 4, hipHostMallocDefault));
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_hist), 17 * 8, hipHostMallocDefault));
     CREATE_TRY(hipStreamCreateWithFlags(&t->stream, hipStreamNonBlocking));
@@ -957,11 +1013,11 @@ int32_t pshbm_queue_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_g
         DevBuf nk, ng;
         size_t cap = std::max(need * 2, (size_t)65536);
         HIP_TRY(t, hipStreamSynchronize(s));
-        HIP_TRY(t, hipMalloc(&nk.p, cap * 8));
+        HIP_TRY(t, dev_malloc(t->device, &nk.p, cap * 8));
         nk.bytes = cap * 8;
-        hipError_t e = hipMalloc(&ng.p, cap * gb);
+        hipError_t e = dev_malloc(t->device, &ng.p, cap * gb);
         if (e != hipSuccess) {
-            (void)hipFree(nk.p);
+            (void)dev_free(t->device, nk.p);
             return hip_fail(t, e, "queue: hipMalloc");
         }
         ng.bytes = cap * gb;
@@ -969,8 +1025,8 @@ int32_t pshbm_queue_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_g
             HIP_TRY(t, hipMemcpy(nk.p, t->q_keys.p, t->q_n * 8, hipMemcpyDeviceToDevice));
             HIP_TRY(t, hipMemcpy(ng.p, t->q_grads.p, t->q_n * gb, hipMemcpyDeviceToDevice));
         }
-        if (t->q_keys.p) (void)hipFree(t->q_keys.p);
-        if (t->q_grads.p) (void)hipFree(t->q_grads.p);
+        if (t->q_keys.p) (void)dev_free(t->device, t->q_keys.p);
+        if (t->q_grads.p) (void)dev_free(t->device, t->q_grads.p);
         t->q_keys = nk;
         t->q_grads = ng;
     }
@@ -1430,17 +1486,17 @@ int32_t pshbm_reserve(pshbm_table* t, uint64_t expected_max_items) {
     uint64_t* n_keys = nullptr;
     uint8_t* n_dirty = nullptr;
     auto undo = [&](hipError_t e, const char* what) {
-        if (n_slots) (void)hipFree(n_slots);
-        if (n_rows) (void)hipFree(n_rows);
-        if (n_keys) (void)hipFree(n_keys);
-        if (n_dirty) (void)hipFree(n_dirty);
+        if (n_slots) (void)dev_free(t->device, n_slots);
+        if (n_rows) (void)dev_free(t->device, n_rows);
+        if (n_keys) (void)dev_free(t->device, n_keys);
+        if (n_dirty) (void)dev_free(t->device, n_dirty);
         return hip_fail(t, e, what);
     };
     hipError_t e;
-    if ((e = hipMalloc(reinterpret_cast<void**>(&n_slots), slots_bytes)) != hipSuccess) return undo(e, "reserve: hash array");
-    if ((e = hipMalloc(reinterpret_cast<void**>(&n_rows), rows_bytes)) != hipSuccess) return undo(e, "reserve: rows");
-    if ((e = hipMalloc(reinterpret_cast<void**>(&n_keys), keys_bytes)) != hipSuccess) return undo(e, "reserve: row keys");
-    if (t->d.dirty && (e = hipMalloc(reinterpret_cast<void**>(&n_dirty), dirty_bytes)) != hipSuccess)
+    if ((e = dev_malloc(t->device, reinterpret_cast<void**>(&n_slots), slots_bytes)) != hipSuccess) return undo(e, "reserve: hash array");
+    if ((e = dev_malloc(t->device, reinterpret_cast<void**>(&n_rows), rows_bytes)) != hipSuccess) return undo(e, "reserve: rows");
+    if ((e = dev_malloc(t->device, reinterpret_cast<void**>(&n_keys), keys_bytes)) != hipSuccess) return undo(e, "reserve: row keys");
+    if (t->d.dirty && (e = dev_malloc(t->device, reinterpret_cast<void**>(&n_dirty), dirty_bytes)) != hipSuccess)
         return undo(e, "reserve: marks");
     // rows keep their numbers: the slab is copied as it is and the hash array rebuilt from row_keys
     if ((e = hipMemsetAsync(n_slots, 0xFF, slots_bytes, s)) != hipSuccess) return undo(e, "reserve: fill");
@@ -1474,10 +1530,10 @@ int32_t pshbm_reserve(pshbm_table* t, uint64_t expected_max_items) {
     t->row_bits = 1;
     while ((1ull << t->row_bits) <= max_rows) ++t->row_bits;
     t->tombstones = 0;
-    (void)hipFree(o_slots);
-    (void)hipFree(o_rows);
-    (void)hipFree(o_keys);
-    if (o_dirty) (void)hipFree(o_dirty);
+    (void)dev_free(t->device, o_slots);
+    (void)dev_free(t->device, o_rows);
+    (void)dev_free(t->device, o_keys);
+    if (o_dirty) (void)dev_free(t->device, o_dirty);
     HIP_TRY(t, launch_reinsert(t->d, rows, s));
     ST_TRY(read_counters(t, s));
     if (t->h_counters[CNT_OVERFLOW]) return fail(t, PSHBM_FATAL, "reserve: the hash array overflowed");
@@ -1507,6 +1563,21 @@ int32_t pshbm_size(pshbm_table* t, uint64_t* n) {
     ST_TRY(read_counters(t, t->stream));
     t->size_bound = t->h_counters[CNT_ROWS];
     *n = t->h_counters[CNT_ROWS];
+    return PSHBM_OK;
+}
+
+int32_t pshbm_set_memory_limit(int32_t device, uint64_t bytes) {
+    if (device < 0 || device >= MAX_DEVICES) return PSHBM_INVALID_ID;
+    std::lock_guard<std::mutex> lk(g_budget[device].mu);
+    g_budget[device].limit = bytes;
+    return PSHBM_OK;
+}
+
+int32_t pshbm_device_memory(int32_t device, uint64_t* in_use, uint64_t* limit) {
+    if (device < 0 || device >= MAX_DEVICES) return PSHBM_INVALID_ID;
+    std::lock_guard<std::mutex> lk(g_budget[device].mu);
+    if (in_use) *in_use = g_budget[device].in_use;
+    if (limit) *limit = g_budget[device].limit;
     return PSHBM_OK;
 }
 

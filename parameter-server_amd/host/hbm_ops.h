@@ -56,6 +56,14 @@ inline pshbm_config table_config(const Configure& c) {
     return cfg;
 }
 
+// The server's memory limit, for the device: what ShardStorageMemory::singleton().initialize(soft,
+// hard) is for the host's memory (pico-ps/storage/Storage.cpp:93-98). Past `hard_limit` bytes held by
+// all tables on `device`, creating a shard, growing one or sizing a workspace fails with
+// OUT_OF_MEMORY, which the operators answer as Status::OOM; 0 lifts the limit.
+inline void initialize_device_memory(int32_t device, uint64_t hard_limit) {
+    PSHBM_SCHECK(pshbm_set_memory_limit(device, hard_limit) == PSHBM_OK, "bad device");
+}
+
 // One pshbm_table per local shard id, the way PmemHashMapShardStorage keeps one handle per shard
 // (storage/DCPmemory.h:400-442). HBM is volatile: need_remote_restore() is true.
 class HbmShardStorage : public Storage {

@@ -369,6 +369,59 @@ static void test_growth() {
     EXPECT(hst->shard_size(0) == 500 && hst->shard_size(1) == 500);
 }
 
+// A device memory limit (the hard limit of ShardStorageMemory, storage/Storage.cpp:93-98): growth
+// that would pass it answers Status::OOM and leaves the shard as it was; with the limit lifted the
+// same request goes through.
+static void test_memory_limit() {
+    Configure op_config;
+    op_config.set("dim", 64);
+    op_config.set("optimizer", "sum");
+    op_config.set("hbm_table.expected_max_items", 1000);
+    op_config.set("hbm_table.grow_limit", 1 << 20);
+    RuntimeInfo rt(0, {0});
+    HbmStorageOperator storage_op(op_config);
+    std::unique_ptr<Storage> storage = storage_op.create_storage(rt, 0);
+    auto* hst = static_cast<HbmShardStorage*>(storage.get());
+    uint64_t in_use = 0, limit = 1;
+    EXPECT(pshbm_device_memory(0, &in_use, &limit) == PSHBM_OK && in_use > 1000 * 64 * 4 && limit == 0);
+    // room for the present arrays and a little more, not for arrays of 8,000 rows beside them
+    initialize_device_memory(0, in_use + (1 << 20));
+    std::vector<char> block;
+    const size_t stride = 8 + 64 * 4;
+    const int n = 5000;
+    block.resize(n * stride);
+    for (int k = 0; k < n; ++k) {
+        const uint64_t key = 100 + k;
+        std::memcpy(&block[k * stride], &key, 8);
+        for (int c = 0; c < 64; ++c) {
+            const float g = (float)(k % 7);
+            std::memcpy(&block[k * stride + 8 + c * 4], &g, 4);
+        }
+    }
+    auto push = [&]() {
+        PSRequest req;
+        req << (int32_t)1 << (int32_t)1 << (int32_t)0 << (int32_t)n;
+        req.lazy().emplace_back(block.begin(), block.end());
+        PSResponse resp;
+        HbmSparsePushOperator push_op(op_config);
+        push_op.apply_async_push_request(rt, req, storage.get(), nullptr, resp);
+        Status status;
+        resp >> status;
+        return status;
+    };
+    Status st = push();
+    EXPECT(st.IsOOM());
+    EXPECT(hst->shard_size(0) == 0);
+    uint64_t after = 0;
+    EXPECT(pshbm_device_memory(0, &after, nullptr) == PSHBM_OK && after <= in_use + (1 << 20));
+    initialize_device_memory(0, 0);
+    st = push();
+    EXPECT(st.ok());
+    EXPECT(hst->shard_size(0) == (size_t)n);
+    storage.reset();
+    EXPECT(pshbm_device_memory(0, &after, nullptr) == PSHBM_OK && after < in_use);
+}
+
 // The learning rate belongs to the push operator (pico-ps/operator/Operator.h:53-57): two operators
 // registered with different rates push to one storage, each with its own.
 static void test_operator_hyperparameters() {
@@ -771,6 +824,7 @@ int main(int argc, char** argv) {
     test_growth();
     test_operator_hyperparameters();
     test_initial_weights();
+    test_memory_limit();
     if (g_failed) {
         std::printf("FAILED: %d expectation(s)\n", g_failed);
         return 1;

@@ -57,3 +57,18 @@ def test_null_handle_is_invalid_id(ps):
 def test_record_layout(ps):
     dt = ps.record_dtype(6)
     assert dt.itemsize == 8 + 24 and dt.fields["value"][1] == 8
+
+
+def test_memory_limit_is_kept_per_device_without_a_gpu(ps):
+    assert ps.device_memory(3) == (0, 0)
+    ps.set_memory_limit(3, 1 << 30)
+    assert ps.device_memory(3) == (0, 1 << 30) and ps.device_memory(2) == (0, 0)
+    ps.set_memory_limit(3, 0)
+    assert ps.device_memory(3) == (0, 0)
+    for bad in (-1, 64):
+        try:
+            ps.set_memory_limit(bad, 1)
+        except ps.PshbmError as e:
+            assert e.status == ps.INVALID_ID
+        else:
+            raise AssertionError("a device ordinal out of range was accepted")

@@ -723,3 +723,44 @@ def test_initial_weights_config_is_validated(ps):
     for bad in (-0.5, float("inf"), float("nan")):
         with pytest.raises(ps.PshbmError):
             ps.Table(4, capacity=16, init_range=bad)
+
+
+def test_device_memory_limit(ps, orc, wl):
+    """A budget of device memory for the library (the hard limit of the reference's
+    ShardStorageMemory, pico-ps/storage/Storage.cpp:93-98, for the device): what would pass it fails
+    with OUT_OF_MEMORY and changes nothing; what is released is given back."""
+    import gc
+    gc.collect()                                   # tables of earlier tests that nobody holds any more
+    base, limit = ps.device_memory(0)
+    assert limit == 0
+    dim = 16
+    t, r = pair(ps, orc, dim, "sgd", capacity=100_000)
+    used, _ = ps.device_memory(0)
+    assert used - base >= t.memory_usage() > 100_000 * (dim * 4 + 8)
+    keys = wl.table_keys_np(0, 60_000, seed=8)
+    g = np.random.default_rng(2).normal(0, 1, (60_000, dim)).astype(np.float32)
+    assert t.push(keys[:50_000], g[:50_000]) == 0 and r.push(keys[:50_000], g[:50_000]) == 0
+    assert_same_table(t, r, exact=True)            # (the first dump allocates the staging buffers)
+    used, _ = ps.device_memory(0)
+    ps.set_memory_limit(0, used + (1 << 20))
+    try:
+        assert ps.device_memory(0) == (used, used + (1 << 20))
+        with pytest.raises(ps.PshbmError) as e:
+            ps.Table(dim, capacity=1_000_000)
+        assert e.value.status == ps.OUT_OF_MEMORY and "limit" in str(e.value)
+        assert ps.device_memory(0)[0] == used                     # nothing of the failed table is left
+        assert t.reserve(1_000_000) == ps.OUT_OF_MEMORY and "limit" in t.last_error()
+        assert ps.device_memory(0)[0] == used and t.stats().capacity == 100_000
+        small = ps.Table(2, capacity=100, max_batch=64)           # what fits is still granted
+        small.close()
+        # the table works on as it was
+        assert t.push(keys[40_000:], g[40_000:]) == 0 and r.push(keys[40_000:], g[40_000:]) == 0
+        assert_same_table(t, r, exact=True)
+    finally:
+        ps.set_memory_limit(0, 0)
+    assert t.reserve(300_000) == 0 and r.reserve(300_000) == 0
+    assert_same_table(t, r, exact=True)
+    t.close()
+    assert ps.device_memory(0)[0] <= base
+    with pytest.raises(ps.PshbmError):
+        ps.set_memory_limit(64, 1)
