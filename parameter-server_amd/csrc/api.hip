@@ -327,13 +327,15 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
 // reading call since (the exclusive side of the same lock, SparsePushOperator.h:220).
 int32_t begin_op(pshbm_table* t, hipStream_t s, bool reads_only = false) {
     if (reads_only) {
-        if (!t->has_writer || t->writer_stream == s) return PSHBM_OK;  // nothing to wait for, or stream order
+        if (t->has_writer && t->writer_stream == s) return PSHBM_OK;  // stream order
         // one wait per reading stream and mutating call: later pulls on s are behind it already
         if (std::find(t->reader_streams.begin(), t->reader_streams.end(), s) != t->reader_streams.end())
             return PSHBM_OK;
-        HIP_TRY(t, hipEventRecord(t->order_ev, t->writer_stream));
-        HIP_TRY(t, hipStreamWaitEvent(s, t->order_ev, 0));
-        t->reader_streams.push_back(s);
+        if (t->has_writer) {
+            HIP_TRY(t, hipEventRecord(t->order_ev, t->writer_stream));
+            HIP_TRY(t, hipStreamWaitEvent(s, t->order_ev, 0));
+        }
+        t->reader_streams.push_back(s);  // (also before the first mutating call, which must wait for it)
         return PSHBM_OK;
     }
     if (t->has_writer && t->writer_stream != s) {
