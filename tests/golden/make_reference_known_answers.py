@@ -101,6 +101,23 @@ def native_ps_roundtrip(num_process=2, per_rank=150):
             "cite": "pico-ps/test/ps_predictor_native_ps_test.cpp:108-170", "ops": ops}
 
 
+def ha_load_pull(num_keys=2500):
+    """pico-ps/test/ps_ha_loader_puller_test.cpp:86-183: keys 0 .. N-1 are pushed once with the value
+    (key+1, key+2) in one batch, dumped, loaded into a new storage (LoadOperator::restore: every key
+    must be new) and pulled repeatedly; every pull answers key+2 in the value's second field.
+    (The reference uses 10000 keys and five pulls; the fixture keeps the key range dense from 0 and
+    the single push, with fewer keys and two pulls.)"""
+    keys = list(range(num_keys))
+    ops = [{"op": "push", "keys": keys, "grads": [[k + 1, k + 2] for k in keys]},
+           {"op": "expect_size", "value": num_keys},
+           {"op": "dump_load_roundtrip", "expect_size": num_keys}]
+    for _ in range(2):
+        ops.append({"op": "expect_pull", "keys": keys, "rows": [[k + 1, k + 2] for k in keys],
+                    "hit": [1] * num_keys})
+    return {"name": "ha_load_pull", "dim": 2, "optimizer": "SUM",
+            "cite": "pico-ps/test/ps_ha_loader_puller_test.cpp:86-183", "ops": ops}
+
+
 DENSE_BLOCK_SIZE = 5  # pico-ps/test/TestOps.h:270
 
 
@@ -156,7 +173,8 @@ def test_dense(num_process=3, per_rank=3):
 
 
 def main():
-    scenarios = [test_sparse(1), test_sparse(3), pmem_three_pushes(), native_ps_roundtrip(), test_dense()]
+    scenarios = [test_sparse(1), test_sparse(3), pmem_three_pushes(), native_ps_roundtrip(), ha_load_pull(),
+                 test_dense()]
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_known_answers.json")
     with open(out, "w") as f:
         json.dump({"scenarios": scenarios}, f, separators=(",", ":"))
