@@ -14,7 +14,8 @@
 //   pso_pull, pso_set, pso_dump, pso_iterate, pso_load, pso_clear, pso_size
 //       associative-container semantics; pinned by a brute-force std::map model, by the
 //       invariants of the reference's test_sparse (pico-ps/test/ps_service_test.cpp:104-184)
-//       and by its known answers (tests/golden/reference_known_answers.json).
+//       and by its known answers (tests/golden/reference_known_answers.json), among them the
+//       map contract's own unit tests (pico-ps/test/ps_pmem_test.cpp:110-193).
 //   pso_aggregate, pso_push (SUM), pso_queue/pso_store (SUM)
 //       pinned by the reference's integer test operator: pushing arg=key c times gives
 //       sum = key*c, count = c (pico-ps/test/TestOps.h:98-117,171-172;

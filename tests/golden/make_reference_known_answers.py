@@ -118,6 +118,51 @@ def ha_load_pull(num_keys=2500):
             "cite": "pico-ps/test/ps_ha_loader_puller_test.cpp:86-183", "ops": ops}
 
 
+def hash_map_contract():
+    """pico-ps/test/ps_pmem_test.cpp:110-157: the map contract the operators use (lock_find,
+    safe_insert, safe_set, safe_erase; storage/KVShardStorage.h:786-834) on int -> int. The test's
+    `it->second = 3` through an accessor and its safe_set calls are upserts here; its second
+    safe_insert of key 0, which must leave the stored 2 alone, is a pull of key 0."""
+    def pull(keys, vals):
+        return {"op": "expect_pull", "keys": keys, "rows": [[v if v is not None else 0] for v in vals],
+                "hit": [int(v is not None) for v in vals]}
+    ops = [{"op": "set", "keys": [0], "values": [[2]]},           # safe_insert(mp, 0, 2)
+           pull([0, 1], [2, None]),                               # the value stays 2; key 1 is absent
+           {"op": "set", "keys": [0], "values": [[3]]},           # it->second = 3
+           {"op": "set", "keys": [1], "values": [[4]]},
+           {"op": "set", "keys": [2], "values": [[5]]},
+           {"op": "set", "keys": [3], "values": [[6]]},
+           {"op": "set", "keys": [4], "values": [[7]]},
+           pull([5], [None]),
+           {"op": "expect_values", "values": [3, 4, 5, 6, 7]},
+           {"op": "set", "keys": [3], "values": [[6666]]},
+           pull([3], [6666]),
+           {"op": "erase", "keys": [3], "erased": 1},
+           pull([3], [None]),
+           {"op": "expect_values", "values": [3, 4, 5, 7]},
+           {"op": "expect_size", "value": 4}]
+    return {"name": "hash_map_contract", "dim": 1, "optimizer": "SUM",
+            "cite": "pico-ps/test/ps_pmem_test.cpp:110-157", "ops": ops}
+
+
+def concurrent_erase():
+    """pico-ps/test/ps_pmem_test.cpp:159-193: ten rounds of: insert keys 0..99 with value = key,
+    size 100, ten erasers take the overlapping ranges [10 i, 10 i + 20) -- every key from 10 on is
+    erased twice, keys 100..109 were never there --, afterwards no key is found and the size is 0.
+    The ten ranges arrive as one batch (the reference's threads race; the outcome is the same)."""
+    ops = []
+    keys = list(range(100))
+    ranges = [k for i in range(10) for k in range(10 * i, 10 * i + 20)]
+    for _ in range(10):
+        ops.append({"op": "set", "keys": keys, "values": [[k] for k in keys]})
+        ops.append({"op": "expect_size", "value": 100})
+        ops.append({"op": "erase", "keys": ranges, "erased": 100})
+        ops.append({"op": "expect_pull", "keys": keys, "rows": [[0]] * 100, "hit": [0] * 100})
+        ops.append({"op": "expect_size", "value": 0})
+    return {"name": "concurrent_erase", "dim": 1, "optimizer": "SUM",
+            "cite": "pico-ps/test/ps_pmem_test.cpp:159-193", "ops": ops}
+
+
 DENSE_BLOCK_SIZE = 5  # pico-ps/test/TestOps.h:270
 
 
@@ -174,7 +219,7 @@ def test_dense(num_process=3, per_rank=3):
 
 def main():
     scenarios = [test_sparse(1), test_sparse(3), pmem_three_pushes(), native_ps_roundtrip(), ha_load_pull(),
-                 test_dense()]
+                 hash_map_contract(), concurrent_erase(), test_dense()]
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_known_answers.json")
     with open(out, "w") as f:
         json.dump({"scenarios": scenarios}, f, separators=(",", ":"))

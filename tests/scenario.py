@@ -1,7 +1,7 @@
 """Runs a golden scenario (tests/golden/reference_known_answers.json) against a backend.
 
 A backend is anything with the method set shared by oracle.Oracle and the product's Table:
-pull / push / queue / store / dump / load / for_each / erase_if / clear / size. `make` builds a fresh backend of the
+pull / push / queue / store / set / erase / dump / load / for_each / erase_if / clear / size. `make` builds a fresh backend of the
 scenario's shape (used for the dump -> load round trip into a new storage).
 """
 import json
@@ -43,6 +43,18 @@ def run(scn, make, predicate):
         elif kind == "store":
             assert b.store() == 0, where
             assert b.queued() == 0, where
+        elif kind == "set":
+            assert b.set(np.array(op["keys"], dtype=np.uint64),
+                         np.array(op["values"], dtype=np.float32)) == 0, where
+        elif kind == "erase":
+            st, erased = b.erase(np.array(op["keys"], dtype=np.uint64))
+            assert st == 0 and erased == op["erased"], where
+        elif kind == "expect_values":
+            # every stored value, in ascending order (the reference walks the map and sorts)
+            st, rec = b.dump()
+            assert st == 0, where
+            np.testing.assert_array_equal(np.sort(rec["value"][:, 0]),
+                                          np.array(op["values"], dtype=np.float32), err_msg=where)
         elif kind == "expect_size":
             assert b.size() == op["value"], where
         elif kind == "clear":

@@ -95,3 +95,35 @@ def test_pulls_on_several_streams_between_pushes(ps, orc, wl):
             np.testing.assert_array_equal(out.cpu().numpy(), rows)
             np.testing.assert_array_equal(hit.cpu().numpy(), rhit)
     t.close()
+
+
+def test_concurrent_erasers_with_overlapping_ranges(ps):
+    """pico-ps/test/ps_pmem_test.cpp:159-193 with its threads: ten rounds of inserting keys 0..99 and
+    ten threads erasing the overlapping ranges [10 i, 10 i + 20) at once; afterwards no key is found
+    and the table is empty. Every key is erased exactly once, whichever thread gets there first."""
+    t = ps.Table(1, ps.OPT_SUM, capacity=256)
+    keys = np.arange(100, dtype=np.uint64)
+    vals = keys.astype(np.float32).reshape(-1, 1)
+    for _ in range(10):
+        assert t.set(keys, vals) == 0 and t.size() == 100
+        erased = [0] * 10
+        errors = []
+
+        def eraser(i):
+            try:
+                st, n = t.erase(np.arange(10 * i, 10 * i + 20, dtype=np.uint64))
+                assert st == 0
+                erased[i] = n
+            except Exception as e:  # noqa: BLE001 - reported by the main thread
+                errors.append(repr(e))
+
+        threads = [threading.Thread(target=eraser, args=(i,)) for i in range(10)]
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join()
+        assert not errors, errors
+        assert sum(erased) == 100
+        st, rows, hit = t.pull(keys)
+        assert st == 0 and not hit.any() and not rows.any() and t.size() == 0
+    t.close()
