@@ -127,3 +127,93 @@ def test_concurrent_erasers_with_overlapping_ranges(ps):
         st, rows, hit = t.pull(keys)
         assert st == 0 and not hit.any() and not rows.any() and t.size() == 0
     t.close()
+
+
+def test_several_tables_pushed_at_once(ps, orc, wl):
+    """A server holds several shards, each a table of its own, and its threads push to them at the
+    same time (pico-ps/service/Server.h:24-26): three tables of different shapes, one thread each,
+    batches of one sort tile up to more than 2^20 keys, so that sort passes of different tables --
+    whose tiles wait for each other's counts -- share the device."""
+    shapes = [(16, dict(optimizer=ps.OPT_SGD, lr=0.5)), (8, dict(optimizer=ps.OPT_SUM)),
+              (64, dict(optimizer=ps.OPT_SGD, lr=0.25))]
+    n = 400_000
+    sizes = [300_000, 3000, 70_000, 1_200_000, 20_000, 300_000]
+    tables, oracles, work = [], [], []
+    for w, (dim, opt) in enumerate(shapes):
+        rng = np.random.default_rng(40 + w)
+        t = ps.Table(dim, capacity=n + 50_000, **opt)
+        r = orc.Oracle(dim, capacity=n + 50_000, **opt)
+        keys = wl.table_keys_np(0, n, seed=20 + w)
+        vals = rng.integers(-8, 9, (n, dim)).astype(np.float32)
+        assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+        mine = []
+        for b in sizes:
+            q = wl.zipf_batch_np(rng, n, 1.1, b, seed=20 + w)
+            q[:50] = wl.fresh_keys_np(rng, 50)
+            g = rng.integers(-2, 3, (b, dim)).astype(np.float32)   # integer sums, steps of 1/2 or 1/4: exact
+            mine.append((q, g))
+        tables.append(t), oracles.append(r), work.append(mine)
+    errors = []
+
+    def worker(w):
+        try:
+            for q, g in work[w]:
+                assert tables[w].push(q, g) == 0
+                st, rows, hit = tables[w].pull(q[:2000])
+                assert st == 0 and hit.all()
+        except Exception as e:  # noqa: BLE001 - reported by the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(w,)) for w in range(len(shapes))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    for w, (t, r) in enumerate(zip(tables, oracles)):
+        for q, g in work[w]:
+            assert r.push(q, g) == 0
+        a = np.sort(t.dump()[1], order="key")
+        b = np.sort(r.dump()[1], order="key")
+        np.testing.assert_array_equal(a["key"], b["key"])
+        np.testing.assert_array_equal(a["value"], b["value"])
+        t.close()
+
+
+def test_several_tables_on_their_own_streams(ps, orc, wl):
+    """The same with device buffers: pushes to three tables are enqueued on three streams without
+    waiting in between, so their kernels really run side by side; the sort's bounded waits must not
+    time out (a time-out would surface as PSHBM_FATAL in size())."""
+    import torch
+    dims = [16, 8, 32]
+    n, b = 500_000, 1_000_000                       # 245 sort tiles per push: one tile per compute unit
+    tables, oracles, streams, bufs = [], [], [], []
+    for w, dim in enumerate(dims):
+        rng = np.random.default_rng(60 + w)
+        t = ps.Table(dim, ps.OPT_SGD, lr=0.5, capacity=n + 1000, max_batch=b)
+        r = orc.Oracle(dim, orc.OPT_SGD, lr=0.5, capacity=n + 1000)
+        keys = wl.table_keys_np(0, n, seed=30 + w)
+        vals = rng.integers(-8, 9, (n, dim)).astype(np.float32)
+        assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+        rounds = []
+        for _ in range(4):
+            q = wl.zipf_batch_np(rng, n, 1.05, b, seed=30 + w)
+            g = rng.integers(-2, 3, (b, dim)).astype(np.float32)
+            rounds.append((q, g, torch.from_numpy(q.view(np.int64)).cuda(), torch.from_numpy(g).cuda()))
+        tables.append(t), oracles.append(r), bufs.append(rounds)
+        streams.append(torch.cuda.Stream())
+    torch.cuda.synchronize()
+    for k in range(4):
+        for w, t in enumerate(tables):
+            q, g, dq, dg = bufs[w][k]
+            assert t.push_dev(dq.data_ptr(), dg.data_ptr(), b, 0, streams[w].cuda_stream) == 0
+    torch.cuda.synchronize()
+    for w, (t, r) in enumerate(zip(tables, oracles)):
+        assert t.size() == n                        # (also reads the sort's error flag)
+        for q, g, _, _ in bufs[w]:
+            assert r.push(q, g) == 0
+        a = np.sort(t.dump()[1], order="key")
+        bb = np.sort(r.dump()[1], order="key")
+        np.testing.assert_array_equal(a["key"], bb["key"])
+        np.testing.assert_array_equal(a["value"], bb["value"])
+        t.close()
