@@ -859,7 +859,7 @@ __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* _
     T acc = vzero(T());
     if (lane_on) {
         if (g == 0) acc = part_val[((u64)w * 2 + 1) * units + col];
-        if (fs >= fe) {
+        if (n_windows == 0 || fs >= fe) {  // no window sums were made, or no whole window inside
             acc = vadd(acc, strided_sum(part_val + col, A + g, B + 1, P, 2 * (u64)units));
         } else {
             acc = vadd(acc, strided_sum(part_val + col, A + g, fs, P, 2 * (u64)units));
@@ -1287,9 +1287,14 @@ hipError_t launch_segreduce(const TableDev& t, const u32* sorted_row, const u32*
 
 // A window lies wholly inside a run only if the run entered it from the window before, so window 0
 // never does: with fewer than two whole windows there is nothing for fixup_windows_kernel to add up,
-// and fixup_kernel (which is told so by n_windows = 0) looks at no window.
-inline u32 window_count(u32 n_chunks) {
-    return n_chunks < 2 * WINDOW ? 0u : (n_chunks + WINDOW - 1) / WINDOW;
+// and fixup_kernel (which is told so by n_windows = 0) looks at no window. Windows are also left
+// out while the longest chain they could shorten is short anyway: a run over all n_chunks chunks
+// is found in n_chunks / 64 steps over the chunk headers and added by the P lane groups of one
+// wavefront, four loads in flight each, in n_chunks / (4 P) steps; up to 8 such steps (about as
+// long as the launch that would avoid them) fixup_windows_kernel costs more than it can save.
+inline u32 window_count(u32 n_chunks, u32 P) {
+    if (n_chunks < 2 * WINDOW || n_chunks <= 32u * P) return 0u;
+    return (n_chunks + WINDOW - 1) / WINDOW;
 }
 
 hipError_t launch_fixup_windows(const TableDev& t, size_t n, const float* grads, const uint4* part_hdr,
@@ -1297,7 +1302,7 @@ hipError_t launch_fixup_windows(const TableDev& t, size_t n, const float* grads,
     if (n == 0) return hipSuccess;
     const bool v4 = vec4_ok(t, grads, part_val) && vec4_ok(t, win_val);  // the layout launch_segreduce chose
     const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
-    const u32 n_windows = window_count(g.n_chunks);
+    const u32 n_windows = window_count(g.n_chunks, g.p);
     if (n_windows == 0) return hipSuccess;
     dim3 grid((n_windows + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per window
     if (v4)
@@ -1317,7 +1322,7 @@ hipError_t launch_fixup(const TableDev& t, size_t n, const float* grads, const u
     const bool v4 = vec4_ok(t, grads, part_val) && vec4_ok(t, win_val);
     const SegGeom g = seg_geometry(t.dim, v4 ? 4 : 1, n);
     if (g.n_chunks <= 1) return hipSuccess;  // no border, no run across one
-    const u32 n_windows = window_count(g.n_chunks);
+    const u32 n_windows = window_count(g.n_chunks, g.p);
     dim3 grid((g.n_chunks + BLOCK / 64 - 1) / (BLOCK / 64), g.col_blocks);  // a wavefront per chunk
     if (v4)
         fixup_kernel<float4><<<grid, BLOCK, 0, s>>>(

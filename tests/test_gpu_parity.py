@@ -138,7 +138,7 @@ def test_aggregation_exact_with_integer_gradients(ps, orc, dim):
     assert_same_table(t, r, exact=True)
     # one key only: a single run spanning every chunk of the segmented reduction; the long one also
     # spans many 64-chunk windows of the border fix-up, and shares the batch with two more long runs
-    for n in (9000, 150000):
+    for n in (9000, 40000, 150000):
         keys = np.full(n, 77, np.uint64)
         keys[n // 2: n // 2 + n // 5] = 78
         keys[: n // 7] = 1999
