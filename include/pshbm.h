@@ -370,7 +370,10 @@ int32_t pshbm_set_memory_limit(int32_t device, uint64_t bytes);
  * may be NULL. The per-table figure is pshbm_memory_usage. */
 int32_t pshbm_device_memory(int32_t device, uint64_t* in_use, uint64_t* limit);
 
-/* Pinned host memory for request/response buffers of the host-pointer entry points. */
+/* Pinned (page-locked) host memory for request/response buffers of the host-pointer entry points.
+ * Buffers from here (or from hipHostMalloc) spare the staging copies: pshbm_pull and pshbm_push
+ * hand batches of up to 1 MB to the kernels as they lie, pshbm_load and pshbm_dump let the copy
+ * engine reach them directly. Pageable buffers work everywhere, through the library's own staging. */
 int32_t pshbm_host_alloc(void** p, size_t bytes);
 int32_t pshbm_host_free(void* p);
 

@@ -308,10 +308,17 @@ class Table:
         return (lib().pshbm_last_error(self._h) or b"").decode()
 
     # -- host-array entry points
-    def pull(self, keys, flags=0):
+    def pull(self, keys, flags=0, out=None, hit=None):
+        """(status, rows, hit mask). `out` / `hit`: arrays of the caller to fill; when they and the
+        keys lie in page-locked memory (pinned_empty) a small pull uses them without a copy."""
         k = _u64(keys)
-        out = np.empty((k.size, self.dim), dtype=np.float32)
-        hit = np.empty(k.size, dtype=np.uint8)
+        if out is None:
+            out = np.empty((k.size, self.dim), dtype=np.float32)
+        if hit is None:
+            hit = np.empty(k.size, dtype=np.uint8)
+        if out.dtype != np.float32 or out.size != k.size * self.dim or not out.flags.c_contiguous or \
+                hit.dtype != np.uint8 or hit.size != k.size or not hit.flags.c_contiguous:
+            raise ValueError("out: contiguous float32 n x dim; hit: contiguous uint8 n")
         st = lib().pshbm_pull(self._h, k.ctypes.data, k.size, out.ctypes.data, hit.ctypes.data, flags)
         return st, out, hit
 

@@ -808,6 +808,13 @@ int32_t pshbm_pull(pshbm_table* t, const uint64_t* keys, size_t n, float* out_ro
     hipStream_t s = lane->stream;
     const size_t key_room = round_up(key_bytes, 256);
     if (key_room + out_bytes + n <= SMALL_HOST_BYTES) {
+        // Buffers of the caller that are page-locked already (pshbm_host_alloc) are used as they
+        // lie: the kernel reads the keys from them and writes the rows into them.
+        if (is_pinned_host(keys, key_bytes) && is_pinned_host(out_rows, out_bytes) && (!hit || is_pinned_host(hit, n))) {
+            ST_TRY(pshbm_pull_dev(t, keys, n, out_rows, hit, flags, s));
+            HIP_TRY(t, hipStreamSynchronize(s));
+            return PSHBM_OK;
+        }
         ST_TRY(lane_pinned(t, lane));
         // The kernel reads the keys from the pinned buffer and writes rows and hit mask into it:
         // page-locked host memory is mapped into the device's address space, and for a few
@@ -883,16 +890,22 @@ int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, siz
     const size_t key_bytes = n * 8, val_bytes = n * (size_t)t->d.dim * 4;
     const size_t key_room = round_up(key_bytes, 256);
     if (key_room + val_bytes <= SMALL_HOST_BYTES) {
-        // the kernels read the batch from a lane's pinned buffer; the thread waits for its own
-        // batch only, so the next thread's push is queued behind it meanwhile
+        // the kernels read the batch from a lane's pinned buffer (or from the caller's buffers, if
+        // those are page-locked already); the thread waits for its own batch only, so the next
+        // thread's push is queued behind it meanwhile
         std::unique_lock<std::mutex> ll;
         pshbm_table::PullLane* lane = take_lane(t, ll);
-        ST_TRY(lane_pinned(t, lane));
-        char* h = static_cast<char*>(lane->h_small);
-        std::memcpy(h, keys, key_bytes);
-        std::memcpy(h + key_room, grads, val_bytes);
-        int32_t st = pshbm_push_dev(t, reinterpret_cast<const uint64_t*>(h),
-                                    reinterpret_cast<const float*>(h + key_room), n, flags, s);
+        const uint64_t* dk = keys;
+        const float* dv = grads;
+        if (!(is_pinned_host(keys, key_bytes) && is_pinned_host(grads, val_bytes))) {
+            ST_TRY(lane_pinned(t, lane));
+            char* h = static_cast<char*>(lane->h_small);
+            std::memcpy(h, keys, key_bytes);
+            std::memcpy(h + key_room, grads, val_bytes);
+            dk = reinterpret_cast<const uint64_t*>(h);
+            dv = reinterpret_cast<const float*>(h + key_room);
+        }
+        int32_t st = pshbm_push_dev(t, dk, dv, n, flags, s);
         HIP_TRY(t, hipEventRecord(lane->done, s));
         HIP_TRY(t, hipEventSynchronize(lane->done));
         return st;

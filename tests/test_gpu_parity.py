@@ -764,3 +764,35 @@ def test_device_memory_limit(ps, orc, wl):
     assert ps.device_memory(0)[0] <= base
     with pytest.raises(ps.PshbmError):
         ps.set_memory_limit(64, 1)
+
+
+@pytest.mark.parametrize("n", [300, 5000, 40000])   # the one-launch push; the chain; beyond 1 MB: staged
+def test_page_locked_request_buffers_are_used_in_place(ps, orc, wl, n):
+    """Small pulls and pushes whose buffers lie in page-locked memory (pshbm_host_alloc) hand them to
+    the kernels as they are; the results are those of pageable buffers."""
+    rng = np.random.default_rng(31)
+    dim = 16
+    t, r = pair(ps, orc, dim, "adagrad", capacity=4 * n + 1000)
+    keys = wl.fresh_keys_np(rng, 2 * n)
+    q = np.concatenate([keys[:n // 2], keys[:n // 2]])
+    rng.shuffle(q)
+    pk = ps.pinned_empty(q.size, np.uint64)
+    pg = ps.pinned_empty((q.size, dim), np.float32)
+    out = ps.pinned_empty((q.size, dim), np.float32)
+    hit = ps.pinned_empty(q.size, np.uint8)
+    for step in range(3):
+        pk[:] = q
+        pg[:] = rng.integers(-3, 4, (q.size, dim)).astype(np.float32)
+        assert t.push(pk, pg) == 0 and r.push(q, np.array(pg)) == 0
+        out[:] = -7.0
+        st, rows, h = t.pull(pk, 0, out=out, hit=hit)
+        b = r.pull(q)
+        assert st == 0 and rows is out
+        np.testing.assert_allclose(out, b[1], rtol=RTOL, atol=ATOL)
+        np.testing.assert_array_equal(hit, b[2])
+        # mixed: page-locked keys, pageable rows -> the staged path
+        st, rows2, h2 = t.pull(pk)
+        np.testing.assert_array_equal(rows2, out)
+        q = np.concatenate([keys[step * 10: step * 10 + n // 2], keys[n: n + n // 2]])
+    assert_same_table(t, r, exact=False)
+    t.close()
