@@ -855,14 +855,19 @@ int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_gr
 
 // Keys and their n x `floats` values from host memory to where kernels on stream s can read them:
 // *dk / *dv. Larger batches are copied into st_keys / st_vals. Small ones are copied into the pinned
-// buffer and read from there by the kernels themselves (page-locked memory is mapped into the
-// device's address space; the buffer is in use until the stream has been waited for). The caller
-// holds st_mu.
+// buffer (unless the caller's buffers are page-locked themselves) and read from there by the
+// kernels (page-locked memory is mapped into the device's address space; the buffer is in use
+// until the stream has been waited for). The caller holds st_mu.
 static int32_t stage_keys_values(pshbm_table* t, const uint64_t* keys, const float* vals, size_t n,
                                  size_t floats, hipStream_t s, const uint64_t** dk, const float** dv) {
     const size_t key_bytes = n * 8, val_bytes = n * floats * 4;
     const size_t key_room = round_up(key_bytes, 256);
     if (key_room + val_bytes <= SMALL_HOST_BYTES) {
+        if (is_pinned_host(keys, key_bytes) && is_pinned_host(vals, val_bytes)) {  // usable as they lie
+            *dk = keys;
+            *dv = vals;
+            return PSHBM_OK;
+        }
         ST_TRY(ensure_small(t));
         char* h = static_cast<char*>(t->h_small);
         std::memcpy(h, keys, key_bytes);

@@ -795,4 +795,10 @@ def test_page_locked_request_buffers_are_used_in_place(ps, orc, wl, n):
         np.testing.assert_array_equal(rows2, out)
         q = np.concatenate([keys[step * 10: step * 10 + n // 2], keys[n: n + n // 2]])
     assert_same_table(t, r, exact=False)
+    m = min(n, 3000)                                   # set from page-locked buffers, in place when small
+    pv = ps.pinned_empty((m, t.value_floats), np.float32)
+    pv[:] = rng.integers(1, 9, (m, t.value_floats)).astype(np.float32)
+    pk[:m] = keys[:m]
+    assert t.set(pk[:m], pv) == 0 and r.set(keys[:m], np.array(pv)) == 0
+    assert_same_table(t, r, exact=False)
     t.close()
