@@ -66,7 +66,18 @@ def test_random_operation_sequences(ps, orc, wl, seed):
             q = batch(n)
             g = grads(q.size)
             flags = ps.PUSH_NO_INSERT if op == "push_no_insert" else 0
-            a, b = t.push(q, g, flags), r.push(q, g, flags)
+            how = int(rng.integers(0, 3))
+            if how == 0:                                 # the wire layout of a push block
+                pairs = np.empty(q.size, np.dtype([("key", np.uint64), ("value", np.float32, (dim,))]))
+                pairs["key"], pairs["value"] = q, g
+                a = t.push_pairs(pairs, flags)
+            elif how == 1:                               # page-locked request buffers
+                pk, pg = ps.pinned_empty(q.size, np.uint64), ps.pinned_empty((q.size, dim), np.float32)
+                pk[:], pg[:] = q, g
+                a = t.push(pk, pg, flags)
+            else:
+                a = t.push(q, g, flags)
+            b = r.push(q, g, flags)
             assert a == b, (op, a, b)
         elif op == "queue_store":
             for _ in range(int(rng.integers(1, 4))):
@@ -85,7 +96,14 @@ def test_random_operation_sequences(ps, orc, wl, seed):
         elif op in ("pull", "pull_insert"):
             q = universe[rng.integers(0, universe.size, n)]
             flags = ps.PULL_INSERT_ON_MISS if op == "pull_insert" else 0
-            a, b = t.pull(q, flags), r.pull(q, flags)
+            if rng.random() < 0.3:                       # page-locked buffers, used in place when small
+                pk = ps.pinned_empty(q.size, np.uint64)
+                pk[:] = q
+                a = t.pull(pk, flags, out=ps.pinned_empty((q.size, dim), np.float32),
+                           hit=ps.pinned_empty(q.size, np.uint8))
+            else:
+                a = t.pull(q, flags)
+            b = r.pull(q, flags)
             assert a[0] == b[0]
             if a[0] == 0:
                 np.testing.assert_array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
