@@ -211,6 +211,11 @@ int32_t pshbm_dump(pshbm_table* t, void* records, size_t capacity_records, size_
  * KVShardIterator::iterate_batch_as_binary_archive (pico-ps/storage/KVShardStorage.h:64-87).
  * *n_out < batch marks the end. */
 int32_t pshbm_iterate(pshbm_table* t, size_t offset, size_t batch, void* records, size_t* n_out);
+/* The keys alone of the same slice, in the same order: what a walk needs that only decides by key,
+ * such as the purge after a change of the shard layout (ShardUpdateContextOperator::
+ * apply_purge_request, pico-ps/operator/UpdateContextOperator.h:143-196, erases every key whose
+ * partition is no longer this shard) -- 8 bytes per record over the link instead of the record. */
+int32_t pshbm_iterate_keys(pshbm_table* t, size_t offset, size_t batch, uint64_t* keys, size_t* n_out);
 
 /* ---- for-each and erase-if ------------------------------------------------------------------
  * The reference's hooks for_each(key, value) and erase_if(key, value) are C++ virtuals

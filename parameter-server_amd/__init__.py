@@ -30,7 +30,7 @@ SYMBOLS = [
     "pshbm_create", "pshbm_destroy", "pshbm_last_error", "pshbm_value_floats", "pshbm_init_weight",
     "pshbm_pull", "pshbm_pull_dev", "pshbm_push", "pshbm_push_dev", "pshbm_push_pairs",
     "pshbm_queue", "pshbm_queue_dev", "pshbm_queue_pairs", "pshbm_queued", "pshbm_store", "pshbm_store_dev",
-    "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate",
+    "pshbm_set", "pshbm_set_dev", "pshbm_load", "pshbm_dump", "pshbm_iterate", "pshbm_iterate_keys",
     "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve", "pshbm_set_hyperparameters", "pshbm_set_memory_limit", "pshbm_device_memory",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
@@ -208,6 +208,7 @@ def lib():
         L.pshbm_size.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pshbm_memory_usage.argtypes = [vp, C.POINTER(C.c_uint64)]
         L.pshbm_get_stats.argtypes = [vp, C.POINTER(Stats)]
+        L.pshbm_iterate_keys.argtypes = [vp, sz, sz, vp, C.POINTER(sz)]
         L.pshbm_set_memory_limit.argtypes = [i32, C.c_uint64]
         L.pshbm_device_memory.argtypes = [i32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
         L.pshbm_host_alloc.argtypes = [C.POINTER(vp), sz]
@@ -378,6 +379,13 @@ class Table:
         got = C.c_size_t()
         st = lib().pshbm_iterate(self._h, offset, batch, rec.ctypes.data, C.byref(got))
         return st, rec[: got.value]
+
+    def iterate_keys(self, offset, batch):
+        """(status, keys of records [offset, offset + batch)): the keys alone, in record order."""
+        keys = np.empty(batch, dtype=np.uint64)
+        got = C.c_size_t()
+        st = lib().pshbm_iterate_keys(self._h, offset, batch, keys.ctypes.data, C.byref(got))
+        return st, keys[: got.value]
 
     def increment_size(self):
         n = C.c_uint64()

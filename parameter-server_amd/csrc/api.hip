@@ -1267,6 +1267,25 @@ int32_t pshbm_iterate(pshbm_table* t, size_t offset, size_t batch, void* records
     return PSHBM_OK;
 }
 
+int32_t pshbm_iterate_keys(pshbm_table* t, size_t offset, size_t batch, uint64_t* keys, size_t* n_out) {
+    if (!t || !n_out) return PSHBM_INVALID_ID;
+    *n_out = 0;
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    hipStream_t s = t->stream;
+    ST_TRY(begin_op(t, s));
+    ST_TRY(read_counters(t, s));
+    const size_t size = t->h_counters[CNT_ROWS];
+    if (offset >= size || batch == 0) return PSHBM_OK;
+    if (!keys) return fail(t, PSHBM_ERROR, "iterate_keys: null buffer");
+    const size_t cnt = std::min(batch, size - offset);
+    // the keys of the rows lie in one array, in the order of the records
+    HIP_TRY(t, hipMemcpyAsync(keys, t->d.row_keys + offset, cnt * 8, hipMemcpyDeviceToHost, s));
+    HIP_TRY(t, hipStreamSynchronize(s));
+    *n_out = cnt;
+    return PSHBM_OK;
+}
+
 int32_t pshbm_dump(pshbm_table* t, void* records, size_t capacity_records, size_t* n_out) {
     if (!t || !n_out) return PSHBM_INVALID_ID;
     *n_out = 0;

@@ -805,17 +805,12 @@ public:
         req >> shard_id;
         if (new_rt.local_shards().count(shard_id)) {
             pshbm_table* t = st.get(shard_id);
-            const size_t rec = st.record_bytes();
-            std::vector<char> buf(_block_items * rec);
-            std::vector<uint64_t> gone;
+            std::vector<uint64_t> keys(_block_items), gone;
             for (size_t offset = 0;;) {  // the keys first: erasing moves rows, which would disturb the walk
                 size_t got = 0;
-                PSHBM_SCHECK(pshbm_iterate(t, offset, _block_items, buf.data(), &got) == PSHBM_OK, "iterate failed");
-                for (size_t i = 0; i < got; ++i) {
-                    uint64_t key;
-                    std::memcpy(&key, buf.data() + i * rec, 8);
-                    if (_key_partitioner.partition(key, new_rt.global_shard_num()) != shard_id) gone.push_back(key);
-                }
+                PSHBM_SCHECK(pshbm_iterate_keys(t, offset, _block_items, keys.data(), &got) == PSHBM_OK, "iterate failed");
+                for (size_t i = 0; i < got; ++i)
+                    if (_key_partitioner.partition(keys[i], new_rt.global_shard_num()) != shard_id) gone.push_back(keys[i]);
                 offset += got;
                 if (got < _block_items) break;
             }

@@ -802,3 +802,27 @@ def test_page_locked_request_buffers_are_used_in_place(ps, orc, wl, n):
     assert t.set(pk[:m], pv) == 0 and r.set(keys[:m], np.array(pv)) == 0
     assert_same_table(t, r, exact=False)
     t.close()
+
+
+def test_iterate_keys_follows_the_record_order(ps, orc, wl):
+    """The keys-only walk names the records of pshbm_iterate, slice by slice, also after erasures
+    have moved rows; past the end it returns nothing."""
+    rng = np.random.default_rng(41)
+    t, r = pair(ps, orc, 8, "sgd", capacity=20000)
+    keys = wl.fresh_keys_np(rng, 12000)
+    g = rng.normal(0, 1, (12000, 8)).astype(np.float32)
+    assert t.push(keys, g) == 0 and r.push(keys, g) == 0
+    assert t.erase(keys[::3]) == r.erase(keys[::3])
+    n = t.size()
+    seen = []
+    for off in range(0, n + 3000, 2500):
+        st, k = t.iterate_keys(off, 2500)
+        st2, rec = t.iterate(off, 2500)
+        assert st == 0 and st2 == 0
+        np.testing.assert_array_equal(k, rec["key"])
+        assert k.size == max(0, min(2500, n - off))
+        seen.append(k)
+    seen = np.concatenate(seen)
+    assert seen.size == n and np.array_equal(np.sort(seen), np.sort(r.dump()[1]["key"]))
+    assert t.iterate_keys(0, 0)[1].size == 0
+    t.close()
