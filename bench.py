@@ -165,6 +165,29 @@ def scan_table(ps, t, cfg, n_table):
             "note": "wall clock of the synchronous calls, read-back of the result included"}
 
 
+def bulk_transfers(ps, t, cfg):
+    """Dump of the whole table into page-locked host memory and Load of the same records into a
+    second, empty table (a restore: every key is new), timed as the synchronous calls they are. The
+    records cross the link once each way; the rate is record bytes over wall clock."""
+    rows = t.size()
+    rec = ps.pinned_empty(rows, ps.record_dtype(t.value_floats))   # page-locking is not timed
+    t0 = time.perf_counter()
+    st, got = t.dump(out=rec)
+    dt_dump = time.perf_counter() - t0
+    assert st == 0 and got.size == rows
+    t2 = ps.Table(cfg["dim"], capacity=rows + 16, max_batch=1 << 20, **cfg["opt"])
+    t0 = time.perf_counter()
+    st = t2.load(got, ps.LOAD_UNIQUE)
+    dt_load = time.perf_counter() - t0
+    assert st == 0 and t2.size() == rows
+    t2.close()
+    nbytes = rows * rec.dtype.itemsize
+    return {"rows": rows, "record_bytes": rec.dtype.itemsize, "bytes": nbytes,
+            "dump_ms": round(dt_dump * 1e3, 2), "dump_GBps": round(nbytes / dt_dump / 1e9, 1),
+            "load_ms": round(dt_load * 1e3, 2), "load_GBps": round(nbytes / dt_load / 1e9, 1),
+            "note": "host buffer page-locked; PCIe-inclusive by nature, never part of `value`"}
+
+
 def cpu_baseline(cfg, wl, budget_keys):
     """The oracle (a scalar port of the reference's operator loops) on a bounded sample of the same
     workload: a table of budget_keys keys and a few batches of the configured size, one thread."""
@@ -276,6 +299,9 @@ def main():
                     help="after the steps, also time the whole-table operations on the same table: "
                          "for-each (count + column sums), for-each under a predicate on a value "
                          "column, erase-if of about a tenth of the keys; reported under \"scan\"")
+    ap.add_argument("--bulk", action="store_true",
+                    help="after the steps, also time Dump of the table into page-locked host memory "
+                         "and Load of those records into an empty table; reported under \"bulk\"")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -349,6 +375,8 @@ def main():
         "roofline": roofline,
         "phases": phases,
     }
+    if args.bulk:
+        result["bulk"] = bulk_transfers(ps, t, cfg)
     if args.scan:
         result["scan"] = scan_table(ps, t, cfg, n_table)
     t.close()
