@@ -5,6 +5,7 @@
 //
 //   HbmShardStorage        <- KVShardStorage / PoolHashMapShardStorage (storage/KVShardStorage.h:22-49, 844-952)
 //   HbmStorageOperator     <- ShardStorageOperator                     (operator/StorageOperator.h:78-158)
+//   HbmSyncOperator        <- KVSyncOperator                           (operator/SyncOperator.h:102-266)
 //   HbmSparsePullOperator  <- SparseTablePullOperator::apply_request   (operator/SparsePullOperator.h:156-254)
 //   HbmSparsePushOperator  <- SparseTablePushOperator server halves    (operator/SparsePushOperator.h:197-416)
 //   HbmDirectPushOperator  <- DirectPushOperator                       (operator/SparsePushOperator.h:520-574)
@@ -825,6 +826,120 @@ public:
 
 private:
     size_t _block_items;
+    PARTITIONER _key_partitioner;
+};
+
+// Sync to another cluster (KVSyncOperator, operator/SyncOperator.h:102-266): the values that pushes
+// wrote since the last sync travel to the storage of, say, an online-serving cluster. The sending
+// side walks the increment -- here the marks inside each shard's table, taken once per walk
+// (IncrementStorage::read_storage, service/IncrementStorage.h:29-36) -- and cuts it into requests
+// of up to block_size items, partitioned for the receiving cluster's shards; the receiving side
+// upserts them (ht[key] = value, :159-163). to_sync_value (:186) is the identity: the whole value
+// travels. PARTITIONER::partition(key, global_shard_num) as in HbmShuffleOperator.
+template <class PARTITIONER>
+class HbmSyncOperator {
+public:
+    explicit HbmSyncOperator(const Configure& config) : _block_size((size_t)config.number("block_size", 1000)) {}  // :24
+
+    // TemplateStorageIterator over the increment (:45-98): the records {key, value} every local
+    // shard's pushes touched, in the order the shards and their slabs give.
+    class IncrIterator {
+    public:
+        IncrIterator(HbmShardStorage& st) : _rec(st.record_bytes()) {
+            for (int32_t shard_id : st.shard_list()) {
+                uint64_t marked = 0;
+                PSHBM_SCHECK(pshbm_increment_size(st.get(shard_id), &marked) == PSHBM_OK, "increment_size failed");
+                if (marked == 0) continue;
+                const size_t at = _records.size();
+                _records.resize(at + marked * _rec);
+                size_t got = 0;
+                PSHBM_SCHECK(pshbm_take_increment(st.get(shard_id), _records.data() + at, marked, &got) == PSHBM_OK,
+                             "take_increment failed");
+                _records.resize(at + got * _rec);
+            }
+        }
+        const char* next() {  // nullptr at the end
+            if (_pos >= _records.size()) return nullptr;
+            const char* p = _records.data() + _pos;
+            _pos += _rec;
+            return p;
+        }
+        size_t record_bytes() const { return _rec; }
+
+    private:
+        std::vector<char> _records;
+        size_t _rec, _pos = 0;
+    };
+
+    std::unique_ptr<IncrIterator> incr_iterator(Storage* storage) {  // :188-190
+        return std::make_unique<IncrIterator>(*static_cast<HbmShardStorage*>(storage));
+    }
+
+    // generate_sync_request, :192-214 + generate_request, :217-258: one request per node of the
+    // receiving cluster `rt`: i32 node_items, i32 n_shards, then per shard i32 shard_id,
+    // i32 shard_items and the items as {key, value} records. Status::Empty when nothing is left.
+    Status generate_sync_request(IncrIterator* it, RuntimeInfo& rt, std::vector<PSRequest>& reqs) {
+        std::vector<std::vector<char>> tables(rt.global_shard_num());
+        const size_t rec = it->record_bytes();
+        size_t cnt = 0;
+        for (; cnt < _block_size; ++cnt) {
+            const char* item = it->next();
+            if (item == nullptr) break;
+            uint64_t key;
+            std::memcpy(&key, item, 8);
+            std::vector<char>& tb = tables[_key_partitioner.partition(key, rt.global_shard_num())];
+            tb.insert(tb.end(), item, item + rec);
+        }
+        if (cnt == 0) return Status::Empty("");
+        for (auto& node : rt.nodes()) {
+            if (node.second.empty()) return Status::NoReplica("");
+            int32_t node_items = 0;
+            for (int32_t shard_id : node.second) node_items += (int32_t)(tables[shard_id].size() / rec);
+            reqs.emplace_back();
+            BinaryArchive& ar = reqs.back().archive();
+            ar << node_items << (int32_t)node.second.size();
+            for (int32_t shard_id : node.second) {
+                ar << shard_id << (int32_t)(tables[shard_id].size() / rec);
+                ar.write_raw(tables[shard_id].data(), tables[shard_id].size());
+            }
+        }
+        return Status();
+    }
+
+    // apply_sync_request, :126-184. The items of a shard lie in the archive as the records
+    // pshbm_load takes; a shard that cannot hold them grows like one that a push fills, and past
+    // its limit the response carries Status::OOM (:164-168).
+    void apply_sync_request(RuntimeInfo& rt, PSRequest& req, Storage* storage, PSResponse& resp_ret) {
+        BinaryArchive& ar = req.archive();
+        auto& st = *static_cast<HbmShardStorage*>(storage);
+        const size_t rec = st.record_bytes();
+        int32_t node_items, n_shards;
+        ar >> node_items >> n_shards;
+        Status status;
+        while (n_shards--) {
+            int32_t shard_id, shard_items;
+            ar >> shard_id;
+            PSHBM_SCHECK(rt.local_shards().count(shard_id) != 0, "Bad Request: invalid shard_id");
+            ar >> shard_items;
+            node_items -= shard_items;
+            PSHBM_SCHECK(ar.readable() >= (size_t)shard_items * rec, "sync block size mismatch");
+            if (status.ok() && shard_items > 0) {
+                pshbm_table* t = st.get(shard_id);
+                int32_t rc = pshbm_load(t, ar.cursor(), (size_t)shard_items, 0);
+                while (rc == PSHBM_OUT_OF_MEMORY && st.grow(shard_id)) rc = pshbm_load(t, ar.cursor(), (size_t)shard_items, 0);
+                if (rc == PSHBM_OUT_OF_MEMORY) status = Status::OOM("PServer OOM during sync op");
+                else if (rc != PSHBM_OK) status = Status::Error(pshbm_last_error(t));
+            }
+            ar.advance((size_t)shard_items * rec);
+        }
+        PSHBM_SCHECK(node_items == 0, "sync request: item counts do not add up");  // :178
+        PSHBM_SCHECK(ar.is_exhausted(), "request not exhausted");                  // :179
+        resp_ret = PSResponse(req);
+        resp_ret << status;
+    }
+
+private:
+    size_t _block_size;
     PARTITIONER _key_partitioner;
 };
 

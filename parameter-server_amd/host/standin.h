@@ -89,7 +89,8 @@ private:
 };
 
 // pico-ps/common/Status.h
-enum class StatusCode : int32_t { OK = 0, INVALID_CONFIG = 1, INVALID_ID = 2, OUT_OF_MEMORY = 3, ERROR = 10, FATAL = 11 };
+enum class StatusCode : int32_t { OK = 0, INVALID_CONFIG = 1, INVALID_ID = 2, OUT_OF_MEMORY = 3, NO_REPLICA = 9,
+                                  ERROR = 10, FATAL = 11, EMPTY = 12 };
 class Status {
 public:
     Status() = default;
@@ -98,6 +99,9 @@ public:
     static Status Fatal(const std::string& m) { return Status(StatusCode::FATAL, m); }
     static Status InvalidConfig(const std::string& m) { return Status(StatusCode::INVALID_CONFIG, m); }
     static Status InvalidID(const std::string& m) { return Status(StatusCode::INVALID_ID, m); }
+    static Status NoReplica(const std::string& m) { return Status(StatusCode::NO_REPLICA, m); }
+    static Status Empty(const std::string& m) { return Status(StatusCode::EMPTY, m); }
+    bool IsEmpty() const { return _code == StatusCode::EMPTY; }
     bool ok() const { return _code == StatusCode::OK; }
     bool IsOOM() const { return _code == StatusCode::OUT_OF_MEMORY; }
     StatusCode code() const { return _code; }
@@ -164,6 +168,10 @@ public:
     const std::set<int32_t>& local_shards() const { return _shards; }
     int32_t node_id() const { return _node; }
     int32_t global_shard_num() const { return (int32_t)_shards.size(); }
+    // node -> the shards it holds (TableDescriptor.h:180-228); the stand-in knows one node
+    std::map<int32_t, std::vector<int32_t>> nodes() const {
+        return {{_node, std::vector<int32_t>(_shards.begin(), _shards.end())}};
+    }
 
 private:
     int32_t _node;

@@ -422,6 +422,83 @@ static void test_memory_limit() {
     EXPECT(pshbm_device_memory(0, &after, nullptr) == PSHBM_OK && after < in_use);
 }
 
+// Sync to another cluster (operator/SyncOperator.h:102-266): what pushes wrote on the training side
+// since the last sync arrives in the serving side's storage, block by block; a second walk finds
+// nothing; later pushes travel with the next one.
+static void test_sync() {
+    struct ModPartitioner {
+        int32_t partition(uint64_t key, int32_t global_shard_num) { return (int32_t)(key % (uint64_t)global_shard_num); }
+    };
+    Configure train_config;
+    train_config.set("dim", 2);
+    train_config.set("optimizer", "sum");
+    train_config.set("hbm_table.expected_max_items", 1000);
+    train_config.set("hbm_table.track_increment", 1);
+    train_config.set("block_size", 64);
+    Configure serve_config = train_config;
+    serve_config.set("hbm_table.track_increment", 0);
+    serve_config.set("hbm_table.expected_max_items", 100);   // grows as the synced items arrive
+    serve_config.set("hbm_table.grow_limit", 4000);
+    RuntimeInfo rt(0, {0, 1});
+    HbmStorageOperator train_storage_op(train_config), serve_storage_op(serve_config);
+    std::unique_ptr<Storage> train = train_storage_op.create_storage(rt, 0);
+    std::unique_ptr<Storage> serve = serve_storage_op.create_storage(rt, 1);
+    HbmSparsePushOperator push_op(train_config);
+    HbmSparsePullOperator train_pull(train_config), serve_pull(serve_config);
+    HbmSyncOperator<ModPartitioner> sync_op(train_config);
+
+    auto push = [&](const std::vector<uint64_t>& keys, float arg) {
+        PSRequest req = make_push_request(keys, std::vector<float>(keys.size(), arg));
+        PSResponse resp;
+        Status status;
+        push_op.apply_async_push_request(rt, req, train.get(), nullptr, resp);
+        resp >> status;
+        EXPECT(status.ok());
+    };
+    auto sync = [&]() {   // returns the number of requests that carried items
+        auto it = sync_op.incr_iterator(train.get());
+        int sent = 0;
+        while (true) {
+            std::vector<PSRequest> reqs;
+            Status st = sync_op.generate_sync_request(it.get(), rt, reqs);
+            if (st.IsEmpty()) break;
+            EXPECT(st.ok() && reqs.size() == 1);
+            for (PSRequest& req : reqs) {
+                PSResponse resp;
+                Status status;
+                sync_op.apply_sync_request(rt, req, serve.get(), resp);
+                resp >> status;
+                EXPECT(status.ok());
+                ++sent;
+            }
+        }
+        return sent;
+    };
+    std::vector<uint64_t> keys;
+    for (uint64_t k = 0; k < 300; ++k) keys.push_back(k * 7 + 1);
+    push(keys, 3.0f);   // [3, 1] per key
+    EXPECT(sync() == 5);  // 300 items in blocks of 64
+    bool ok;
+    auto a = pull(train_pull, rt, train.get(), keys, &ok);
+    EXPECT(ok);
+    auto b = pull(serve_pull, rt, serve.get(), keys, &ok);
+    EXPECT(ok);
+    EXPECT(a == b);
+    for (size_t i = 0; i < keys.size(); ++i) EXPECT(b[i * 2] == 3.0f && b[i * 2 + 1] == 1.0f);
+    EXPECT(static_cast<HbmShardStorage*>(serve.get())->shard_size(0) + static_cast<HbmShardStorage*>(serve.get())->shard_size(1) == 300);
+    EXPECT(sync() == 0);  // nothing was pushed since
+    std::vector<uint64_t> some(keys.begin(), keys.begin() + 10), fresh{5000, 5001};
+    push(some, 1.0f);
+    push(fresh, 2.0f);
+    EXPECT(sync() == 1);
+    std::vector<uint64_t> all = keys;
+    all.insert(all.end(), fresh.begin(), fresh.end());
+    a = pull(train_pull, rt, train.get(), all, &ok);
+    b = pull(serve_pull, rt, serve.get(), all, &ok);
+    EXPECT(a == b);
+    EXPECT(b[0] == 4.0f && b[1] == 2.0f && b[10 * 2] == 3.0f && b[300 * 2] == 2.0f && b[300 * 2 + 1] == 1.0f);
+}
+
 // The learning rate belongs to the push operator (pico-ps/operator/Operator.h:53-57): two operators
 // registered with different rates push to one storage, each with its own.
 static void test_operator_hyperparameters() {
@@ -825,6 +902,7 @@ int main(int argc, char** argv) {
     test_operator_hyperparameters();
     test_initial_weights();
     test_memory_limit();
+    test_sync();
     if (g_failed) {
         std::printf("FAILED: %d expectation(s)\n", g_failed);
         return 1;
