@@ -52,6 +52,10 @@ MEASURED_TRAFFIC_BYTES = {
     ("c2", "pull"): 191_800_000, ("c2", "locate"): 75_700_000, ("c2", "assign_rows"): 100_000,
     ("c2", "sort_hist"): 6_400_000, ("c2", "sort_pass"): 26_200_000, ("c2", "segreduce"): 194_800_000,
     ("c2", "fixup_windows"): 300_000, ("c2", "fixup"): 1_900_000,
+    ("c1", "pull"): 19_200_000,
+    ("c3", "pull"): 694_600_000, ("c3", "locate"): 79_900_000, ("c3", "segreduce"): 739_400_000,
+    ("c4", "pull"): 562_800_000, ("c4", "locate"): 273_200_000, ("c4", "segreduce"): 789_000_000,
+    ("c5", "pull"): 3_185_700_000, ("c5", "segreduce"): 3_744_100_000,
 }
 
 
