@@ -375,6 +375,15 @@ int32_t pshbm_set_memory_limit(int32_t device, uint64_t bytes);
  * may be NULL. The per-table figure is pshbm_memory_usage. */
 int32_t pshbm_device_memory(int32_t device, uint64_t* in_use, uint64_t* limit);
 
+/* Test hook, no counterpart in the reference: how many times a tile of the aggregation sort polls
+ * for a predecessor's counts before it gives up (0xFFFFFFFF = the default, 2^24). A tile that gives
+ * up raises a flag, the kernels after the sort then apply nothing, and the table answers
+ * PSHBM_FATAL from its next call that reads its counters (size, dump, for_each, ...) until
+ * pshbm_clear: the push is not applied, keys it inserted keep their initial values. 0 makes every
+ * waiting tile give up at once, which is how the tests reach that path while every kernel still
+ * runs to its end. Process-wide. */
+int32_t pshbm_debug_sort_spin_limit(uint32_t polls);
+
 /* Pinned (page-locked) host memory for request/response buffers of the host-pointer entry points.
  * Buffers from here (or from hipHostMalloc) spare the staging copies: pshbm_pull and pshbm_push
  * hand batches of up to 1 MB to the kernels as they lie, pshbm_load and pshbm_dump let the copy

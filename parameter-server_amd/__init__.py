@@ -34,6 +34,7 @@ SYMBOLS = [
     "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve", "pshbm_set_hyperparameters", "pshbm_set_memory_limit", "pshbm_device_memory",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
+    "pshbm_debug_sort_spin_limit",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
           "fixup_windows", "assign_rows", "push_small"]
@@ -182,6 +183,7 @@ def lib():
         L.pshbm_pull_dev.argtypes = [vp, vp, sz, vp, vp, u32, vp]
         L.pshbm_push.argtypes = [vp, vp, vp, sz, u32]
         L.pshbm_push_dev.argtypes = [vp, vp, vp, sz, u32, vp]
+        L.pshbm_debug_sort_spin_limit.argtypes = [u32]
         L.pshbm_push_pairs.argtypes = [vp, vp, sz, sz, u32]
         L.pshbm_queue.argtypes = [vp, vp, vp, sz]
         L.pshbm_queue_dev.argtypes = [vp, vp, vp, sz, vp]
@@ -240,6 +242,11 @@ def device_memory(device=0):
     if st != OK:
         raise PshbmError(st, "device_memory: bad device")
     return a.value, b.value
+
+
+def debug_sort_spin_limit(polls=0xFFFFFFFF):
+    """Test hook: polls a sort tile grants its predecessors (default 2^24; 0 = give up at once)."""
+    return lib().pshbm_debug_sort_spin_limit(polls)
 
 
 def init_weight(init_range, key, column):

@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <deque>
 #include <mutex>
 #include <new>
 #include <shared_mutex>
@@ -31,6 +32,22 @@ inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 struct DevBuf {
     void* p = nullptr;
     size_t bytes = 0;
+};
+
+// Scratch of one push: where the probe leaves slots, rows and batch indices, the sort's buffers, the
+// partial sums of the segmented reduction. The table's own workspace grows with the batch; the
+// entry point that must not allocate brings a fixed one.
+struct Workspace {
+    uint32_t *slot, *idx, *row, *srow, *sidx;
+    void* sort;
+    size_t sort_bytes;
+    unsigned sort_parity;  // which half of the sort head is zero and will be used
+    uint4* hdr;
+    float* pval;
+    uint32_t* wrow;
+    float* wval;
+    uint32_t *won_cur, *won_next;  // per-block winner counts: counted into / zeroed for the next operation
+    size_t won_words;
 };
 
 // Is [p, p + bytes) page-locked host memory that the runtime knows (hipHostMalloc,
@@ -196,7 +213,15 @@ struct pshbm_table {
     std::vector<hipStream_t> reader_streams;
 
     std::shared_mutex mu;
-    uint64_t size_bound = 0;  // upper bound of the rows handed out
+    // Upper bound of the rows handed out, kept without device round trips: the kernels that hand
+    // out rows leave {operation number, row count} in the page-locked word h_pub; the bound is the
+    // last count seen there (or read back) plus the sizes of the inserting batches enqueued since.
+    unsigned long long* h_pub = nullptr;
+    uint32_t op_seq = 0;    // number of the last inserting operation enqueued
+    uint32_t base_seq = 0;  // rows_base is the row count after this operation
+    uint64_t rows_base = 0;
+    uint64_t pending_sum = 0;
+    std::deque<std::pair<uint32_t, uint32_t>> pending;  // {operation number, keys} enqueued after base_seq
 
     // optional per-kernel timing (pshbm_profile_*)
     bool prof_on = false;
@@ -357,28 +382,58 @@ int32_t read_counters(pshbm_table* t, hipStream_t s) {
     HIP_TRY(t, hipMemcpyAsync(t->h_counters, t->d.counters, CNT_WORDS * 4, hipMemcpyDeviceToHost, s));
     HIP_TRY(t, hipStreamSynchronize(s));
     if (t->h_counters[CNT_SORT_ERR])
-        return fail(t, PSHBM_FATAL, "a radix-sort tile timed out waiting for its predecessor; "
-                                    "the last push may be wrong");
+        return fail(t, PSHBM_FATAL, "a radix-sort tile timed out waiting for its predecessor: the push it "
+                                    "belonged to, and every push since, was not applied (keys they inserted "
+                                    "keep their initial values); pshbm_clear resets the table");
     return PSHBM_OK;
 }
 
-// Capacity accounting without a device round trip in the common case: `size_bound` is an upper
-// bound of the rows handed out (every inserting batch of n keys adds at most n). Only when the
-// bound would pass the capacity is the exact count read back; if even that leaves less than n
-// free rows the batch runs in checked mode (`*checked`), where the caller inspects the overflow
-// flag after the claim and rolls the batch back when it is set.
+// The table holds exactly `rows` rows and nothing that inserts is in flight.
+void set_exact_rows(pshbm_table* t, uint64_t rows) {
+    t->rows_base = rows;
+    t->base_seq = t->op_seq;
+    t->pending.clear();
+    t->pending_sum = 0;
+}
+
+// Upper bound of the rows handed out, from what the device has published so far.
+uint64_t rows_upper_bound(pshbm_table* t) {
+    const unsigned long long pub = *static_cast<volatile unsigned long long*>(t->h_pub);
+    const uint32_t pseq = (uint32_t)(pub >> 32);
+    if ((int32_t)(pseq - t->base_seq) > 0 && (int32_t)(t->op_seq - pseq) >= 0) {
+        while (!t->pending.empty() && (int32_t)(t->pending.front().first - pseq) <= 0) {
+            t->pending_sum -= t->pending.front().second;
+            t->pending.pop_front();
+        }
+        t->rows_base = (uint32_t)pub;
+        t->base_seq = pseq;
+    }
+    return t->rows_base + t->pending_sum;
+}
+
+// Books an inserting batch of n keys: the launches that follow carry its number.
+void book_insert(pshbm_table* t, size_t n) {
+    ++t->op_seq;
+    t->d.op_seq = t->op_seq;
+    t->pending.emplace_back(t->op_seq, (uint32_t)n);
+    t->pending_sum += n;
+}
+
+// Capacity accounting without a device round trip in the common case: the bound above is exact up
+// to the batches still in flight. Only when it would pass the capacity is the exact count read back
+// (one stream synchronisation); if even that leaves fewer than n free rows the batch runs in
+// checked mode (`*checked`), where the caller inspects the overflow flag after the claim and rolls
+// the batch back when it is set.
 int32_t reserve_rows(pshbm_table* t, size_t n, hipStream_t s, bool* checked, uint32_t* rows_before) {
     *checked = false;
-    if (t->size_bound + n <= t->d.max_rows) {
-        t->size_bound += n;
+    if (rows_upper_bound(t) + n <= t->d.max_rows) {
+        book_insert(t, n);
         return PSHBM_OK;
     }
     ST_TRY(read_counters(t, s));
-    t->size_bound = t->h_counters[CNT_ROWS];
-    if (t->size_bound + n <= t->d.max_rows) {
-        t->size_bound += n;
-        return PSHBM_OK;
-    }
+    set_exact_rows(t, t->h_counters[CNT_ROWS]);
+    book_insert(t, n);
+    if (t->rows_base + n <= t->d.max_rows) return PSHBM_OK;
     *checked = true;
     *rows_before = t->h_counters[CNT_ROWS];
     return PSHBM_OK;
@@ -391,12 +446,12 @@ int32_t settle_rows(pshbm_table* t, const uint32_t* slot_idx, size_t n, hipStrea
     if (t->h_counters[CNT_OVERFLOW] || t->h_counters[CNT_ROWS] > t->d.max_rows) {
         HIP_TRY(t, launch_rollback(t->d, slot_idx, n, rows_before, s));
         HIP_TRY(t, hipStreamSynchronize(s));
-        t->size_bound = rows_before;
+        set_exact_rows(t, rows_before);
         return fail(t, PSHBM_OUT_OF_MEMORY,
                     "table full: %u keys stored, capacity %u, batch of %zu does not fit",
                     rows_before, t->d.max_rows, n);
     }
-    t->size_bound = t->h_counters[CNT_ROWS];
+    set_exact_rows(t, t->h_counters[CNT_ROWS]);
     return PSHBM_OK;
 }
 
@@ -407,30 +462,52 @@ bool has_reserved_key(const uint64_t* keys, size_t n) {
 }
 
 // The probe of a mutating operation: slots of the keys, claiming one for each missing key when
-// `insert`, followed by the launch that gives the claimed slots their rows. The two arrays of
-// per-block winner counts alternate: each operation counts into one and zeroes the other.
+// `insert`, followed by the launch that gives the claimed slots their rows. won_cur / won_next are
+// the two arrays of per-block winner counts: the operation counts into one and zeroes the other.
 int32_t locate_and_assign(pshbm_table* t, const uint64_t* d_keys, size_t n, uint32_t* slot, uint32_t* idx,
-                          uint32_t* row, bool insert, bool init_rows, bool count_dups, hipStream_t s) {
+                          uint32_t* row, bool insert, bool init_rows, bool count_dups, uint32_t* won_cur,
+                          uint32_t* won_next, size_t won_words, hipStream_t s) {
     if (!insert) {
         HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE,
                      launch_locate(t->d, d_keys, n, slot, idx, row, nullptr, count_dups, s));
         return PSHBM_OK;
     }
-    const size_t half = t->ws_won.bytes / 8;  // words per array
-    uint32_t* cur = static_cast<uint32_t*>(t->ws_won.p) + (t->won_parity & 1u) * half;
-    uint32_t* next = static_cast<uint32_t*>(t->ws_won.p) + ((t->won_parity & 1u) ^ 1u) * half;
-    ++t->won_parity;
-    HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE, launch_locate(t->d, d_keys, n, slot, idx, row, cur, count_dups, s));
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_LOCATE, launch_locate(t->d, d_keys, n, slot, idx, row, won_cur, count_dups, s));
     HIP_TRY_PROF(t, s, PSHBM_PHASE_ASSIGN_ROWS,
-                 launch_assign_rows(t->d, d_keys, n, slot, row, cur, next, half, init_rows, s));
+                 launch_assign_rows(t->d, d_keys, n, slot, row, won_cur, won_next, won_words, init_rows, s));
     return PSHBM_OK;
 }
 
-int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
-                    uint32_t flags, hipStream_t s) {
-    if (n == 0) return PSHBM_OK;
-    ST_TRY(begin_op(t, s));
-    ST_TRY(ensure_workspace(t, n));
+// The table's own workspace for the operation that is about to be enqueued (ensure_workspace has
+// sized it). The caller flips the halves that alternate between operations once it has used them:
+// won_parity after a locate_and_assign that inserts, sort_parity after a sort that used the head.
+Workspace table_workspace(pshbm_table* t) {
+    Workspace w{};
+    w.slot = static_cast<uint32_t*>(t->ws_slot.p);
+    w.idx = static_cast<uint32_t*>(t->ws_idx.p);
+    w.row = static_cast<uint32_t*>(t->ws_row.p);
+    w.srow = static_cast<uint32_t*>(t->ws_srow.p);
+    w.sidx = static_cast<uint32_t*>(t->ws_sidx.p);
+    w.sort = t->ws_sort.p;
+    w.sort_bytes = t->ws_sort.bytes;
+    w.sort_parity = t->sort_parity;
+    w.hdr = static_cast<uint4*>(t->ws_hdr.p);
+    w.pval = static_cast<float*>(t->ws_pval.p);
+    w.wrow = static_cast<uint32_t*>(t->ws_wrow.p);
+    w.wval = static_cast<float*>(t->ws_wval.p);
+    const size_t half = t->ws_won.bytes / 8;  // words per array
+    w.won_cur = static_cast<uint32_t*>(t->ws_won.p) + (t->won_parity & 1u) * half;
+    w.won_next = static_cast<uint32_t*>(t->ws_won.p) + ((t->won_parity & 1u) ^ 1u) * half;
+    w.won_words = half;
+    return w;
+}
+
+// One push on stream s with the scratch of `w`. *used_sort_head: the sort took the half of the sort
+// head that w.sort_parity names (and zeroed the other one).
+int32_t push_with(pshbm_table* t, const Workspace& w, const uint64_t* d_keys, const float* d_grads, size_t n,
+                  uint32_t flags, hipStream_t s, bool* used_sort_head, bool* used_won) {
+    *used_sort_head = false;
+    *used_won = false;
     const bool insert = !(flags & PSHBM_PUSH_NO_INSERT);
     const bool unique = (flags & PSHBM_PUSH_ASSUME_UNIQUE) != 0;
     bool checked = false;
@@ -442,47 +519,52 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
         HIP_TRY_PROF(t, s, PSHBM_PHASE_PUSH_SMALL, launch_push_small(t->d, d_keys, d_grads, n, insert, s));
         return PSHBM_OK;
     }
-    uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
-    uint32_t* idx = static_cast<uint32_t*>(t->ws_idx.p);
     // Everything after the probe works on row ids: they are dense, so the sort needs fewer bits
     // than for slot indices, the update needs no second look at the hash array, and sorted
     // positions walk the row slab in ascending address order.
-    uint32_t* row = static_cast<uint32_t*>(t->ws_row.p);
-    ST_TRY(locate_and_assign(t, d_keys, n, slot, unique ? nullptr : idx, row, insert, true, false, s));
-    if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
+    *used_won = insert;  // counted into one array of winner counts, zeroed the other
+    ST_TRY(locate_and_assign(t, d_keys, n, w.slot, unique ? nullptr : w.idx, w.row, insert, true, false,
+                             w.won_cur, w.won_next, w.won_words, s));
+    if (checked) ST_TRY(settle_rows(t, w.slot, n, s, rows_before));
     if (unique) {
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_UPDATE_UNIQUE, launch_update_unique(t->d, row, n, d_grads, s));
-    } else {
-        uint32_t* srow = static_cast<uint32_t*>(t->ws_srow.p);
-        uint32_t* sidx = static_cast<uint32_t*>(t->ws_sidx.p);
-        SortPlan plan;
-        // a key inserted by this batch more than once: only the claiming occurrence got the row
-        const SortLateKeys late{ROW_PENDING, slot, t->d.slots};
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_HIST,
-                     sort_begin(t->ws_sort.p, t->ws_sort.bytes, t->sort_parity, row, n, t->row_bits,
-                                &plan, s, insert ? &late : nullptr));
-        if (plan.uses_head) ++t->sort_parity;  // each such sort zeroes the other half for the next
-        uint32_t *kin = row, *vin = idx, *kout = srow, *vout = sidx;
-        for (uint32_t p = 0; p < plan.passes; ++p) {
-            HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_PASS,
-                         sort_pass(plan, p, kin, vin, kout, vout, t->d.counters + CNT_SORT_ERR, s));
-            std::swap(kin, kout);
-            std::swap(vin, vout);
-        }
-        const bool in_b = (plan.passes & 1u) != 0;
-        const uint32_t* fs = in_b ? srow : row;
-        const uint32_t* fi = in_b ? sidx : idx;
-        uint4* hdr = static_cast<uint4*>(t->ws_hdr.p);
-        float* pval = static_cast<float*>(t->ws_pval.p);
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_SEGREDUCE,
-                     launch_segreduce(t->d, fs, fi, n, d_grads, hdr, pval, s));
-        uint32_t* wrow = static_cast<uint32_t*>(t->ws_wrow.p);
-        float* wval = static_cast<float*>(t->ws_wval.p);
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP_WINDOWS,
-                     launch_fixup_windows(t->d, n, d_grads, hdr, pval, wrow, wval, s));
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP, launch_fixup(t->d, n, d_grads, hdr, pval, wrow, wval, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_UPDATE_UNIQUE, launch_update_unique(t->d, w.row, n, d_grads, s));
+        return PSHBM_OK;
     }
+    SortPlan plan;
+    // a key inserted by this batch more than once: only the claiming occurrence got the row
+    const SortLateKeys late{ROW_PENDING, w.slot, t->d.slots};
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_HIST,
+                 sort_begin(w.sort, w.sort_bytes, w.sort_parity, w.row, n, t->row_bits, &plan, s,
+                            insert ? &late : nullptr));
+    *used_sort_head = plan.uses_head;  // each such sort zeroes the other half for the next
+    uint32_t *kin = w.row, *vin = w.idx, *kout = w.srow, *vout = w.sidx;
+    for (uint32_t p = 0; p < plan.passes; ++p) {
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_SORT_PASS,
+                     sort_pass(plan, p, kin, vin, kout, vout, t->d.counters + CNT_SORT_ERR, s));
+        std::swap(kin, kout);
+        std::swap(vin, vout);
+    }
+    const bool in_b = (plan.passes & 1u) != 0;
+    const uint32_t* fs = in_b ? w.srow : w.row;
+    const uint32_t* fi = in_b ? w.sidx : w.idx;
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_SEGREDUCE, launch_segreduce(t->d, fs, fi, n, d_grads, w.hdr, w.pval, s));
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP_WINDOWS,
+                 launch_fixup_windows(t->d, n, d_grads, w.hdr, w.pval, w.wrow, w.wval, s));
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_FIXUP, launch_fixup(t->d, n, d_grads, w.hdr, w.pval, w.wrow, w.wval, s));
     return PSHBM_OK;
+}
+
+int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
+                    uint32_t flags, hipStream_t s) {
+    if (n == 0) return PSHBM_OK;
+    ST_TRY(begin_op(t, s));
+    ST_TRY(ensure_workspace(t, n));
+    const Workspace w = table_workspace(t);
+    bool used_head = false, used_won = false;
+    const int32_t st = push_with(t, w, d_keys, d_grads, n, flags, s, &used_head, &used_won);
+    if (used_head) ++t->sort_parity;
+    if (used_won) ++t->won_parity;
+    return st;
 }
 
 int32_t set_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_values, size_t n,
@@ -493,8 +575,11 @@ int32_t set_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_values
     bool checked = false;
     uint32_t rows_before = 0;
     ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
-    uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
-    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, nullptr, true, false, count_dups, s));
+    const Workspace w = table_workspace(t);
+    ++t->won_parity;
+    uint32_t* slot = w.slot;
+    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, nullptr, true, false, count_dups, w.won_cur,
+                             w.won_next, w.won_words, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
     HIP_TRY(t, launch_write_values(t->d, slot, n, d_values, s));
     return PSHBM_OK;
@@ -539,6 +624,7 @@ void destroy_impl(pshbm_table* t) {
     if (t->d_hist) (void)dev_free(t->device, t->d_hist);
     if (t->h_counters) (void)hipHostFree(t->h_counters);
     if (t->h_hist) (void)hipHostFree(t->h_hist);
+    if (t->h_pub) (void)hipHostFree(t->h_pub);
     if (t->d_info) (void)dev_free(t->device, t->d_info);
     if (t->h_info) (void)hipHostFree(t->h_info);
     if (t->h_fe) (void)hipHostFree(t->h_fe);
@@ -607,7 +693,7 @@ int32_t erase_flagged(pshbm_table* t, uint32_t rows, hipStream_t s, uint64_t* er
     HIP_TRY(t, hipStreamSynchronize(s));
     const uint32_t gone = t->h_info[0];
     if (erased) *erased = gone;
-    t->size_bound = rows - gone;
+    set_exact_rows(t, rows - gone);
     if (gone == 0) return PSHBM_OK;
     ST_TRY(ensure(t, t->ms_lists, 3 * (size_t)gone * 4));
     HIP_TRY(t, launch_erase_apply(t->d, rows, gone, dead, tiles, t->d_info,
@@ -721,6 +807,9 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     CREATE_TRY(dev_malloc(t->device, reinterpret_cast<void**>(&t->d_hist), 17 * 8));
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_counters), CNT_WORDS * 4, hipHostMallocDefault));
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_hist), 17 * 8, hipHostMallocDefault));
+    CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_pub), 8, hipHostMallocDefault));
+    *t->h_pub = 0;
+    d.pub = t->h_pub;
     CREATE_TRY(hipStreamCreateWithFlags(&t->stream, hipStreamNonBlocking));
     CREATE_TRY(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));
     for (pshbm_table::PullLane& l : t->lanes) {
@@ -767,8 +856,11 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     bool checked = false;
     uint32_t rows_before = 0;
     ST_TRY(reserve_rows(t, n, s, &checked, &rows_before));
-    uint32_t* slot = static_cast<uint32_t*>(t->ws_slot.p);
-    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, nullptr, true, true, false, s));
+    const Workspace w = table_workspace(t);
+    ++t->won_parity;
+    uint32_t* slot = w.slot;
+    ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, nullptr, true, true, false, w.won_cur, w.won_next,
+                             w.won_words, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
     HIP_TRY_PROF(t, s, PSHBM_PHASE_GATHER, launch_gather_slots(t->d, d_keys, slot, n, d_out_rows, d_hit, s));
     return PSHBM_OK;
@@ -1589,7 +1681,7 @@ int32_t pshbm_clear(pshbm_table* t) {
     HIP_TRY(t, hipMemsetAsync(t->d.counters, 0, CNT_WORDS * 4, s));
     if (t->d.dirty) HIP_TRY(t, hipMemsetAsync(t->d.dirty, 0, round_up(t->d.max_rows, 4), s));
     HIP_TRY(t, hipStreamSynchronize(s));
-    t->size_bound = 0;
+    set_exact_rows(t, 0);
     t->tombstones = 0;
     return PSHBM_OK;
 }
@@ -1600,7 +1692,7 @@ int32_t pshbm_size(pshbm_table* t, uint64_t* n) {
     std::unique_lock<std::shared_mutex> lk(t->mu);
     ST_TRY(begin_op(t, t->stream));
     ST_TRY(read_counters(t, t->stream));
-    t->size_bound = t->h_counters[CNT_ROWS];
+    set_exact_rows(t, t->h_counters[CNT_ROWS]);
     *n = t->h_counters[CNT_ROWS];
     return PSHBM_OK;
 }
@@ -1671,6 +1763,11 @@ int32_t pshbm_profile_read(pshbm_table* t, pshbm_profile* out) {
         out->launches[ph] += 1;
     }
     t->prof_phase.clear();
+    return PSHBM_OK;
+}
+
+int32_t pshbm_debug_sort_spin_limit(uint32_t polls) {
+    sort_set_spin_limit(polls);
     return PSHBM_OK;
 }
 

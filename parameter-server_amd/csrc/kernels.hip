@@ -30,6 +30,15 @@ __device__ __forceinline__ u64 div_big(u64 n, u64 m, u32 d) { return d == 1 ? n 
 inline u64 magic32(u32 d) { return ((1ull << 32) + d - 1) / d; }
 inline u64 magic64(u32 d) { return d <= 1 ? 0 : (~0ull / d) + 1; }
 
+// The row count an inserting operation leaves, told to the host without a round trip: one 64-bit
+// word in page-locked memory, {operation number, rows}. The host adds the sizes of the operations
+// it has enqueued since to get an upper bound of the row count.
+__device__ __forceinline__ void publish_rows(const TableDev& t, u32 rows) {
+    if (t.pub)
+        __hip_atomic_store(t.pub, ((unsigned long long)t.op_seq << 32) | rows, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // float f of the value a key starts with: weights, then optimizer state
 __device__ __forceinline__ float init_float(const TableDev& t, u64 key, u32 f) {
     if (f < t.dim) return t.opt.init_range != 0.0f ? init_weight(t.opt.init_range, key, f) : 0.0f;
@@ -325,6 +334,7 @@ __global__ __launch_bounds__(BLOCK) void assign_rows_kernel(TableDev t, const u6
         if (tid == 0) {
             t.counters[CNT_ROWS] = entry + sum;
             if (entry + sum > t.max_rows) t.counters[CNT_OVERFLOW] = 1u;
+            publish_rows(t, entry + sum);
         }
         if (mine == 0) return;
         sum = 0;
@@ -573,6 +583,9 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
     const u32 wv = threadIdx.x >> 6;
     const u32 w = blockIdx.x * (SEG_BLOCK / 64) + wv;
     if (w >= n_chunks) return;  // no workgroup barriers below
+    // a sort that gave up (a tile's bounded wait ran out) left pairs that are not grouped by row:
+    // nothing is applied, the host reports the push as failed
+    if (t.counters[CNT_SORT_ERR]) return;
     char* base = reinterpret_cast<char*>(seg_lds) + (size_t)wv * (val_bytes + 3 * arr_bytes);
     T* s_val = reinterpret_cast<T*>(base);
     u32* s_row = reinterpret_cast<u32*>(base + val_bytes);
@@ -806,6 +819,7 @@ __global__ __launch_bounds__(BLOCK) void fixup_kernel(TableDev t, const uint4* _
     const u32 lane = threadIdx.x & 63u;
     const u32 w = blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
     if (w >= n_chunks) return;
+    if (t.counters[CNT_SORT_ERR]) return;  // the sort gave up: segreduce_kernel wrote no partial sums
     const uint4 h = part_hdr[w];
     if (!(h.w & 1u)) return;  // wave-uniform
     const u32 col0 = blockIdx.y * 64u;
@@ -975,6 +989,7 @@ __global__ __launch_bounds__(SMALL_PUSH) void push_small_kernel(TableDev t, cons
         t.counters[CNT_ENTRY] = entry;
         t.counters[CNT_ROWS] = entry + n_won;
         if (entry + n_won > t.max_rows) t.counters[CNT_OVERFLOW] = 1u;
+        publish_rows(t, entry + n_won);
     }
     __threadfence();
     __syncthreads();

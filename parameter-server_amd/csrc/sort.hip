@@ -44,6 +44,7 @@ constexpr u32 RADIX_MAX = 1u << MAX_BITS;  // = SORT_BLOCK: a thread per digit
 constexpr u32 MAX_PASSES = 4;
 constexpr u32 FLAG_READY = 1u << 30, COUNT_MASK = (1u << 30) - 1u;
 constexpr u32 SPIN_LIMIT = 1u << 24;
+u32 g_spin_limit = SPIN_LIMIT;  // polls a tile grants a predecessor (sort_set_spin_limit)
 constexpr u32 GROUP = 16;                      // tiles per group of the two-level tile prefix
 constexpr u32 LOOKBACK_TILES = GROUP * GROUP;  // largest input of the one-launch passes, in tiles
 
@@ -224,8 +225,12 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_scan_kernel(u32* __restrict__
 // Sum of `count` (<= GROUP) published words spaced RADIX_MAX apart, starting at `words`. The loads
 // are issued together; the batch is fetched again until every word carries FLAG_READY. The wait is
 // bounded: past SPIN_LIMIT polls the caller gets what is there and *err_flag is raised.
-__device__ __forceinline__ u32 wait_sum(const u32* words, u32 count, u32* err_flag) {
+__device__ __forceinline__ u32 wait_sum(const u32* words, u32 count, u32* err_flag, u32 spin_limit) {
     if (count == 0) return 0;
+    if (spin_limit == 0) {  // no patience at all: the host asked for the failure path
+        *err_flag = 1u;
+        return 0;
+    }
     u32 spins = 0;
     while (true) {
         u32 sw[GROUP];
@@ -241,7 +246,7 @@ __device__ __forceinline__ u32 wait_sum(const u32* words, u32 count, u32* err_fl
             sum += sw[q] & COUNT_MASK;
         }
         if (ready & FLAG_READY) return sum;
-        if (++spins > SPIN_LIMIT) {  // never expected; keeps the grid from hanging
+        if (++spins > spin_limit) {  // never expected; keeps the grid from hanging
             *err_flag = 1u;
             return sum;
         }
@@ -257,7 +262,7 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
     const u32* __restrict__ kin, const u32* __restrict__ vin, u32* __restrict__ kout,
     u32* __restrict__ vout, u32 n, u32 shift, const u32* __restrict__ totals,
     u32* __restrict__ totals_next, u32* status, u32* group_status, const u32* __restrict__ first_pos,
-    u32 n_tiles, u32* err_flag) {
+    u32 n_tiles, u32* err_flag, u32 spin_limit) {
     constexpr u32 RADIX = 1u << BITS;
     // 32 KiB used twice: the per-wave digit counts (16 bits each: a wave holds 256 pairs, a tile
     // 4096) while ranking, then the tile's pairs in digit order
@@ -354,14 +359,14 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(
             const u32 b = tid;
             const u32 grp = tile / GROUP, first = grp * GROUP;
             // (a) the tiles before this one in its group of GROUP: one batch of loads
-            const u32 in_group = wait_sum(status + (size_t)first * RADIX_MAX + b, tile - first, err_flag);
+            const u32 in_group = wait_sum(status + (size_t)first * RADIX_MAX + b, tile - first, err_flag, spin_limit);
             // the last tile of a group (or of the input) publishes the group's total
             if (tile + 1 == first + GROUP || tile + 1 == n_tiles)
                 __hip_atomic_store(group_status + (size_t)grp * RADIX_MAX + b,
                                    FLAG_READY | ((in_group + tile_count) & COUNT_MASK), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
             // (b) the groups before this one (at most GROUP - 1): one more batch
-            gpos = digit_base + in_group + wait_sum(group_status + b, grp, err_flag);
+            gpos = digit_base + in_group + wait_sum(group_status + b, grp, err_flag, spin_limit);
         }
     }
     if (tid < RADIX) {
@@ -520,17 +525,17 @@ hipError_t launch_pass(u32 bits, u32 n_tiles, hipStream_t s, const u32* kin, con
         case 8:
             sort_pass_kernel<8, LOOKBACK><<<n_tiles, SORT_BLOCK, 0, s>>>(
                 kin, vin, kout, vout, n, shift, totals, totals_next, status, group_status, first_pos,
-                n_tiles, err_flag);
+                n_tiles, err_flag, g_spin_limit);
             break;
         case 9:
             sort_pass_kernel<9, LOOKBACK><<<n_tiles, SORT_BLOCK, 0, s>>>(
                 kin, vin, kout, vout, n, shift, totals, totals_next, status, group_status, first_pos,
-                n_tiles, err_flag);
+                n_tiles, err_flag, g_spin_limit);
             break;
         case 10:
             sort_pass_kernel<10, LOOKBACK><<<n_tiles, SORT_BLOCK, 0, s>>>(
                 kin, vin, kout, vout, n, shift, totals, totals_next, status, group_status, first_pos,
-                n_tiles, err_flag);
+                n_tiles, err_flag, g_spin_limit);
             break;
         default: return hipErrorInvalidValue;
     }
@@ -550,6 +555,8 @@ size_t sort_pairs_temp_bytes(size_t n) {
 }
 
 size_t sort_pairs_head_bytes() { return OFF_ROWS * 4; }
+
+void sort_set_spin_limit(uint32_t polls) { g_spin_limit = polls == ~0u ? SPIN_LIMIT : polls; }
 
 hipError_t sort_begin(void* temp, size_t temp_bytes, unsigned parity, uint32_t* keys, size_t n,
                       unsigned end_bit, SortPlan* plan, hipStream_t s, const SortLateKeys* late) {

@@ -48,11 +48,13 @@ struct TableDev {
     uint64_t* row_keys;  // max_rows
     uint32_t* counters;  // CNT_WORDS
     uint8_t* dirty;      // max_rows bytes, or null: 1 = a push updated the row since the last take
+    unsigned long long* pub;  // page-locked host word: {op_seq, rows} as the last inserting operation left them
     uint32_t bucket_mask;
     uint32_t max_rows;
     uint32_t dim;       // weights per key
     uint32_t vf;        // floats per value = dim * (1 + state blocks)
     uint32_t stride_f;  // floats between rows, multiple of 4
+    uint32_t op_seq;    // number of the inserting operation this launch belongs to (set per launch)
     OptParams opt;
 };
 
@@ -223,6 +225,10 @@ hipError_t launch_reinsert(const TableDev& t, uint32_t n_rows, hipStream_t s);
 // and is kept zeroed by the sorts themselves as long as `parity` alternates 0,1,0,1,...
 size_t sort_pairs_temp_bytes(size_t n);
 size_t sort_pairs_head_bytes();
+// How many times a tile of a one-launch pass polls for a predecessor's counts before it gives up
+// and raises the error flag (~0u = the default). 0 makes every waiting tile give up at once: the
+// way a test reaches the failure path while every kernel still runs to its end.
+void sort_set_spin_limit(uint32_t polls);
 // The same sort step by step (sort_begin counts, then sort_pass places digit p = 0 .. passes-1,
 // alternating between the two buffer pairs), for callers that time or interleave the launches.
 // late (may be null): every keys[i] equal to late->marker is first replaced (for inputs of more

@@ -235,7 +235,8 @@ def test_push_zipf_within_tolerance(ps, orc, wl, opt, dim, s, batch):
         mult[np.searchsorted(a["key"], uk)] = cnt
         assert_push_parity(a, b, c, mult)
         # next step: everyone restarts from the reference-order state
-        assert t.set(b["key"], b["value"]) == 0 and x.set(b["key"], b["value"]) == 0
+        assert t.set(b["key"], b["value"]) == 0, t.last_error()
+        assert x.set(b["key"], b["value"]) == 0
     assert t.size() == r.size()
     t.close()
 
@@ -825,4 +826,35 @@ def test_iterate_keys_follows_the_record_order(ps, orc, wl):
     seen = np.concatenate(seen)
     assert seen.size == n and np.array_equal(np.sort(seen), np.sort(r.dump()[1]["key"]))
     assert t.iterate_keys(0, 0)[1].size == 0
+    t.close()
+
+
+def test_sort_that_gives_up_applies_nothing(ps, orc, wl):
+    """A tile of the aggregation sort that gives up its bounded wait raises a flag; the kernels
+    after the sort then leave the rows alone and the table reports FATAL until it is cleared. The
+    host makes the wait give up (a limit of zero polls): every kernel still runs to its end."""
+    rng = np.random.default_rng(21)
+    n_table, dim, n = 30000, 8, 20000          # 5 tiles of 4096 pairs: one-launch passes that wait
+    t = ps.Table(dim, capacity=n_table + n, optimizer=1, lr=0.5)
+    keys = wl.table_keys_np(0, n_table, seed=7)
+    vals = rng.normal(0, 0.01, (n_table, dim)).astype(np.float32)
+    assert t.set(keys, vals) == 0
+    q = keys[rng.integers(0, n_table, n)]
+    g = rng.normal(0, 1.0, (n, dim)).astype(np.float32)
+    try:
+        ps.debug_sort_spin_limit(0)
+        assert t.push(q, g) == 0                # enqueued; the failure shows at the next counter read
+    finally:
+        ps.debug_sort_spin_limit()
+    with pytest.raises(ps.PshbmError) as e:
+        t.size()
+    assert e.value.status == ps.FATAL and "not applied" in str(e.value)
+    assert t.push(q, g) == 0                    # later pushes are refused on the device as well
+    st, rows, hit = t.pull(keys)
+    assert st == 0 and hit.all()
+    np.testing.assert_array_equal(rows, vals)   # no row was touched
+    assert t.clear() == 0 and t.size() == 0
+    assert t.set(keys, vals) == 0 and t.push(q, g) == 0 and t.size() == n_table
+    st, rows, hit = t.pull(keys)
+    assert not np.array_equal(rows, vals)
     t.close()
