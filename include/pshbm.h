@@ -160,6 +160,19 @@ int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, siz
 int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
                        uint32_t flags, void* stream);
 
+/* pshbm_push_dev for callers that cannot allocate device memory while they run: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid it. It has no counterpart in the reference.
+ * The scratch of the push (probe results, sort buffers, partial sums) lies in a fixed array of
+ * about 2.8 MB inside the library, one copy per device, instead of the table's workspace, and the
+ * call allocates nothing on the device or through any library; it synchronizes only where
+ * pshbm_push_dev does (a table within n keys of its capacity). Limits: n <= 16384 keys and
+ * n * dim <= 2^20 gradient floats per call, PSHBM_ERROR beyond. Results are those of pshbm_push_dev.
+ * All tables of a device share the one array: calls that overlap on the device (different streams,
+ * no ordering between them) race on it, also across tables; calls on one stream, or ordered by
+ * events, are safe. */
+int32_t pshbm_push_dev_noalloc(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
+                               uint32_t flags, void* stream);
+
 /* Same, from the wire layout of a push block: n records of std::pair<KEY, PUSH_VALUE> laid out
  * back to back (SparsePushOperator.h:176-177,246-247), i.e. a uint64 key then dim floats, every
  * `stride` bytes (stride >= 8 + 4*dim, a multiple of 4). */

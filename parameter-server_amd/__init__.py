@@ -34,7 +34,7 @@ SYMBOLS = [
     "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve", "pshbm_set_hyperparameters", "pshbm_set_memory_limit", "pshbm_device_memory",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
-    "pshbm_debug_sort_spin_limit",
+    "pshbm_push_dev_noalloc", "pshbm_debug_sort_spin_limit",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
           "fixup_windows", "assign_rows", "push_small"]
@@ -183,6 +183,7 @@ def lib():
         L.pshbm_pull_dev.argtypes = [vp, vp, sz, vp, vp, u32, vp]
         L.pshbm_push.argtypes = [vp, vp, vp, sz, u32]
         L.pshbm_push_dev.argtypes = [vp, vp, vp, sz, u32, vp]
+        L.pshbm_push_dev_noalloc.argtypes = [vp, vp, vp, sz, u32, vp]
         L.pshbm_debug_sort_spin_limit.argtypes = [u32]
         L.pshbm_push_pairs.argtypes = [vp, vp, sz, sz, u32]
         L.pshbm_queue.argtypes = [vp, vp, vp, sz]
@@ -492,6 +493,10 @@ class Table:
 
     def push_dev(self, d_keys, d_grads, n, flags=0, stream=0):
         return lib().pshbm_push_dev(self._h, d_keys, d_grads, n, flags, stream)
+
+    def push_dev_noalloc(self, d_keys, d_grads, n, flags=0, stream=0):
+        """push_dev with its scratch in the library's fixed device array: allocates nothing."""
+        return lib().pshbm_push_dev_noalloc(self._h, d_keys, d_grads, n, flags, stream)
 
     def queue_dev(self, d_keys, d_grads, n, stream=0):
         return lib().pshbm_queue_dev(self._h, d_keys, d_grads, n, stream)

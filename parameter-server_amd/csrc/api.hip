@@ -146,6 +146,42 @@ hipError_t dev_free(int device, void* p) {
     return ::hipFree(p);
 }
 
+// ---- scratch of the entry point that allocates nothing -------------------------------------------
+// pshbm_push_dev_noalloc takes the scratch of a push from this array instead of the table's growing
+// workspace. Every device the library runs on holds its own copy until the process ends; in host
+// code the array's name is only a stand-in, so the device address is looked up once per device
+// (scratch_init) and used from then on.
+constexpr size_t NOALLOC_MAX_KEYS = 16384;        // keys per call
+constexpr size_t NOALLOC_MAX_FLOATS = 1u << 20;   // keys * dim per call
+constexpr size_t NA_WON = 0;                                        // 2 x 17 words, then the sort buffers: one fill clears both
+constexpr size_t NA_SORT = 256;
+constexpr size_t NA_SORT_ROOM = 1u << 20;
+constexpr size_t NA_KEYS5 = NA_SORT + NA_SORT_ROOM;                 // slot, idx, row, srow, sidx
+constexpr size_t NA_HDR = NA_KEYS5 + 5 * NOALLOC_MAX_KEYS * 4;
+constexpr size_t NA_HDR_ROOM = (NOALLOC_MAX_KEYS / 8 + 1) * sizeof(uint4);
+constexpr size_t NA_PVAL = (NA_HDR + NA_HDR_ROOM + 255) / 256 * 256;
+constexpr size_t NA_PVAL_ROOM = NOALLOC_MAX_FLOATS + (256u << 10);  // bytes: chunks * 2 * dim floats
+constexpr size_t NA_WROW = NA_PVAL + NA_PVAL_ROOM;
+constexpr size_t NA_WROW_ROOM = 1024;
+constexpr size_t NA_WVAL = NA_WROW + NA_WROW_ROOM;
+constexpr size_t NA_WVAL_ROOM = 128u << 10;
+constexpr size_t NOALLOC_BYTES = NA_WVAL + NA_WVAL_ROOM;            // about 2.8 MB
+static __device__ __align__(256) unsigned char scratch[NOALLOC_BYTES];
+
+std::mutex g_scratch_mu;
+unsigned char* g_scratch_ptr[MAX_DEVICES] = {};
+
+// Device address of this device's copy of `scratch`; `device` must be current.
+hipError_t scratch_init(int device) {
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_ptr[device]) return hipSuccess;
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    g_scratch_ptr[device] = static_cast<unsigned char*>(p);
+    return hipSuccess;
+}
+
 }  // namespace
 
 struct pshbm_table {
@@ -757,6 +793,11 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     t->cfg.max_load_factor = lf;
     t->device = cfg->device;
     DeviceGuard g(t->device);
+    if (hipError_t se = scratch_init(t->device); se != hipSuccess) {
+        g_error = std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(se);
+        delete t;
+        return PSHBM_ERROR;
+    }
 
     const uint64_t max_rows = cfg->expected_max_items;
     uint64_t want_slots = (uint64_t)((double)max_rows / lf) + 1;
@@ -943,6 +984,59 @@ int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_gr
     DeviceGuard g(t->device);
     std::unique_lock<std::shared_mutex> lk(t->mu);
     return push_locked(t, d_keys, d_grads, n, flags, static_cast<hipStream_t>(stream));
+}
+
+// The same push with its scratch in the library's fixed device array: nothing is allocated, by this
+// call or by anything it calls. One array per device, shared by every table on it.
+int32_t pshbm_push_dev_noalloc(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
+                               uint32_t flags, void* stream) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!d_keys || !d_grads) return fail(t, PSHBM_ERROR, "push_noalloc: null buffer");
+    if (n > NOALLOC_MAX_KEYS || n * (size_t)t->d.dim > NOALLOC_MAX_FLOATS)
+        return fail(t, PSHBM_ERROR, "push_noalloc: at most %zu keys and %zu gradient floats per call (got %zu keys of dim %u)",
+                    NOALLOC_MAX_KEYS, NOALLOC_MAX_FLOATS, n, t->d.dim);
+    DeviceGuard g(t->device);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    std::lock_guard<std::mutex> sk(g_scratch_mu);  // one enqueue at a time per process; overlap on the device is the caller's to avoid
+    unsigned char* base = g_scratch_ptr[t->device];
+    if (!base) return fail(t, PSHBM_FATAL, "push_noalloc: the scratch array was not set up for device %d", t->device);
+    // what this batch needs of the array, by the same geometry the kernels use
+    const SegGeom g1 = seg_geometry(t->d.dim, 1, n);
+    const SegGeom g4 = seg_geometry(t->d.dim, (t->d.dim % 4 == 0) ? 4 : 1, n);
+    const size_t chunks = std::max(g1.n_chunks, g4.n_chunks);
+    if (sort_pairs_temp_bytes(n) > NA_SORT_ROOM || chunks * sizeof(uint4) > NA_HDR_ROOM ||
+        chunks * 2 * (size_t)t->d.dim * 4 > NA_PVAL_ROOM || (chunks / 64 + 1) * 4 > NA_WROW_ROOM ||
+        (chunks / 64 + 1) * (size_t)t->d.dim * 4 > NA_WVAL_ROOM || 2 * (assign_blocks(n) + 1) * 4 > NA_SORT - NA_WON)
+        return fail(t, PSHBM_ERROR, "push_noalloc: a batch of %zu keys of dim %u does not fit the fixed scratch", n, t->d.dim);
+    ST_TRY(begin_op(t, s));
+    Workspace w{};
+    uint32_t* k5 = reinterpret_cast<uint32_t*>(base + NA_KEYS5);
+    w.slot = k5;
+    w.idx = k5 + NOALLOC_MAX_KEYS;
+    w.row = k5 + 2 * NOALLOC_MAX_KEYS;
+    w.srow = k5 + 3 * NOALLOC_MAX_KEYS;
+    w.sidx = k5 + 4 * NOALLOC_MAX_KEYS;
+    w.sort = base + NA_SORT;
+    w.sort_bytes = NA_SORT_ROOM;
+    w.sort_parity = 0;
+    w.hdr = reinterpret_cast<uint4*>(base + NA_HDR);
+    w.pval = reinterpret_cast<float*>(base + NA_PVAL);
+    w.wrow = reinterpret_cast<uint32_t*>(base + NA_WROW);
+    w.wval = reinterpret_cast<float*>(base + NA_WVAL);
+    w.won_words = assign_blocks(NOALLOC_MAX_KEYS) + 1;
+    w.won_cur = reinterpret_cast<uint32_t*>(base + NA_WON);
+    w.won_next = w.won_cur + w.won_words;
+    // The array keeps what the last call left: the winner counts and the sort's digit totals must
+    // start at zero (a fill kernel, not a memset: the call may be recorded into a graph).
+    HIP_TRY(t, launch_fill_u32(reinterpret_cast<uint32_t*>(base + NA_WON), (NA_SORT + sort_pairs_head_bytes()) / 4, 0u, s));
+    const bool prof = t->prof_on;  // the per-kernel timers create events on demand
+    t->prof_on = false;
+    bool used_head = false, used_won = false;
+    const int32_t st = push_with(t, w, d_keys, d_grads, n, flags, s, &used_head, &used_won);
+    t->prof_on = prof;
+    return st;
 }
 
 // Keys and their n x `floats` values from host memory to where kernels on stream s can read them:
