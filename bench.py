@@ -45,7 +45,9 @@ KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist"
                    "fixup": "fixup_kernel", "fixup_windows": "fixup_windows_kernel",
                    "assign_rows": "assign_rows_kernel", "update_unique": "update_unique_kernel",
                    "push_small": "push_small_kernel",
-                   "gather": "gather_slots_kernel"}
+                   "gather": "gather_slots_kernel", "part_tile": "part_tile_kernel",
+                   "part_scan": "part_scan_kernel", "part_scatter": "part_scatter_kernel",
+                   "part_apply": "part_apply_kernel", "part_insert": "part_insert_kernel"}
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by the factors a plain
 # copy of known size gave), measured on an MI355X; the summaries are under profiles/.
 MEASURED_TRAFFIC_BYTES = {

@@ -367,7 +367,12 @@ int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out);
 #define PSHBM_PHASE_FIXUP_WINDOWS 8 /* window sums of runs that span many chunks */
 #define PSHBM_PHASE_ASSIGN_ROWS 9   /* rows for the slots an inserting operation claimed */
 #define PSHBM_PHASE_PUSH_SMALL 10   /* a whole push of a small batch in one launch */
-#define PSHBM_PHASES 12
+#define PSHBM_PHASE_PART_TILE 11    /* partitioned push: repeats inside a tile pre-summed, entries staged */
+#define PSHBM_PHASE_PART_SCAN 12    /* partitioned push: where each tile's entries go */
+#define PSHBM_PHASE_PART_SCATTER 13 /* partitioned push: entries moved into partition order */
+#define PSHBM_PHASE_PART_APPLY 14   /* partitioned push: one probe, sum and update per distinct key */
+#define PSHBM_PHASE_PART_INSERT 15  /* partitioned push: rows for the keys it inserted */
+#define PSHBM_PHASES 16
 typedef struct pshbm_profile {
     double ms[PSHBM_PHASES];
     uint64_t launches[PSHBM_PHASES];
@@ -396,6 +401,10 @@ int32_t pshbm_device_memory(int32_t device, uint64_t* in_use, uint64_t* limit);
  * waiting tile give up at once, which is how the tests reach that path while every kernel still
  * runs to its end. Process-wide. */
 int32_t pshbm_debug_sort_spin_limit(uint32_t polls);
+/* Test hook, no counterpart in the reference: entries one pass of the partitioned push's apply
+ * kernel takes (0 = the default, 2048). A small value makes ordinary batches go through the
+ * several-passes path that otherwise only partitions crowded by hot keys take. Process-wide. */
+int32_t pshbm_debug_part_pass_capacity(uint32_t entries);
 
 /* Pinned (page-locked) host memory for request/response buffers of the host-pointer entry points.
  * Buffers from here (or from hipHostMalloc) spare the staging copies: pshbm_pull and pshbm_push

@@ -34,10 +34,11 @@ SYMBOLS = [
     "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve", "pshbm_set_hyperparameters", "pshbm_set_memory_limit", "pshbm_device_memory",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
-    "pshbm_push_dev_noalloc", "pshbm_debug_sort_spin_limit",
+    "pshbm_push_dev_noalloc", "pshbm_debug_sort_spin_limit", "pshbm_debug_part_pass_capacity",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
-          "fixup_windows", "assign_rows", "push_small"]
+          "fixup_windows", "assign_rows", "push_small", "part_tile", "part_scan", "part_scatter", "part_apply",
+          "part_insert"]
 
 
 class Config(C.Structure):
@@ -132,7 +133,7 @@ def update(op, first_column, n_columns, a, b):
 
 
 class Profile(C.Structure):
-    _fields_ = [("ms", C.c_double * 12), ("launches", C.c_uint64 * 12)]
+    _fields_ = [("ms", C.c_double * 16), ("launches", C.c_uint64 * 16)]
 
 
 class PshbmError(RuntimeError):
@@ -185,6 +186,7 @@ def lib():
         L.pshbm_push_dev.argtypes = [vp, vp, vp, sz, u32, vp]
         L.pshbm_push_dev_noalloc.argtypes = [vp, vp, vp, sz, u32, vp]
         L.pshbm_debug_sort_spin_limit.argtypes = [u32]
+        L.pshbm_debug_part_pass_capacity.argtypes = [u32]
         L.pshbm_push_pairs.argtypes = [vp, vp, sz, sz, u32]
         L.pshbm_queue.argtypes = [vp, vp, vp, sz]
         L.pshbm_queue_dev.argtypes = [vp, vp, vp, sz, vp]
@@ -248,6 +250,11 @@ def device_memory(device=0):
 def debug_sort_spin_limit(polls=0xFFFFFFFF):
     """Test hook: polls a sort tile grants its predecessors (default 2^24; 0 = give up at once)."""
     return lib().pshbm_debug_sort_spin_limit(polls)
+
+
+def debug_part_pass_capacity(entries=0):
+    """Test hook: entries one pass of the partitioned push's apply kernel takes (0 = default)."""
+    return lib().pshbm_debug_part_pass_capacity(entries)
 
 
 def init_weight(init_range, key, column):

@@ -48,6 +48,8 @@ struct Workspace {
     float* wval;
     uint32_t *won_cur, *won_next;  // per-block winner counts: counted into / zeroed for the next operation
     size_t won_words;
+    PartBufs part;    // scratch of the partitioned push, for batches of up to part_keys keys (0: none)
+    size_t part_keys;
 };
 
 // Is [p, p + bytes) page-locked host memory that the runtime knows (hipHostMalloc,
@@ -201,6 +203,10 @@ struct pshbm_table {
     unsigned sort_parity = 0;  // which half of the sort head the next sort uses
     DevBuf ws_slot, ws_row, ws_idx, ws_srow, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wrow, ws_wval, ws_won;
     unsigned won_parity = 0;  // which half of ws_won the next inserting operation counts into
+    // scratch of the partitioned push (batches of PART_MIN_KEYS keys and more)
+    DevBuf pt_stage_key, pt_stage_ref, pt_ent_key, pt_ent_ref, pt_counts, pt_starts, pt_blocktot, pt_tile_total,
+        pt_pstart, pt_psum, pt_new_slot, pt_new_count, pt_ngrad;
+    size_t part_keys = 0;       // batch size those arrays serve
 
     // staging of the host-pointer entry points
     std::mutex st_mu;
@@ -377,6 +383,25 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     ST_TRY(ensure(t, t->ws_won, 2 * (assign_blocks(cap) + 1) * 4));
     HIP_TRY(t, hipMemset(t->ws_won.p, 0, t->ws_won.bytes));
     t->won_parity = 0;
+    PartPlan probe_plan;
+    if (cap >= PART_MIN_KEYS && part_plan(t->d, std::min(cap, PART_MAX_KEYS), &probe_plan)) {
+        const size_t pk = std::min(cap, PART_MAX_KEYS);
+        const PartSizes z = part_sizes(t->d.dim, pk);
+        ST_TRY(ensure(t, t->pt_stage_key, z.stage_key));
+        ST_TRY(ensure(t, t->pt_stage_ref, z.stage_ref));
+        ST_TRY(ensure(t, t->pt_ent_key, z.ent_key));
+        ST_TRY(ensure(t, t->pt_ent_ref, z.ent_ref));
+        ST_TRY(ensure(t, t->pt_counts, z.counts));
+        ST_TRY(ensure(t, t->pt_starts, z.starts));
+        ST_TRY(ensure(t, t->pt_blocktot, z.blocktot));
+        ST_TRY(ensure(t, t->pt_tile_total, z.tile_total));
+        ST_TRY(ensure(t, t->pt_pstart, z.pstart));
+        ST_TRY(ensure(t, t->pt_psum, z.psum));
+        ST_TRY(ensure(t, t->pt_new_slot, z.new_slot));
+        ST_TRY(ensure(t, t->pt_new_count, z.new_count));
+        ST_TRY(ensure(t, t->pt_ngrad, z.ngrad));
+        t->part_keys = pk;
+    }
     t->ws_cap = cap;
     return PSHBM_OK;
 }
@@ -421,6 +446,9 @@ int32_t read_counters(pshbm_table* t, hipStream_t s) {
         return fail(t, PSHBM_FATAL, "a radix-sort tile timed out waiting for its predecessor: the push it "
                                     "belonged to, and every push since, was not applied (keys they inserted "
                                     "keep their initial values); pshbm_clear resets the table");
+    if (t->h_counters[CNT_PART_ERR])
+        return fail(t, PSHBM_FATAL, "a partition of a push held more entries of one hash class than a pass takes: "
+                                    "that push was applied in part; pshbm_clear resets the table");
     return PSHBM_OK;
 }
 
@@ -535,15 +563,32 @@ Workspace table_workspace(pshbm_table* t) {
     w.won_cur = static_cast<uint32_t*>(t->ws_won.p) + (t->won_parity & 1u) * half;
     w.won_next = static_cast<uint32_t*>(t->ws_won.p) + ((t->won_parity & 1u) ^ 1u) * half;
     w.won_words = half;
+    w.part_keys = t->part_keys;
+    if (t->part_keys) {
+        w.part.stage_key = static_cast<uint64_t*>(t->pt_stage_key.p);
+        w.part.stage_ref = static_cast<uint32_t*>(t->pt_stage_ref.p);
+        w.part.ent_key = static_cast<uint64_t*>(t->pt_ent_key.p);
+        w.part.ent_ref = static_cast<uint32_t*>(t->pt_ent_ref.p);
+        w.part.counts = static_cast<uint32_t*>(t->pt_counts.p);
+        w.part.starts = static_cast<uint32_t*>(t->pt_starts.p);
+        w.part.blocktot = static_cast<uint32_t*>(t->pt_blocktot.p);
+        w.part.tile_total = static_cast<uint32_t*>(t->pt_tile_total.p);
+        w.part.pstart = static_cast<uint32_t*>(t->pt_pstart.p);
+        w.part.psum = static_cast<float*>(t->pt_psum.p);
+        w.part.new_slot = static_cast<uint32_t*>(t->pt_new_slot.p);
+        w.part.new_count = static_cast<uint32_t*>(t->pt_new_count.p);
+        w.part.ngrad = static_cast<float*>(t->pt_ngrad.p);
+    }
     return w;
 }
 
 // One push on stream s with the scratch of `w`. *used_sort_head: the sort took the half of the sort
 // head that w.sort_parity names (and zeroed the other one).
 int32_t push_with(pshbm_table* t, const Workspace& w, const uint64_t* d_keys, const float* d_grads, size_t n,
-                  uint32_t flags, hipStream_t s, bool* used_sort_head, bool* used_won) {
+                  uint32_t flags, hipStream_t s, bool* used_sort_head, bool* used_won, bool* used_part) {
     *used_sort_head = false;
     *used_won = false;
+    *used_part = false;
     const bool insert = !(flags & PSHBM_PUSH_NO_INSERT);
     const bool unique = (flags & PSHBM_PUSH_ASSUME_UNIQUE) != 0;
     bool checked = false;
@@ -553,6 +598,18 @@ int32_t push_with(pshbm_table* t, const Workspace& w, const uint64_t* d_keys, co
     // table is nearly full: undoing a batch that does not fit needs the separate steps.)
     if (!unique && !checked && n <= push_small_max()) {
         HIP_TRY_PROF(t, s, PSHBM_PHASE_PUSH_SMALL, launch_push_small(t->d, d_keys, d_grads, n, insert, s));
+        return PSHBM_OK;
+    }
+    // A large batch is cut into tiles and partitions (push_part.hip): no global sort, one probe per
+    // distinct key. (Not in checked mode: it updates rows in the launch that claims slots.)
+    PartPlan pl;
+    if (!unique && !checked && n <= w.part_keys && part_plan(t->d, n, &pl)) {
+        *used_part = true;
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_TILE, launch_part_tile(t->d, pl, w.part, d_keys, d_grads, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_SCAN, launch_part_scan(pl, w.part, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_SCATTER, launch_part_scatter(t->d, pl, w.part, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_APPLY, launch_part_apply(t->d, pl, w.part, d_grads, insert, s));
+        if (insert) HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_INSERT, launch_part_insert(t->d, pl, w.part, d_grads, s));
         return PSHBM_OK;
     }
     // Everything after the probe works on row ids: they are dense, so the sort needs fewer bits
@@ -596,8 +653,8 @@ int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads
     ST_TRY(begin_op(t, s));
     ST_TRY(ensure_workspace(t, n));
     const Workspace w = table_workspace(t);
-    bool used_head = false, used_won = false;
-    const int32_t st = push_with(t, w, d_keys, d_grads, n, flags, s, &used_head, &used_won);
+    bool used_head = false, used_won = false, used_part = false;
+    const int32_t st = push_with(t, w, d_keys, d_grads, n, flags, s, &used_head, &used_won, &used_part);
     if (used_head) ++t->sort_parity;
     if (used_won) ++t->won_parity;
     return st;
@@ -643,6 +700,9 @@ void destroy_impl(pshbm_table* t) {
     DevBuf* bufs[] = {&t->ws_slot, &t->ws_row, &t->ws_idx,  &t->ws_srow, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
                       &t->ws_pval, &t->ws_wrow, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_raw,
                       &t->ms_dead, &t->ms_tiles, &t->ms_lists, &t->ms_fe,
+                      &t->pt_stage_key, &t->pt_stage_ref, &t->pt_ent_key, &t->pt_ent_ref, &t->pt_counts, &t->pt_starts,
+                      &t->pt_blocktot, &t->pt_tile_total, &t->pt_pstart, &t->pt_psum, &t->pt_new_slot, &t->pt_new_count,
+                      &t->pt_ngrad,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
         if (b->p) (void)dev_free(t->device, b->p);
@@ -799,6 +859,11 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
         return PSHBM_ERROR;
     }
 
+    if (hipError_t pe = part_init(); pe != hipSuccess) {
+        g_error = std::string("hipFuncSetAttribute (LDS of the partitioned push): ") + hipGetErrorString(pe);
+        delete t;
+        return PSHBM_ERROR;
+    }
     const uint64_t max_rows = cfg->expected_max_items;
     uint64_t want_slots = (uint64_t)((double)max_rows / lf) + 1;
     uint64_t nb = 16;
@@ -1033,8 +1098,8 @@ int32_t pshbm_push_dev_noalloc(pshbm_table* t, const uint64_t* d_keys, const flo
     HIP_TRY(t, launch_fill_u32(reinterpret_cast<uint32_t*>(base + NA_WON), (NA_SORT + sort_pairs_head_bytes()) / 4, 0u, s));
     const bool prof = t->prof_on;  // the per-kernel timers create events on demand
     t->prof_on = false;
-    bool used_head = false, used_won = false;
-    const int32_t st = push_with(t, w, d_keys, d_grads, n, flags, s, &used_head, &used_won);
+    bool used_head = false, used_won = false, used_part = false;  // (w.part_keys = 0: never the partitioned path)
+    const int32_t st = push_with(t, w, d_keys, d_grads, n, flags, s, &used_head, &used_won, &used_part);
     t->prof_on = prof;
     return st;
 }
@@ -1862,6 +1927,11 @@ int32_t pshbm_profile_read(pshbm_table* t, pshbm_profile* out) {
 
 int32_t pshbm_debug_sort_spin_limit(uint32_t polls) {
     sort_set_spin_limit(polls);
+    return PSHBM_OK;
+}
+
+int32_t pshbm_debug_part_pass_capacity(uint32_t entries) {
+    part_set_pass_capacity(entries);
     return PSHBM_OK;
 }
 

@@ -7,6 +7,7 @@
 // response.
 #include "table.h"
 #include "probe.h"
+#include "rowops.h"
 
 namespace pshbm {
 
@@ -14,45 +15,6 @@ namespace {
 
 constexpr u32 WON_BIT = 0x80000000u;  // in a located slot index: this key claimed the slot in this launch
 constexpr u32 ASSIGN_KEYS = 1024;     // keys per workgroup of assign_rows_kernel
-
-// ---- small vector helpers ------------------------------------------------------------------
-__device__ __forceinline__ float vzero(float) { return 0.0f; }
-__device__ __forceinline__ float4 vzero(float4) { return make_float4(0.f, 0.f, 0.f, 0.f); }
-__device__ __forceinline__ float vadd(float a, float b) { return a + b; }
-__device__ __forceinline__ float4 vadd(float4 a, float4 b) {
-    return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
-}
-// n / d for n*d < 2^32 by one multiply: m = ceil(2^32 / d) (d == 1 handled by m = 2^32).
-__device__ __forceinline__ u32 div_small(u32 n, u64 m) { return (u32)(((u64)n * m) >> 32); }
-// n / d for any 64-bit n by one multiply-high: m = ceil(2^64 / d), d >= 2.
-__device__ __forceinline__ u64 div_big(u64 n, u64 m, u32 d) { return d == 1 ? n : __umul64hi(n, m); }
-
-inline u64 magic32(u32 d) { return ((1ull << 32) + d - 1) / d; }
-inline u64 magic64(u32 d) { return d <= 1 ? 0 : (~0ull / d) + 1; }
-
-// The row count an inserting operation leaves, told to the host without a round trip: one 64-bit
-// word in page-locked memory, {operation number, rows}. The host adds the sizes of the operations
-// it has enqueued since to get an upper bound of the row count.
-__device__ __forceinline__ void publish_rows(const TableDev& t, u32 rows) {
-    if (t.pub)
-        __hip_atomic_store(t.pub, ((unsigned long long)t.op_seq << 32) | rows, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_SYSTEM);
-}
-
-// float f of the value a key starts with: weights, then optimizer state
-__device__ __forceinline__ float init_float(const TableDev& t, u64 key, u32 f) {
-    if (f < t.dim) return t.opt.init_range != 0.0f ? init_weight(t.opt.init_range, key, f) : 0.0f;
-    return t.opt.kind == 2 /*ADAGRAD*/ ? t.opt.init_acc : 0.0f;
-}
-// the weights a pull answers for a key that is not stored (init_store_value + fetch_pull_value of
-// pico-ps/operator/SparsePullOperator.h:217,226), column unit c of T
-__device__ __forceinline__ float init_pulled(const TableDev& t, u64 key, u32 c, float) {
-    return init_weight(t.opt.init_range, key, c);
-}
-__device__ __forceinline__ float4 init_pulled(const TableDev& t, u64 key, u32 c, float4) {
-    return make_float4(init_weight(t.opt.init_range, key, c * 4), init_weight(t.opt.init_range, key, c * 4 + 1),
-                       init_weight(t.opt.init_range, key, c * 4 + 2), init_weight(t.opt.init_range, key, c * 4 + 3));
-}
 
 // ---- row gather into the packed response -----------------------------------------------------
 // `row` holds, in the lanes of group k, the row of key base + k (ROW_NONE = miss -> the weights a
@@ -130,113 +92,6 @@ __global__ __launch_bounds__(BLOCK) void gather_slots_kernel(TableDev t,
 }
 
 // ---- locate / claim ------------------------------------------------------------------------
-struct Located {
-    u32 slot;  // slot of the key, SLOT_NONE if it is neither stored nor claimable
-    u32 row;   // its row; ROW_PENDING if the slot was claimed in this launch (by this call or another)
-    bool won;  // this call claimed the slot
-    bool dup;  // the key was there already, or another call of this launch claimed it
-};
-
-// Four lanes (sub = 0..3 of group grp) find `key` or claim a slot for it. Every lane of the
-// wavefront must call this; lanes whose `active` is false only take part in the ballots.
-// need_row: also fetch the row word where the key is found by the slow path.
-__device__ __forceinline__ Located find_or_claim(const TableDev& t, u64 key, bool active, u32 grp,
-                                                 u32 sub, bool need_row) {
-    Located r{SLOT_NONE, ROW_NONE, false, false};
-    // Most keys of a batch are stored already: look for them with ordinary cached loads first.
-    // What those loads show may be older than this launch, never wrong: a key that is seen is
-    // stored (slots only go from empty to a key), and a key that is not seen is dealt with below.
-    const Found f = probe_find(t, key, active, grp, sub);
-    if (f.slot != SLOT_NONE) {
-        r.slot = f.slot;
-        r.row = f.row < t.max_rows ? f.row : ROW_PENDING;
-        r.dup = true;
-    }
-    bool done = !active || f.slot != SLOT_NONE;
-    u32 b = (u32)hash64(key) & t.bucket_mask;
-    u32 steps = 0;
-    // A key that is not seen goes straight for the first slot that looked empty. The view may be
-    // old, but only in one direction (slots go from empty to a key and stay), so the first slot
-    // that is truly empty is not before this one, and a copy of the key that another group stored
-    // during this launch is either seen, or in this slot, or behind a slot that looked empty and
-    // is not -- the compare-and-swap tells which: it finds the slot empty (claimed), holding the
-    // key (a repeat), or holding another key (then the bucket is looked at again, with loads that
-    // bypass the caches).
-    if (__ballot(!done)) {
-        const bool try_it = !done && f.empty != SLOT_NONE;
-        u64 old = 0;
-        if (try_it && sub == 0)
-            old = atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[f.empty]),
-                            (unsigned long long)KEY_EMPTY, (unsigned long long)key);
-        const u64 oldb = shfl64(old, grp * 4);
-        if (try_it) {
-            b = f.empty >> 2;  // the buckets before it are full and stay full
-            if (oldb == KEY_EMPTY || oldb == key) {
-                r.slot = f.empty;
-                r.row = ROW_PENDING;
-                r.won = oldb == KEY_EMPTY;
-                r.dup = !r.won;
-                done = true;
-            }
-        }
-    }
-    while (__ballot(!done)) {
-        u64 skey = 0;
-        u32 srow = ROW_NONE;
-        // Coherent at the device level: a slot claimed by another compute unit during this
-        // launch must be seen, so the loads bypass the per-CU cache.
-        if (!done) {
-            uint4* sp = &t.slots[(u64)b * 4 + sub];
-            skey = __hip_atomic_load(reinterpret_cast<u64*>(sp), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (need_row)
-                srow = __hip_atomic_load(reinterpret_cast<u32*>(sp) + 2, __ATOMIC_RELAXED,
-                                         __HIP_MEMORY_SCOPE_AGENT);
-        }
-        const bool match = !done && skey == key;
-        const bool empty = !done && skey == KEY_EMPTY;
-        const u32 m4 = (u32)(__ballot(match) >> (grp * 4)) & 0xFu;
-        const u32 e4 = (u32)(__ballot(empty) >> (grp * 4)) & 0xFu;
-        const u32 tgt = e4 ? (u32)__ffs((int)e4) - 1u : 0u;
-        const bool do_cas = !done && !m4 && e4 && sub == tgt;
-        u64 old = 0;
-        if (do_cas)
-            old = atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[(u64)b * 4 + tgt]),
-                            (unsigned long long)KEY_EMPTY, (unsigned long long)key);
-        const u64 oldb = shfl64(old, grp * 4 + tgt);
-        const u32 msub = m4 ? (u32)__ffs((int)m4) - 1u : 0u;
-        const u32 mrow = __shfl(srow, (int)(grp * 4 + msub));
-        if (!done) {
-            if (m4) {
-                r.slot = b * 4 + msub;
-                // a key that another group claimed in this launch has no row yet
-                r.row = mrow < t.max_rows ? mrow : ROW_PENDING;
-                r.dup = true;
-                done = true;
-            } else if (e4) {
-                if (oldb == KEY_EMPTY) {
-                    r.slot = b * 4 + tgt;
-                    r.row = ROW_PENDING;
-                    r.won = true;
-                    done = true;
-                } else if (oldb == key) {  // the same key, claimed by another group
-                    r.slot = b * 4 + tgt;
-                    r.row = ROW_PENDING;
-                    r.dup = true;
-                    done = true;
-                }
-                // otherwise another key took the slot: look at this bucket again
-            } else {
-                b = (b + 1) & t.bucket_mask;
-                if (++steps > t.bucket_mask) {
-                    done = true;
-                    if (sub == 0) t.counters[CNT_OVERFLOW] = 1u;
-                }
-            }
-        }
-    }
-    return r;
-}
-
 template <bool kInsert>
 __global__ __launch_bounds__(BLOCK) void locate_kernel(TableDev t, const u64* __restrict__ keys,
                                                         u32 n, u32* __restrict__ slot_out,
@@ -403,91 +258,6 @@ __global__ __launch_bounds__(BLOCK) void rollback_kernel(TableDev t, const u32* 
 
 __global__ __launch_bounds__(BLOCK) void fill_u32_kernel(u32* p, u64 n, u32 v) {
     for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (u64)gridDim.x * BLOCK) p[i] = v;
-}
-
-// ---- optimizer step ------------------------------------------------------------------------
-// One fp32 element; each operation rounds on its own (the file is compiled with
-// -ffp-contract=off and correctly rounded divide / sqrt).
-template <int KIND>
-__device__ __forceinline__ void opt_step(const OptParams& o, float g, float& w, float& s1,
-                                         float& s2) {
-    if constexpr (KIND == 0) {  // SUM
-        w = w + g;
-    } else if constexpr (KIND == 1) {  // SGD
-        float step = o.lr * g;
-        w = w - step;
-    } else if constexpr (KIND == 2) {  // ADAGRAD: s1 = accumulator
-        float gg = g * g;
-        float nn = s1 + gg;
-        float num = o.lr * g;
-        float step = num / sqrtf(nn);
-        s1 = nn;
-        w = w - step;
-    } else {  // FTRL: s1 = z, s2 = n
-        float gg = g * g;
-        float n_new = s2 + gg;
-        float sq_new = sqrtf(n_new);
-        float sigma = (sq_new - sqrtf(s2)) / o.alpha;
-        float sw = sigma * w;
-        float z = (s1 + g) - sw;
-        float w_new;
-        if (fabsf(z) <= o.l1) {
-            w_new = 0.0f;
-        } else {
-            float shrunk = z > 0.0f ? z - o.l1 : z + o.l1;
-            float denom = (o.beta + sq_new) / o.alpha + o.l2;
-            w_new = -shrunk / denom;
-        }
-        w = w_new;
-        s1 = z;
-        s2 = n_new;
-    }
-}
-
-// N consecutive elements; the optimizer is chosen once, outside the element loop.
-template <int N>
-__device__ __forceinline__ void opt_step_n(const OptParams& o, const float* g, float* w, float* s1,
-                                           float* s2) {
-    switch (o.kind) {
-        case 0:
-#pragma unroll
-            for (int e = 0; e < N; ++e) opt_step<0>(o, g[e], w[e], s1[e], s2[e]);
-            break;
-        case 1:
-#pragma unroll
-            for (int e = 0; e < N; ++e) opt_step<1>(o, g[e], w[e], s1[e], s2[e]);
-            break;
-        case 2:
-#pragma unroll
-            for (int e = 0; e < N; ++e) opt_step<2>(o, g[e], w[e], s1[e], s2[e]);
-            break;
-        default:
-#pragma unroll
-            for (int e = 0; e < N; ++e) opt_step<3>(o, g[e], w[e], s1[e], s2[e]);
-            break;
-    }
-}
-
-// Applies the aggregated gradient `g` (columns [col, col+1) in units of T) to row `row`.
-template <typename T>
-__device__ __forceinline__ void finalize(const TableDev& t, u32 row, u32 col, u32 units, T g) {
-    constexpr int N = sizeof(T) / 4;
-    if (row >= t.max_rows) return;
-    T* r = reinterpret_cast<T*>(t.rows + (u64)row * t.stride_f);
-    const int kind = t.opt.kind;
-    T wv = r[col];
-    T av = vzero(T()), bv = vzero(T());
-    if (kind >= 2) av = r[units + col];
-    if (kind == 3) bv = r[2 * units + col];
-    float* gp = reinterpret_cast<float*>(&g);
-    float* wp = reinterpret_cast<float*>(&wv);
-    float* ap = reinterpret_cast<float*>(&av);
-    float* bp = reinterpret_cast<float*>(&bv);
-    opt_step_n<N>(t.opt, gp, wp, ap, bp);
-    if (t.dirty && col == 0) t.dirty[row] = 1;
-    r[col] = wv;
-    if (kind >= 2) r[units + col] = av;
-    if (kind == 3) r[2 * units + col] = bv;
 }
 
 // ---- duplicate aggregation + update over row-sorted pairs --------------------------------------

@@ -1,0 +1,1076 @@
+// The partitioned push: duplicate-key aggregation and row update of a large batch without a global
+// sort (the duplicate merge of pico-ps/operator/SparsePushOperator.h:134-141 and the per-item loop
+// of :245-268).
+//
+// The batch is cut into tiles of 4096 keys and the key space into P partitions, a partition being a
+// range of home buckets of the hash array. Five launches:
+//   1. part_tile_kernel     a workgroup per tile: finds the keys that repeat inside the tile (a hash
+//                           table in LDS), adds up their gradient rows into one pre-summed row per
+//                           key, and leaves one entry {key, reference} per distinct key of the tile,
+//                           grouped by partition, in the tile's staging block; a reference is the
+//                           batch index of the gradient row or the number of a pre-summed row.
+//   2. part_scan_kernel     where each (tile, partition) segment goes in the partitioned entry array.
+//   3. part_scatter_kernel  moves the entries there.
+//   4. part_apply_kernel    a workgroup per partition: groups the partition's entries by key (LDS hash
+//                           table again; a key has at most one entry per tile, so the hottest key of
+//                           a batch is a list of a few hundred references, not of a hundred thousand),
+//                           probes the table ONCE per distinct key, adds up each key's rows and takes
+//                           the optimizer step. A key that is not stored claims a slot; its summed
+//                           gradient is parked for the last launch.
+//   5. part_insert_kernel   numbers the new keys densely (prefix over the partitions' counts),
+//                           initialises their rows and takes their step.
+// Sums are accumulated in double precision and rounded to fp32 once per tile and once per key: the
+// result does not depend on the order in which a key's rows are met beyond the last bit of a
+// 53-bit sum.
+#include "table.h"
+#include "probe.h"
+#include "rowops.h"
+
+namespace pshbm {
+
+namespace {
+
+using u16 = uint16_t;
+
+#ifdef PART_EXPERIMENT
+// Build-time option for the developer: phases switched off by bits of a process-wide word, to see
+// what each costs (results are then wrong).
+#define DBG(flags, bit) (((flags) >> (bit)) & 1u)
+#else
+#define DBG(flags, bit) false
+#endif
+
+#ifdef PART_TIMING
+// Build-time option for the developer: time spent per phase of the tile and apply kernels, summed
+// over the workgroups (ticks of the 100 MHz wall clock), read back by pshbm_debug_part_timing.
+__device__ unsigned long long g_part_ticks[2][16];
+#define TICK_INIT long long tick_last = wall_clock64()
+#define TICK(kernel, phase)                                                                  \
+    do {                                                                                      \
+        if (threadIdx.x == 0) {                                                               \
+            const long long now = wall_clock64();                                             \
+            atomicAdd(&g_part_ticks[kernel][phase], (unsigned long long)(now - tick_last));   \
+            tick_last = now;                                                                  \
+        }                                                                                     \
+    } while (0)
+#else
+#define TICK_INIT
+#define TICK(kernel, phase)
+#endif
+
+constexpr u32 PT_TILE = 4096, PT_BLOCK = 1024, PT_ITEMS = PT_TILE / PT_BLOCK;
+constexpr u32 PT_HT = 2 * PT_TILE;            // slots of a tile's LDS hash table
+constexpr u32 PT_MAX_MULTI = PT_TILE / 2;     // pre-summed rows a tile can produce
+constexpr u32 PT_ACC_DOUBLES = PT_TILE;       // accumulators: the room of the tile's key array (32 KiB)
+constexpr u32 REF_PSUM = 0x80000000u;         // reference to a pre-summed row
+constexpr u32 NONE32 = 0xFFFFFFFFu;
+constexpr u32 PA_BLOCK = 512, PA_ITEMS = 4, PA_CAP = PA_BLOCK * PA_ITEMS;  // entries a partition pass holds
+constexpr u32 PA_HT = 2 * PA_CAP;
+constexpr u32 PA_ACC_DOUBLES = PA_HT / 2;     // the room of the partition's hash table (16 KiB)
+constexpr u32 AUX_NEW = 0x80000000u;
+
+// exclusive scan over the NT threads of the block (64-bit packed fields); all threads call it
+template <u32 NT>
+__device__ __forceinline__ u64 block_scan_excl(u64 v, u32 tid, u64* sums, u64* total) {
+    const u32 lane = tid & 63u, w = tid >> 6;
+    u64 incl = v;
+    for (u32 off = 1; off < 64; off <<= 1) {
+        const u64 o = shfl64(incl, (lane >= off) ? lane - off : lane);
+        if (lane >= off) incl += o;
+    }
+    if (lane == 63) sums[w] = incl;
+    __syncthreads();
+    u64 before = 0, all = 0;
+    for (u32 x = 0; x < NT / 64; ++x) {
+        const u64 c = sums[x];
+        if (x < w) before += c;
+        all += c;
+    }
+    *total = all;
+    __syncthreads();
+    return before + incl - v;
+}
+
+// Item q (key lkey[q], hash h) finds the item that stands for its key -- the first one to claim
+// the key's slot of the LDS hash table -- and its arrival number among the items of that key.
+__device__ __forceinline__ void dedupe_insert(u64 key, u32 q, u64 h, const u64* lkey, u32* owner, u32* cnt,
+                                              u32 ht_mask, u32& rep, u32& arrival) {
+    u32 s = (u32)(h >> 40) & ht_mask;
+    while (true) {
+        const u32 old = atomicCAS(&owner[s], NONE32, q);
+        if (old == NONE32) {
+            rep = q;
+            break;
+        }
+        if (lkey[old] == key) {
+            rep = old;
+            break;
+        }
+        s = (s + 1) & ht_mask;
+    }
+    arrival = atomicAdd(&cnt[rep], 1u);
+}
+
+template <typename T>
+struct Acc;
+template <>
+struct Acc<float> {
+    double a;
+    __device__ __forceinline__ void zero() { a = 0.0; }
+    __device__ __forceinline__ void add(float v) { a += (double)v; }
+    __device__ __forceinline__ void flush(double* p) const { atomicAdd(p, a); }
+    __device__ __forceinline__ static float load(const double* p) { return (float)p[0]; }
+};
+template <>
+struct Acc<float4> {
+    double a, b, c, d;
+    __device__ __forceinline__ void zero() { a = b = c = d = 0.0; }
+    __device__ __forceinline__ void add(float4 v) {
+        a += (double)v.x;
+        b += (double)v.y;
+        c += (double)v.z;
+        d += (double)v.w;
+    }
+    __device__ __forceinline__ void flush(double* p) const {
+        atomicAdd(p, a);
+        atomicAdd(p + 1, b);
+        atomicAdd(p + 2, c);
+        atomicAdd(p + 3, d);
+    }
+    __device__ __forceinline__ static float4 load(const double* p) {
+        return make_float4((float)p[0], (float)p[1], (float)p[2], (float)p[3]);
+    }
+};
+
+// Sums of lists of gradient rows, all lists at once: elements [lo, hi) are dealt to the NG lane
+// groups in turn (so a long list is spread over all of them), element e belongs to list lid[e]
+// (ascending in e) and its row is src(e); a group adds consecutive elements of one list in
+// registers and adds the sum to the list's accumulators in LDS when the list changes.
+// acc[((list - list_base) * units + c) * N + x], double, zero on entry.
+template <typename T>
+struct ListSum {
+    Acc<T> a;
+    u32 cur, list_base, units, c;
+    double* acc;
+    __device__ __forceinline__ void begin(double* acc_, u32 list_base_, u32 units_, u32 c_) {
+        acc = acc_;
+        list_base = list_base_;
+        units = units_;
+        c = c_;
+        cur = NONE32;
+        a.zero();
+    }
+    __device__ __forceinline__ void flush() {
+        if (cur != NONE32) a.flush(acc + ((size_t)(cur - list_base) * units + c) * (sizeof(T) / 4));
+    }
+    __device__ __forceinline__ void take(u32 l, T v) {
+        if (l != cur) {
+            flush();
+            cur = l;
+            a.zero();
+        }
+        a.add(v);
+    }
+};
+
+// elements first, first + NG, ... below hi
+template <typename T, typename SRC>
+__device__ __forceinline__ void flat_sum_from(SRC src, const u16* lid, u32 first, u32 hi, u32 NG, u32 c,
+                                              ListSum<T>& ls) {
+    u32 e = first;
+    for (; e + 3 * NG < hi; e += 4 * NG) {  // four rows in flight
+        const u32 l0 = lid[e], l1 = lid[e + NG], l2 = lid[e + 2 * NG], l3 = lid[e + 3 * NG];
+        const T v0 = src(e)[c], v1 = src(e + NG)[c], v2 = src(e + 2 * NG)[c], v3 = src(e + 3 * NG)[c];
+        ls.take(l0, v0);
+        ls.take(l1, v1);
+        ls.take(l2, v2);
+        ls.take(l3, v3);
+    }
+    for (; e < hi; e += NG) ls.take(lid[e], src(e)[c]);
+}
+
+template <typename T, typename SRC>
+__device__ __forceinline__ void flat_sum(SRC src, const u16* lid, u32 lo, u32 hi, u32 list_base, double* acc,
+                                         u32 units, u32 NG, u32 g, u32 c) {
+    ListSum<T> ls;
+    ls.begin(acc, list_base, units, c);
+    flat_sum_from<T>(src, lid, lo + g, hi, NG, c, ls);
+    ls.flush();
+}
+
+__device__ __forceinline__ u32 partition_of(const TableDev& t, u64 h, u32 part_shift) {
+    return ((u32)h & t.bucket_mask) >> part_shift;
+}
+
+// ---- 1. tile kernel ---------------------------------------------------------------------------
+// LDS (dynamic, 128 KiB): keys of the tile (later the accumulators) | hash table (later the list of
+// keys that repeat) | per-item counts | per-item aux | list of repeating items + their list numbers |
+// partition histogram.
+constexpr u32 PT_OFF_OWNER = PT_TILE * 8;
+constexpr u32 PT_OFF_CNT = PT_OFF_OWNER + PT_HT * 4;
+constexpr u32 PT_OFF_AUX = PT_OFF_CNT + PT_TILE * 4;
+constexpr u32 PT_OFF_LIST = PT_OFF_AUX + PT_TILE * 4;
+constexpr u32 PT_OFF_LOWN = PT_OFF_LIST + PT_TILE * 2;
+constexpr u32 PT_OFF_HIST = PT_OFF_LOWN + PT_TILE * 2;
+constexpr u32 PT_MAX_PARTS = 4096;
+constexpr u32 PT_LDS = PT_OFF_HIST + PT_MAX_PARTS * 4;  // 131072
+
+template <typename T>
+__global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
+    TableDev t, const u64* __restrict__ keys, const T* __restrict__ grads, u32 n, u32 P, u32 part_shift,
+    u64* __restrict__ stage_key, u32* __restrict__ stage_ref, u32* __restrict__ counts, u32* __restrict__ starts,
+    u32* __restrict__ blocktot, u32* __restrict__ tile_total, T* __restrict__ psum, u32 units, u32 dbg) {
+    extern __shared__ __align__(16) unsigned char pt_lds[];
+    u64* lkey = reinterpret_cast<u64*>(pt_lds);
+    u32* owner = reinterpret_cast<u32*>(pt_lds + PT_OFF_OWNER);
+    u32* cnt = reinterpret_cast<u32*>(pt_lds + PT_OFF_CNT);
+    u32* aux = reinterpret_cast<u32*>(pt_lds + PT_OFF_AUX);
+    u16* list = reinterpret_cast<u16*>(pt_lds + PT_OFF_LIST);
+    u16* lown = reinterpret_cast<u16*>(pt_lds + PT_OFF_LOWN);
+    u32* hist = reinterpret_cast<u32*>(pt_lds + PT_OFF_HIST);
+    __shared__ u64 sums[PT_BLOCK / 64];
+    constexpr u32 N = sizeof(T) / 4;
+    const u32 tid = threadIdx.x;
+    const u32 tile = blockIdx.x;
+    const u64 tb = (u64)tile * PT_TILE;
+    TICK_INIT;
+
+    u64 key[PT_ITEMS], hh[PT_ITEMS];
+    bool valid[PT_ITEMS];
+    u32 nbad = 0;
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j) {
+        const u32 q = j * PT_BLOCK + tid;
+        const u64 i = tb + q;
+        key[j] = i < n ? keys[i] : KEY_EMPTY;
+        valid[j] = i < n && key[j] < KEY_DELETED;
+        nbad += (i < n && !valid[j]) ? 1u : 0u;
+        lkey[q] = key[j];
+        cnt[q] = 0;
+        hh[j] = hash64(key[j]);
+    }
+#pragma unroll
+    for (u32 x = 0; x < PT_HT / PT_BLOCK; ++x) owner[x * PT_BLOCK + tid] = NONE32;
+    for (u32 x = tid; x < P; x += PT_BLOCK) hist[x] = 0;
+    if (nbad) atomicAdd(&t.counters[CNT_BADKEY], nbad);  // reserved keys are skipped (and rare)
+    __syncthreads();
+    TICK(0, 0);
+
+    // the items of one key agree on a representative and number themselves
+    u32 rep[PT_ITEMS], arr[PT_ITEMS];
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j) {
+        rep[j] = arr[j] = 0;
+        if (valid[j]) dedupe_insert(key[j], j * PT_BLOCK + tid, hh[j], lkey, owner, cnt, PT_HT - 1, rep[j], arr[j]);
+    }
+    __syncthreads();
+    TICK(0, 1);
+
+    // keys that repeat: a number each (in thread order) and a range of the item list
+    u32 m[PT_ITEMS];
+    bool isrep[PT_ITEMS], multi[PT_ITEMS];
+    u32 my_multi = 0, my_len = 0;
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j) {
+        m[j] = valid[j] ? cnt[rep[j]] : 0u;
+        isrep[j] = valid[j] && rep[j] == j * PT_BLOCK + tid;
+        multi[j] = isrep[j] && m[j] >= 2;
+        my_multi += multi[j] ? 1u : 0u;
+        my_len += multi[j] ? m[j] : 0u;
+    }
+    u64 tot = 0;
+    const u64 ex = block_scan_excl<PT_BLOCK>(((u64)my_len << 32) | my_multi, tid, sums, &tot);
+    const u32 n_multi = (u32)tot, n_elems = (u32)(tot >> 32);
+    u32* mrep = owner;  // the hash table is done with
+    {
+        u32 mr = (u32)ex, lo = (u32)(ex >> 32);
+#pragma unroll
+        for (u32 j = 0; j < PT_ITEMS; ++j)
+            if (multi[j]) {
+                aux[j * PT_BLOCK + tid] = lo | (mr << 16);
+                mrep[mr] = j * PT_BLOCK + tid;
+                ++mr;
+                lo += m[j];
+            }
+    }
+    __syncthreads();
+    TICK(0, 2);
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j)
+        if (valid[j] && m[j] >= 2) {
+            const u32 a = aux[rep[j]];
+            list[(a & 0xFFFFu) + arr[j]] = (u16)(j * PT_BLOCK + tid);
+            lown[(a & 0xFFFFu) + arr[j]] = (u16)(a >> 16);
+        }
+
+    // one entry per distinct key, grouped by partition in the tile's staging block
+    u32 prank[PT_ITEMS], part[PT_ITEMS];
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j) {
+        part[j] = partition_of(t, hh[j], part_shift);
+        prank[j] = isrep[j] ? atomicAdd(&hist[part[j]], 1u) : 0u;
+    }
+    __syncthreads();
+    TICK(0, 3);
+
+    // Pre-summed rows of the keys that repeat, as many lists per round as the accumulators hold
+    // (the room of the key array, which nobody reads any more). The rows of the first round are
+    // requested now and added up after the staging block is written: their latency covers that.
+    double* acc = reinterpret_cast<double*>(pt_lds);
+    const u32 G = units;  // lanes per row (the host admits units <= PT_BLOCK)
+    const u32 NG = PT_BLOCK / G;
+    const u32 g = tid / G, c = tid - g * G;
+    const bool on = g < NG;
+    const u32 B = PT_ACC_DOUBLES / (units * N);  // lists per round, at least 1
+    const T* tile_grads = grads + tb * units;
+    constexpr u32 PF = 4;
+    T pv[PF];
+    u32 pl[PF];
+    const u32 first_b1 = B < n_multi ? B : n_multi;
+    const u32 first_hi = first_b1 < n_multi ? (aux[mrep[first_b1]] & 0xFFFFu) : n_elems;
+    for (u32 x = tid; x < first_b1 * units * N; x += PT_BLOCK) acc[x] = 0.0;
+#pragma unroll
+    for (u32 k = 0; k < PF; ++k) {
+        const u32 e = g + k * NG;
+        const bool ok = on && e < first_hi;
+        pl[k] = ok ? (u32)lown[e] : NONE32;
+        pv[k] = vzero(T());
+        if (ok && !DBG(dbg, 1)) pv[k] = tile_grads[(size_t)list[e] * units + c];
+    }
+    {
+        // thread x owns PP consecutive partitions (P is a power of two, at least 64): their counts,
+        // where their entries start in the staging block, and the count of each block of 64
+        const u32 PP = P > PT_BLOCK ? P / PT_BLOCK : 1u;
+        u32 cc[PT_MAX_PARTS / PT_BLOCK];
+        u32 local = 0;
+#pragma unroll
+        for (u32 x = 0; x < PT_MAX_PARTS / PT_BLOCK; ++x) {
+            const u32 p = tid * PP + x;
+            cc[x] = (x < PP && p < P) ? hist[p] : 0u;
+            local += cc[x];
+        }
+        u64 all = 0;
+        u32 run = (u32)block_scan_excl<PT_BLOCK>(local, tid, sums, &all);
+        if (tid == 0) tile_total[tile] = (u32)all;
+        u32 blk = local;
+        for (u32 off = 1; off < 64u / PP; off <<= 1) blk += __shfl_xor(blk, (int)off);
+        if ((tid & (64u / PP - 1u)) == 0 && tid * PP < P) blocktot[(size_t)tile * (P / 64u) + tid * PP / 64u] = blk;
+#pragma unroll
+        for (u32 x = 0; x < PT_MAX_PARTS / PT_BLOCK; ++x) {
+            const u32 p = tid * PP + x;
+            if (x < PP && p < P) {
+                hist[p] = run;
+                counts[(size_t)tile * P + p] = cc[x];
+                starts[(size_t)tile * P + p] = run;
+                run += cc[x];
+            }
+        }
+    }
+    __syncthreads();
+    TICK(0, 4);
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j)
+        if (isrep[j]) {
+            const u64 pos = tb + hist[part[j]] + prank[j];
+            stage_key[pos] = key[j];
+            stage_ref[pos] = multi[j] ? (REF_PSUM | (tile * PT_MAX_MULTI + (aux[j * PT_BLOCK + tid] >> 16)))
+                                      : (u32)(tb + j * PT_BLOCK + tid);
+        }
+    if (n_multi == 0 || DBG(dbg, 0)) return;  // block-uniform
+    TICK(0, 5);
+
+    for (u32 b0 = 0; b0 < n_multi; b0 += B) {
+        const u32 b1 = b0 + B < n_multi ? b0 + B : n_multi;
+        const u32 lo = aux[mrep[b0]] & 0xFFFFu;
+        const u32 hi = b1 < n_multi ? (aux[mrep[b1]] & 0xFFFFu) : n_elems;
+        auto row_of = [&](u32 e) { return tile_grads + (size_t)list[e] * units; };
+        if (b0 == 0) {  // the accumulators are zero (barriers since) and the first rows are here
+            if (on) {
+                ListSum<T> ls;
+                ls.begin(acc, 0u, units, c);
+#pragma unroll
+                for (u32 k = 0; k < PF; ++k)
+                    if (pl[k] != NONE32) ls.take(pl[k], pv[k]);
+                flat_sum_from<T>(row_of, lown, g + PF * NG, hi, NG, c, ls);
+                ls.flush();
+            }
+        } else {
+            for (u32 x = tid; x < (b1 - b0) * units * N; x += PT_BLOCK) acc[x] = 0.0;
+            __syncthreads();
+            if (on) flat_sum<T>(row_of, lown, lo, hi, b0, acc, units, NG, g, c);
+        }
+        __syncthreads();
+        TICK(0, 7);
+        if (on)
+            for (u32 l = b0 + g; l < b1; l += NG)
+                psum[((size_t)tile * PT_MAX_MULTI + l) * units + c] =
+                    Acc<T>::load(acc + ((size_t)(l - b0) * units + c) * N);
+        __syncthreads();
+        TICK(0, 8);
+    }
+}
+
+// ---- 2. scan ------------------------------------------------------------------------------------
+// counts[tile][p] becomes delta[tile][p] = (position of the tile's first entry of partition p in the
+// partitioned array) - starts[tile][p], so that entry j of the tile's staging block goes to
+// delta + j; pstart[p] = first entry of partition p. A workgroup owns a block of 64 partitions
+// (lane = partition) over all tiles, which its 16 wavefronts split into consecutive parts; what the
+// lower blocks hold it adds up from the per-tile block counts the tile kernel left (no atomic
+// additions anywhere: additions to one address from all over the device are resolved one by one).
+__global__ __launch_bounds__(PT_BLOCK) void part_scan_kernel(u32* __restrict__ counts, const u32* __restrict__ starts,
+                                                              const u32* __restrict__ blocktot,
+                                                              u32* __restrict__ pstart, u32 n_tiles, u32 P) {
+    __shared__ u32 red[PT_BLOCK / 64];
+    __shared__ u32 colbase[64];
+    __shared__ u32 part_sum[PT_BLOCK / 64][64];
+    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const u32 blk = blockIdx.x, d0 = blk * 64u, NB = P / 64u;
+    // entries of the lower blocks, over all tiles
+    u32 before = 0;
+    for (u32 t0 = tid / 64u; t0 < n_tiles; t0 += PT_BLOCK / 64u)
+        for (u32 x = lane; x < blk; x += 64u) before += blocktot[(size_t)t0 * NB + x];
+    for (u32 off = 32; off >= 1; off >>= 1) before += __shfl_down(before, off);
+    if (lane == 0) red[w] = before;
+    const u32 per = (n_tiles + PT_BLOCK / 64 - 1) / (PT_BLOCK / 64);
+    const u32 t0 = w * per < n_tiles ? w * per : n_tiles;
+    const u32 t1 = t0 + per < n_tiles ? t0 + per : n_tiles;
+    u32* col = counts + d0 + lane;
+    const u32* scol = starts + d0 + lane;
+    u32 s = 0;
+    {
+        u32 tt = t0;
+        for (; tt + 8 <= t1; tt += 8) {
+            u32 v[8];
+#pragma unroll
+            for (u32 x = 0; x < 8; ++x) v[x] = col[(size_t)(tt + x) * P];
+#pragma unroll
+            for (u32 x = 0; x < 8; ++x) s += v[x];
+        }
+        for (; tt < t1; ++tt) s += col[(size_t)tt * P];
+    }
+    part_sum[w][lane] = s;
+    __syncthreads();
+    if (w == 0) {  // this block's partitions: totals, their exclusive prefix over the lanes
+        u32 base = 0;
+        for (u32 x = 0; x < PT_BLOCK / 64; ++x) base += red[x];
+        u32 tot = 0;
+        for (u32 x = 0; x < PT_BLOCK / 64; ++x) tot += part_sum[x][lane];
+        u32 incl = tot;
+        for (u32 off = 1; off < 64; off <<= 1) {
+            const u32 o = __shfl_up(incl, off);
+            if (lane >= off) incl += o;
+        }
+        colbase[lane] = base + incl - tot;
+        pstart[d0 + lane] = base + incl - tot;
+        if (blk + 1 == NB && lane == 63) pstart[P] = base + incl;
+    }
+    __syncthreads();
+    u32 pos = colbase[lane];
+    for (u32 x = 0; x < w; ++x) pos += part_sum[x][lane];
+    {
+        u32 tt = t0;
+        for (; tt + 8 <= t1; tt += 8) {
+            u32 v[8], st[8];
+#pragma unroll
+            for (u32 x = 0; x < 8; ++x) {
+                v[x] = col[(size_t)(tt + x) * P];
+                st[x] = scol[(size_t)(tt + x) * P];
+            }
+#pragma unroll
+            for (u32 x = 0; x < 8; ++x) {
+                col[(size_t)(tt + x) * P] = pos - st[x];
+                pos += v[x];
+            }
+        }
+        for (; tt < t1; ++tt) {
+            const u32 v = col[(size_t)tt * P];
+            col[(size_t)tt * P] = pos - scol[(size_t)tt * P];
+            pos += v;
+        }
+    }
+}
+
+// ---- 3. scatter -----------------------------------------------------------------------------------
+__global__ __launch_bounds__(PT_BLOCK) void part_scatter_kernel(TableDev t, const u64* __restrict__ stage_key,
+                                                                 const u32* __restrict__ stage_ref,
+                                                                 const u32* __restrict__ delta,
+                                                                 const u32* __restrict__ tile_total, u32 P,
+                                                                 u32 part_shift, u64* __restrict__ ent_key,
+                                                                 u32* __restrict__ ent_ref) {
+    const u32 tile = blockIdx.x, tid = threadIdx.x;
+    const u64 tb = (u64)tile * PT_TILE;
+    const u32 cnt = tile_total[tile];
+    u64 key[PT_ITEMS];
+    u32 ref[PT_ITEMS];
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j) {
+        const u32 q = j * PT_BLOCK + tid;
+        key[j] = q < cnt ? stage_key[tb + q] : KEY_EMPTY;
+        ref[j] = q < cnt ? stage_ref[tb + q] : 0u;
+    }
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j) {
+        const u32 q = j * PT_BLOCK + tid;
+        if (q >= cnt) continue;
+        const u32 p = partition_of(t, hash64(key[j]), part_shift);
+        const u32 pos = delta[(size_t)tile * P + p] + q;
+        ent_key[pos] = key[j];
+        ent_ref[pos] = ref[j];
+    }
+}
+
+// ---- 4. apply -------------------------------------------------------------------------------------
+// LDS (dynamic, 72 KiB): entry keys | hash table (later the accumulators) | counts | aux |
+// entry references (later the rows of the distinct keys) | references grouped by key | list numbers |
+// distinct keys | keys with more than one entry.
+constexpr u32 PA_OFF_OWNER = PA_CAP * 8;
+constexpr u32 PA_OFF_CNT = PA_OFF_OWNER + PA_HT * 4;
+constexpr u32 PA_OFF_AUX = PA_OFF_CNT + PA_CAP * 4;
+constexpr u32 PA_OFF_LREF = PA_OFF_AUX + PA_CAP * 4;
+constexpr u32 PA_OFF_LIST = PA_OFF_LREF + PA_CAP * 4;
+constexpr u32 PA_OFF_LOWN = PA_OFF_LIST + PA_CAP * 4;
+constexpr u32 PA_OFF_UREP = PA_OFF_LOWN + PA_CAP * 2;
+constexpr u32 PA_OFF_MREP = PA_OFF_UREP + PA_CAP * 2;
+constexpr u32 PA_LDS = PA_OFF_MREP + PA_CAP * 2;  // 75776
+
+struct ApplyArgs {
+    const u64* ent_key;
+    const u32* ent_ref;
+    const u32* pstart;
+    u32* new_slot;
+    u32* new_count;
+    u32 units;
+    int insert;
+    u32 cap;  // entries a pass holds: PA_CAP, or less when a test wants to see the passes
+    u32 dbg;
+};
+
+// The keys of a pass that have one entry: their gradient row is their sum. Lane group g takes keys
+// g, g + NG, ..., KS of them at a time, so that the loads of KS gradient rows and KS table rows are
+// in flight together.
+template <typename T, int KIND, u32 KS>
+__device__ __forceinline__ void apply_singles(const TableDev& t, unsigned char* lds, const T* __restrict__ grads,
+                                              const T* __restrict__ psum, T* __restrict__ ngrad, u32 s, u32 U,
+                                              u32 units, u32 NG, u32 g, u32 c) {
+    constexpr u32 N = sizeof(T) / 4;
+    constexpr int STATES = KIND <= 1 ? 0 : KIND - 1;
+    const u32* cnt = reinterpret_cast<const u32*>(lds + PA_OFF_CNT);
+    const u32* aux = reinterpret_cast<const u32*>(lds + PA_OFF_AUX);
+    const u32* urow = reinterpret_cast<const u32*>(lds + PA_OFF_LREF);
+    const u32* list = reinterpret_cast<const u32*>(lds + PA_OFF_LIST);
+    const u16* urep = reinterpret_cast<const u16*>(lds + PA_OFF_UREP);
+    T* rows = reinterpret_cast<T*>(t.rows);
+    const u32 stride_units = t.stride_f / N;
+    for (u32 u0 = g; u0 < U; u0 += KS * NG) {
+        u32 rowk[KS], dst[KS];
+        bool single[KS], isnew[KS];
+        T gv[KS], wv[KS], av[STATES >= 1 ? KS : 1], bv[STATES >= 2 ? KS : 1];
+#pragma unroll
+        for (u32 k = 0; k < KS; ++k) {
+            const u32 u = u0 + k * NG;
+            single[k] = false;
+            isnew[k] = false;
+            rowk[k] = ROW_NONE;
+            dst[k] = 0;
+            gv[k] = vzero(T());
+            if (u < U) {
+                const u32 i = urep[u];
+                if (cnt[i] == 1) {
+                    single[k] = true;
+                    const u32 av_ = aux[i];
+                    isnew[k] = (av_ & AUX_NEW) != 0;
+                    const u32 ref = list[av_ & 0xFFFFu];
+                    gv[k] = ((ref & REF_PSUM) ? psum + (size_t)(ref & ~REF_PSUM) * units : grads + (size_t)ref * units)[c];
+                    dst[k] = urow[u];
+                    if (!isnew[k] && dst[k] < t.max_rows) rowk[k] = dst[k];
+                }
+            }
+        }
+#pragma unroll
+        for (u32 k = 0; k < KS; ++k) {
+            wv[k] = vzero(T());
+            if (rowk[k] != ROW_NONE) {
+                const T* r = rows + (size_t)rowk[k] * stride_units + c;
+                wv[k] = r[0];
+                if constexpr (STATES >= 1) av[k] = r[units];
+                if constexpr (STATES >= 2) bv[k] = r[2 * units];
+            }
+        }
+#pragma unroll
+        for (u32 k = 0; k < KS; ++k) {
+            if (!single[k]) continue;
+            if (isnew[k]) {
+                ngrad[(size_t)(s + dst[k]) * units + c] = gv[k];
+            } else if (rowk[k] != ROW_NONE) {
+                T a0 = vzero(T()), b0 = vzero(T());
+                if constexpr (STATES >= 1) a0 = av[k];
+                if constexpr (STATES >= 2) b0 = bv[k];
+                float* gp = reinterpret_cast<float*>(&gv[k]);
+                float* wp = reinterpret_cast<float*>(&wv[k]);
+                float* ap = reinterpret_cast<float*>(&a0);
+                float* bp = reinterpret_cast<float*>(&b0);
+#pragma unroll
+                for (u32 e = 0; e < N; ++e) opt_step<KIND>(t.opt, gp[e], wp[e], ap[e], bp[e]);
+                T* r = rows + (size_t)rowk[k] * stride_units + c;
+                if (t.dirty && c == 0) t.dirty[rowk[k]] = 1;
+                r[0] = wv[k];
+                if constexpr (STATES >= 1) r[units] = a0;
+                if constexpr (STATES >= 2) r[2 * units] = b0;
+            }
+        }
+    }
+}
+
+// Everything a pass does with the `count` entries that lie in lkey / lref.
+template <typename T>
+__device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds, u64* sums, u32* s_nnew,
+                                           const T* __restrict__ grads, const T* __restrict__ psum,
+                                           T* __restrict__ ngrad, const ApplyArgs& a, u32 s, u32 count) {
+    constexpr u32 N = sizeof(T) / 4;
+    u64* lkey = reinterpret_cast<u64*>(lds);
+    u32* owner = reinterpret_cast<u32*>(lds + PA_OFF_OWNER);
+    u32* cnt = reinterpret_cast<u32*>(lds + PA_OFF_CNT);
+    u32* aux = reinterpret_cast<u32*>(lds + PA_OFF_AUX);
+    u32* lref = reinterpret_cast<u32*>(lds + PA_OFF_LREF);
+    u32* list = reinterpret_cast<u32*>(lds + PA_OFF_LIST);
+    u16* lown = reinterpret_cast<u16*>(lds + PA_OFF_LOWN);
+    u16* urep = reinterpret_cast<u16*>(lds + PA_OFF_UREP);
+    u16* mrep = reinterpret_cast<u16*>(lds + PA_OFF_MREP);
+    const u32 tid = threadIdx.x, lane = tid & 63u;
+    const u32 units = a.units;
+    TICK_INIT;
+
+#pragma unroll
+    for (u32 x = 0; x < PA_HT / PA_BLOCK; ++x) owner[x * PA_BLOCK + tid] = NONE32;
+#pragma unroll
+    for (u32 j = 0; j < PA_ITEMS; ++j) cnt[j * PA_BLOCK + tid] = 0;
+    __syncthreads();
+    TICK(1, 0);
+
+    u32 rep[PA_ITEMS], arr[PA_ITEMS];
+    bool valid[PA_ITEMS];
+#pragma unroll
+    for (u32 j = 0; j < PA_ITEMS; ++j) {
+        const u32 i = j * PA_BLOCK + tid;
+        valid[j] = i < count;
+        rep[j] = arr[j] = 0;
+        if (valid[j]) {
+            const u64 key = lkey[i];
+            dedupe_insert(key, i, hash64(key), lkey, owner, cnt, PA_HT - 1, rep[j], arr[j]);
+        }
+    }
+    __syncthreads();
+    TICK(1, 1);
+
+    // distinct keys numbered; the references of the keys with several entries come first in the list
+    u32 m[PA_ITEMS];
+    bool isrep[PA_ITEMS];
+    u32 my_u = 0, my_multi = 0, my_len = 0;
+#pragma unroll
+    for (u32 j = 0; j < PA_ITEMS; ++j) {
+        m[j] = valid[j] ? cnt[rep[j]] : 0u;
+        isrep[j] = valid[j] && rep[j] == j * PA_BLOCK + tid;
+        my_u += isrep[j] ? 1u : 0u;
+        my_multi += (isrep[j] && m[j] >= 2) ? 1u : 0u;
+        my_len += (isrep[j] && m[j] >= 2) ? m[j] : 0u;
+    }
+    u64 tot = 0;
+    const u64 ex = block_scan_excl<PA_BLOCK>((u64)my_u | ((u64)my_multi << 16) | ((u64)my_len << 32), tid, sums, &tot);
+    const u32 U = (u32)(tot & 0xFFFFu), n_multi = (u32)((tot >> 16) & 0xFFFFu), n_elems = (u32)(tot >> 32);
+    {
+        u32 ur = (u32)(ex & 0xFFFFu), mr = (u32)((ex >> 16) & 0xFFFFu), lo = (u32)(ex >> 32);
+#pragma unroll
+        for (u32 j = 0; j < PA_ITEMS; ++j)
+            if (isrep[j]) {
+                const u32 i = j * PA_BLOCK + tid;
+                urep[ur] = (u16)i;
+                if (m[j] >= 2) {
+                    aux[i] = lo | (mr << 16);
+                    mrep[mr] = (u16)ur;  // the key's number among the distinct keys
+                    ++mr;
+                    lo += m[j];
+                } else {
+                    aux[i] = n_elems + (ur - mr);  // single entries follow the lists
+                }
+                ++ur;
+            }
+    }
+    __syncthreads();
+    TICK(1, 2);
+#pragma unroll
+    for (u32 j = 0; j < PA_ITEMS; ++j)
+        if (valid[j]) {
+            const u32 av = aux[rep[j]];
+            const u32 pos = (av & 0xFFFFu) + arr[j];
+            list[pos] = lref[j * PA_BLOCK + tid];
+            lown[pos] = (u16)(av >> 16);
+        }
+    __syncthreads();
+    TICK(1, 3);
+
+    // One probe per distinct key, four lanes each. A lane group looks at the home buckets of
+    // several keys at once (all the loads in flight together); a key that is not in its home
+    // bucket -- or must claim a slot -- then takes the ordinary walk.
+    u32* urow = lref;
+    const u32 grp = lane >> 2, sub = lane & 3u;
+    constexpr u32 KP = 4, QUADS = PA_BLOCK / 4;
+    if (DBG(a.dbg, 0))
+        for (u32 u = tid; u < U; u += PA_BLOCK) urow[u] = ROW_NONE;
+    for (u32 u0 = 0; u0 < U && !DBG(a.dbg, 0); u0 += QUADS * KP) {
+        u32 uu[KP], ii[KP];
+        u64 kk[KP];
+        bool act[KP];
+        uint4 sv[KP];
+#pragma unroll
+        for (u32 k = 0; k < KP; ++k) {
+            uu[k] = u0 + k * QUADS + (tid >> 2);
+            act[k] = uu[k] < U;
+            ii[k] = act[k] ? urep[uu[k]] : 0u;
+            kk[k] = act[k] ? lkey[ii[k]] : KEY_EMPTY;
+            sv[k] = make_uint4(0u, 0u, 0u, 0u);
+            if (act[k]) sv[k] = t.slots[(u64)((u32)hash64(kk[k]) & t.bucket_mask) * 4 + sub];
+        }
+#pragma unroll
+        for (u32 k = 0; k < KP; ++k) {
+            const u64 skey = ((u64)sv[k].y << 32) | sv[k].x;
+            const bool match = act[k] && skey == kk[k];
+            const bool empty = act[k] && skey == KEY_EMPTY;
+            const u32 m4 = (u32)(__ballot(match) >> (grp * 4)) & 0xFu;
+            const u32 e4 = (u32)(__ballot(empty) >> (grp * 4)) & 0xFu;
+            const u32 srcl = grp * 4 + (m4 ? (u32)__ffs((int)m4) - 1u : 0u);
+            const u32 hrow = __shfl(sv[k].z, (int)srcl);
+            // found at home: done. Absent for sure (an empty slot at home) and nothing to insert: done.
+            const bool slow = act[k] && !m4 && (a.insert || !e4);
+            if (act[k] && sub == 0 && !slow) urow[uu[k]] = (m4 && hrow < t.max_rows) ? hrow : ROW_NONE;
+            if (__ballot(slow)) {
+                u32 row = ROW_NONE, slot = SLOT_NONE;
+                bool won = false;
+                if (a.insert) {
+                    const Located l = find_or_claim(t, kk[k], slow, grp, sub, true);
+                    row = l.row;
+                    slot = l.slot;
+                    won = l.won;
+                } else {
+                    const Found f = probe_find(t, kk[k], slow, grp, sub);
+                    row = f.row;
+                }
+                if (slow && sub == 0) {
+                    if (won) {
+                        const u32 kn = atomicAdd(s_nnew, 1u);
+                        a.new_slot[s + kn] = slot;
+                        urow[uu[k]] = kn;
+                        aux[ii[k]] |= AUX_NEW;
+                    } else {
+                        urow[uu[k]] = row < t.max_rows ? row : ROW_NONE;
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    TICK(1, 4);
+
+    const u32 G = units;  // the host admits units <= PA_BLOCK
+    const u32 NG = PA_BLOCK / G;
+    const u32 g = tid / G, c = tid - g * G;
+    const bool on = g < NG;
+    auto src = [&](u32 ref) -> const T* {
+        return (ref & REF_PSUM) ? psum + (size_t)(ref & ~REF_PSUM) * units : grads + (size_t)ref * units;
+    };
+    auto apply = [&](u32 u, u32 i, T gv) {
+        if (aux[i] & AUX_NEW) {
+            ngrad[(size_t)(s + urow[u]) * units + c] = gv;
+        } else {
+            const u32 row = urow[u];
+            if (row != ROW_NONE) finalize<T>(t, row, c, units, gv);
+        }
+    };
+    // keys with one entry: the gradient row is the sum; several keys per lane group in flight
+    if (on && !DBG(a.dbg, 1)) {
+        switch (t.opt.kind) {
+            case 0: apply_singles<T, 0, 4>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c); break;
+            case 1: apply_singles<T, 1, 4>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c); break;
+            case 2: apply_singles<T, 2, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c); break;
+            default: apply_singles<T, 3, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c); break;
+        }
+    }
+    TICK(1, 5);
+    if (n_multi == 0 || DBG(a.dbg, 2)) return;  // block-uniform
+    // keys with several entries: sums in LDS accumulators, as many keys at a time as they hold
+    double* acc = reinterpret_cast<double*>(owner);
+    const u32 B = PA_ACC_DOUBLES / (units * N);
+    for (u32 b0 = 0; b0 < n_multi; b0 += B) {
+        const u32 b1 = b0 + B < n_multi ? b0 + B : n_multi;
+        const u32 lo = aux[urep[mrep[b0]]] & 0xFFFFu;
+        const u32 hi = b1 < n_multi ? (aux[urep[mrep[b1]]] & 0xFFFFu) : n_elems;
+        for (u32 x = tid; x < (b1 - b0) * units * N; x += PA_BLOCK) acc[x] = 0.0;
+        __syncthreads();
+        TICK(1, 6);
+        if (on) flat_sum<T>([&](u32 e) { return src(list[e]); }, lown, lo, hi, b0, acc, units, NG, g, c);
+        __syncthreads();
+        TICK(1, 7);
+        if (on)
+            for (u32 l = b0 + g; l < b1; l += NG) {
+                const u32 u = mrep[l];
+                apply(u, urep[u], Acc<T>::load(acc + ((size_t)(l - b0) * units + c) * N));
+            }
+        __syncthreads();
+        TICK(1, 8);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, const T* __restrict__ grads,
+                                                               const T* __restrict__ psum, T* __restrict__ ngrad,
+                                                               ApplyArgs a) {
+    extern __shared__ __align__(16) unsigned char pa_lds[];
+    __shared__ u64 sums[PA_BLOCK / 64];
+    __shared__ u32 s_nnew, s_sel;
+    u64* lkey = reinterpret_cast<u64*>(pa_lds);
+    u32* lref = reinterpret_cast<u32*>(pa_lds + PA_OFF_LREF);
+    const u32 tid = threadIdx.x;
+    const u32 p = blockIdx.x;
+    const u32 s = a.pstart[p], np = a.pstart[p + 1] - s;
+    // the row count as it is when this operation begins (this launch hands out no rows)
+    if (p == 0 && tid == 0) t.counters[CNT_ENTRY] = t.counters[CNT_ROWS];
+    if (tid == 0) s_nnew = 0;
+    if (np == 0) {
+        if (tid == 0) a.new_count[p] = 0;
+        return;
+    }
+    if (np <= a.cap) {
+        for (u32 i = tid; i < np; i += PA_BLOCK) {
+            lkey[i] = a.ent_key[s + i];
+            lref[i] = a.ent_ref[s + i];
+        }
+        __syncthreads();
+        apply_pass<T>(t, pa_lds, sums, &s_nnew, grads, psum, ngrad, a, s, np);
+    } else {
+        // More entries than a pass holds (several keys that are met in most tiles share the
+        // partition): passes over the entries, pass r taking the keys whose hash says r.
+        u32 R = 2;
+        while (np / R > a.cap / 2 && R < 1024u) R <<= 1;
+        for (u32 r = 0; r < R; ++r) {
+            __syncthreads();
+            if (tid == 0) s_sel = 0;
+            __syncthreads();
+            for (u32 i = tid; i < np; i += PA_BLOCK) {
+                const u64 key = a.ent_key[s + i];
+                if (((u32)(hash64(key) >> 53) & (R - 1u)) == r) {
+                    const u32 pos = atomicAdd(&s_sel, 1u);
+                    if (pos < a.cap) {
+                        lkey[pos] = key;
+                        lref[pos] = a.ent_ref[s + i];
+                    }
+                }
+            }
+            __syncthreads();
+            const u32 sel = s_sel;
+            if (sel > a.cap) {  // not expected of any hash that spreads keys; reported, never silent
+                if (tid == 0) t.counters[CNT_PART_ERR] = 1u;
+                continue;
+            }
+            if (sel) apply_pass<T>(t, pa_lds, sums, &s_nnew, grads, psum, ngrad, a, s, sel);
+        }
+    }
+    __syncthreads();
+    if (tid == 0) a.new_count[p] = s_nnew;
+}
+
+// ---- 5. insert ------------------------------------------------------------------------------------
+constexpr u32 PI_BLOCK = 256;
+
+template <typename T>
+__global__ __launch_bounds__(PI_BLOCK) void part_insert_kernel(TableDev t, const u32* __restrict__ new_slot,
+                                                                const T* __restrict__ ngrad,
+                                                                const u32* __restrict__ new_count,
+                                                                const u32* __restrict__ pstart, u32 P, u32 units) {
+    constexpr u32 N = sizeof(T) / 4;
+    __shared__ u32 red[PI_BLOCK / 64];
+    const u32 p = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const u32 mine = new_count[p];
+    if (mine == 0 && p != 0) return;  // block-uniform
+    const u32 upto = p == 0 ? P : p;
+    u32 part = 0;
+    for (u32 x = tid; x < upto; x += PI_BLOCK) part += new_count[x];
+    for (u32 off = 32; off >= 1; off >>= 1) part += __shfl_down(part, off);
+    if (lane == 0) red[w] = part;
+    __syncthreads();
+    u32 sum = 0;
+    for (u32 x = 0; x < PI_BLOCK / 64; ++x) sum += red[x];
+    const u32 entry = t.counters[CNT_ENTRY];
+    if (p == 0) {
+        if (tid == 0) {
+            t.counters[CNT_ROWS] = entry + sum;
+            if (entry + sum > t.max_rows) t.counters[CNT_OVERFLOW] = 1u;
+            publish_rows(t, entry + sum);
+        }
+        if (mine == 0) return;
+        sum = 0;
+    }
+    const u32 first_row = entry + sum;
+    const u32 s = pstart[p];
+    const u32 G = units < PI_BLOCK ? units : PI_BLOCK;
+    const u32 NG = PI_BLOCK / G;
+    const u32 g = tid / G, c0 = tid - g * G;
+    if (g >= NG) return;
+    const u32 dim = t.dim;
+    for (u32 k = g; k < mine; k += NG) {
+        const u32 slot = new_slot[s + k];
+        const u32 row = first_row + k;
+        if (row >= t.max_rows) continue;  // does not fit (the host rules this out before it takes this path)
+        const uint4 sv = t.slots[slot];
+        const u64 key = ((u64)sv.y << 32) | sv.x;
+        if (c0 == 0) {
+            reinterpret_cast<u32*>(&t.slots[slot])[2] = row;
+            t.row_keys[row] = key;
+            if (t.dirty) t.dirty[row] = 1;
+        }
+        T* r = reinterpret_cast<T*>(t.rows + (size_t)row * t.stride_f);
+        for (u32 c = c0; c < units; c += G) {
+            T gv = ngrad[(size_t)(s + k) * units + c];
+            T wv, av = vzero(T()), bv = vzero(T());
+            float* gp = reinterpret_cast<float*>(&gv);
+            float* wp = reinterpret_cast<float*>(&wv);
+            float* ap = reinterpret_cast<float*>(&av);
+            float* bp = reinterpret_cast<float*>(&bv);
+#pragma unroll
+            for (u32 x = 0; x < N; ++x) {
+                wp[x] = init_float(t, key, c * N + x);
+                ap[x] = init_float(t, key, dim + c * N + x);
+                bp[x] = init_float(t, key, 2 * dim + c * N + x);
+            }
+            opt_step_n<(int)N>(t.opt, gp, wp, ap, bp);
+            r[c] = wv;
+            if (t.opt.kind >= 2) r[units + c] = av;
+            if (t.opt.kind == 3) r[2 * units + c] = bv;
+        }
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+// ---- host side --------------------------------------------------------------------------------
+namespace {
+u32 g_part_cap = PA_CAP;
+u32 g_part_dbg = 0;
+}
+#ifdef PART_TIMING
+extern "C" int32_t pshbm_debug_part_timing(unsigned long long* out) {  // 32 words; the counters restart
+    unsigned long long zero[32] = {};
+    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(g_part_ticks), sizeof zero) != hipSuccess) return 10;
+    if (hipMemcpyToSymbol(HIP_SYMBOL(g_part_ticks), zero, sizeof zero) != hipSuccess) return 10;
+    return 0;
+}
+#endif
+void part_set_pass_capacity(uint32_t entries) {
+#ifdef PART_EXPERIMENT
+    g_part_dbg = entries >> 16;
+    entries &= 0xFFFFu;
+#endif
+    g_part_cap = entries == 0 || entries > PA_CAP ? PA_CAP : entries;
+}
+
+bool part_plan(const TableDev& t, size_t n, PartPlan* plan) {
+    if (n < PART_MIN_KEYS || n > PART_MAX_KEYS) return false;
+    const u32 vec = (t.dim % 4 == 0) ? 4u : 1u;
+    if (t.dim / vec > PA_BLOCK) return false;  // a lane per 4 or 16 bytes of a row
+    u32 bucket_bits = 0;
+    while ((1ull << bucket_bits) <= t.bucket_mask) ++bucket_bits;
+    u32 lp = 6;  // at least 64 partitions, about 1024 keys each
+    while ((1ull << lp) * 1024 < n && lp < 12) ++lp;
+    if (lp > bucket_bits) return false;  // a tiny table under a large batch: the sort path serves it
+    plan->n = (u32)n;
+    plan->n_tiles = (u32)((n + PT_TILE - 1) / PT_TILE);
+    plan->P = 1u << lp;
+    plan->part_shift = bucket_bits - lp;
+    return true;
+}
+
+PartSizes part_sizes(uint32_t dim, size_t n) {
+    PartSizes z{};
+    const size_t n_tiles = (n + PT_TILE - 1) / PT_TILE;
+    const size_t np = n_tiles * PT_TILE;
+    z.stage_key = np * 8;
+    z.stage_ref = np * 4;
+    z.ent_key = np * 8;
+    z.ent_ref = np * 4;
+    z.counts = n_tiles * PT_MAX_PARTS * 4;
+    z.starts = z.counts;
+    z.blocktot = n_tiles * (PT_MAX_PARTS / 64) * 4;
+    z.tile_total = n_tiles * 4;
+    z.pstart = (PT_MAX_PARTS + 1) * 4;
+    z.psum = n_tiles * PT_MAX_MULTI * (size_t)dim * 4;
+    z.new_slot = np * 4;
+    z.new_count = PT_MAX_PARTS * 4;
+    z.ngrad = np * (size_t)dim * 4;
+    return z;
+}
+
+hipError_t part_init() {
+    hipError_t e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&part_tile_kernel<float>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, PT_LDS)) != hipSuccess) return e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&part_tile_kernel<float4>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, PT_LDS)) != hipSuccess) return e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&part_apply_kernel<float>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, PA_LDS)) != hipSuccess) return e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&part_apply_kernel<float4>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, PA_LDS)) != hipSuccess) return e;
+    return hipSuccess;
+}
+
+hipError_t launch_part_tile(const TableDev& t, const PartPlan& pl, const PartBufs& b, const uint64_t* keys,
+                            const float* grads, hipStream_t s) {
+    if ((t.dim % 4 == 0) && aligned16(grads))
+        part_tile_kernel<float4><<<pl.n_tiles, PT_BLOCK, PT_LDS, s>>>(
+            t, keys, reinterpret_cast<const float4*>(grads), pl.n, pl.P, pl.part_shift, b.stage_key, b.stage_ref,
+            b.counts, b.starts, b.blocktot, b.tile_total, reinterpret_cast<float4*>(b.psum), t.dim / 4, g_part_dbg);
+    else
+        part_tile_kernel<float><<<pl.n_tiles, PT_BLOCK, PT_LDS, s>>>(t, keys, grads, pl.n, pl.P, pl.part_shift,
+                                                                    b.stage_key, b.stage_ref, b.counts, b.starts,
+                                                                    b.blocktot, b.tile_total, b.psum, t.dim,
+                                                                    g_part_dbg);
+    return hipGetLastError();
+}
+
+hipError_t launch_part_scan(const PartPlan& pl, const PartBufs& b, hipStream_t s) {
+    part_scan_kernel<<<pl.P / 64, PT_BLOCK, 0, s>>>(b.counts, b.starts, b.blocktot, b.pstart, pl.n_tiles, pl.P);
+    return hipGetLastError();
+}
+
+hipError_t launch_part_scatter(const TableDev& t, const PartPlan& pl, const PartBufs& b, hipStream_t s) {
+    part_scatter_kernel<<<pl.n_tiles, PT_BLOCK, 0, s>>>(t, b.stage_key, b.stage_ref, b.counts, b.tile_total, pl.P,
+                                                        pl.part_shift, b.ent_key, b.ent_ref);
+    return hipGetLastError();
+}
+
+hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads, bool insert,
+                             hipStream_t s) {
+    const bool v4 = (t.dim % 4 == 0) && aligned16(grads);
+    ApplyArgs a{b.ent_key, b.ent_ref, b.pstart, b.new_slot, b.new_count, v4 ? t.dim / 4 : t.dim, insert ? 1 : 0,
+                g_part_cap, g_part_dbg >> 8};
+    if (v4)
+        part_apply_kernel<float4><<<pl.P, PA_BLOCK, PA_LDS, s>>>(t, reinterpret_cast<const float4*>(grads),
+                                                                 reinterpret_cast<const float4*>(b.psum),
+                                                                 reinterpret_cast<float4*>(b.ngrad), a);
+    else
+        part_apply_kernel<float><<<pl.P, PA_BLOCK, PA_LDS, s>>>(t, grads, b.psum, b.ngrad, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads,
+                              hipStream_t s) {
+    if ((t.dim % 4 == 0) && aligned16(grads))
+        part_insert_kernel<float4><<<pl.P, PI_BLOCK, 0, s>>>(t, b.new_slot, reinterpret_cast<const float4*>(b.ngrad),
+                                                             b.new_count, b.pstart, pl.P, t.dim / 4);
+    else
+        part_insert_kernel<float><<<pl.P, PI_BLOCK, 0, s>>>(t, b.new_slot, b.ngrad, b.new_count, b.pstart, pl.P,
+                                                            t.dim);
+    return hipGetLastError();
+}
+
+}  // namespace pshbm
+

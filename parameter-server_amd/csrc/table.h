@@ -33,6 +33,7 @@ enum {
     CNT_ENTRY = 3,     // CNT_ROWS as it was when the current inserting operation began
     CNT_BADKEY = 4,    // reserved keys met in a batch (skipped)
     CNT_SORT_ERR = 5,  // a sort tile gave up waiting for its predecessor
+    CNT_PART_ERR = 6,  // a partition of a push held more entries of one hash class than a pass takes
     CNT_WORDS = 8
 };
 
@@ -180,6 +181,38 @@ hipError_t launch_unpack_records(const uint32_t* records, size_t n, uint32_t str
 // probe-distance histogram over the stored keys: hist[0..15], hist[16] = max distance.
 hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long long* hist,
                              hipStream_t s);
+
+// ---- partitioned push (push_part.hip) ---------------------------------------------------------
+// Aggregation and update of a batch of PART_MIN_KEYS .. PART_MAX_KEYS keys without a global sort:
+// tiles of 4096 keys, partitions of about 1024 keys. part_plan says whether a batch qualifies (and
+// how it is cut); part_sizes gives the bytes of each scratch array for batches of up to n keys.
+constexpr size_t PART_MIN_KEYS = 16384, PART_MAX_KEYS = 1u << 22;
+struct PartPlan {
+    uint32_t n, n_tiles, P, part_shift;
+};
+struct PartSizes {
+    size_t stage_key, stage_ref, ent_key, ent_ref, counts, starts, blocktot, tile_total, pstart, psum, new_slot,
+        new_count, ngrad;
+};
+struct PartBufs {
+    uint64_t *stage_key, *ent_key;
+    uint32_t *stage_ref, *ent_ref, *counts, *starts, *blocktot, *tile_total, *pstart, *new_slot, *new_count;
+    float *psum, *ngrad;
+};
+bool part_plan(const TableDev& t, size_t n, PartPlan* plan);
+PartSizes part_sizes(uint32_t dim, size_t n);
+hipError_t part_init();  // once per device, before the first launch
+hipError_t launch_part_tile(const TableDev& t, const PartPlan& pl, const PartBufs& b, const uint64_t* keys,
+                            const float* grads, hipStream_t s);
+hipError_t launch_part_scan(const PartPlan& pl, const PartBufs& b, hipStream_t s);
+hipError_t launch_part_scatter(const TableDev& t, const PartPlan& pl, const PartBufs& b, hipStream_t s);
+hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads, bool insert,
+                             hipStream_t s);
+hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads,
+                              hipStream_t s);
+// Entries a pass of the apply kernel takes (0 = the default, 2048): a test hook that makes small
+// batches go through the multi-pass path.
+void part_set_pass_capacity(uint32_t entries);
 
 // ---- for-each / erase / rebuild (maint.hip) -------------------------------------------------
 // Count and column sums of the rows that satisfy `pred`. scratch: for_each_scratch_bytes();

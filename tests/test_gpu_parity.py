@@ -834,7 +834,7 @@ def test_sort_that_gives_up_applies_nothing(ps, orc, wl):
     after the sort then leave the rows alone and the table reports FATAL until it is cleared. The
     host makes the wait give up (a limit of zero polls): every kernel still runs to its end."""
     rng = np.random.default_rng(21)
-    n_table, dim, n = 30000, 8, 20000          # 5 tiles of 4096 pairs: one-launch passes that wait
+    n_table, dim, n = 30000, 8, 14000          # 4 tiles of 4096 pairs: one-launch passes that wait
     t = ps.Table(dim, capacity=n_table + n, optimizer=1, lr=0.5)
     keys = wl.table_keys_np(0, n_table, seed=7)
     vals = rng.normal(0, 0.01, (n_table, dim)).astype(np.float32)

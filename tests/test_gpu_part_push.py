@@ -1,0 +1,139 @@
+"""The partitioned push (batches of 16,384 keys and more: tiles, partitions, one probe per distinct
+key) against the CPU oracle, through the C ABI. Bars as everywhere: stored key sets bit-exact,
+values bit-exact with integer gradients, within 1e-6 relative / 1e-7 absolute otherwise."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-6, 1e-7
+OPTS = {
+    "sum": dict(optimizer=0),
+    "sgd": dict(optimizer=1, lr=0.01),
+    "adagrad": dict(optimizer=2, lr=0.05, init_acc=0.1),
+    "ftrl": dict(optimizer=3, alpha=0.05, beta=1.0, l1=1e-4, l2=1e-5),
+}
+
+
+def sorted_dump(b):
+    st, rec = b.dump()
+    assert st == 0
+    return np.sort(rec, order="key")
+
+
+def same(t, r, exact):
+    a, b = sorted_dump(t), sorted_dump(r)
+    np.testing.assert_array_equal(a["key"], b["key"])
+    if exact:
+        np.testing.assert_array_equal(a["value"], b["value"])
+    else:
+        np.testing.assert_allclose(a["value"], b["value"], rtol=RTOL, atol=ATOL)
+
+
+def fill(t, r, wl, rng, n_table, opt, dim, seed):
+    keys = wl.table_keys_np(0, n_table, seed=seed)
+    vals = rng.normal(0, 0.01, (n_table, t.value_floats)).astype(np.float32)
+    if opt == "adagrad":
+        vals[:, dim:] = 0.1
+    if opt == "ftrl":
+        vals[:, 2 * dim:] = vals[:, dim:2 * dim] ** 2
+    assert t.set(keys, vals) == 0 and r.set(keys, vals) == 0
+    return keys
+
+
+@pytest.mark.parametrize("opt,dim,s", [("sgd", 16, 1.05), ("adagrad", 64, 1.2), ("ftrl", 8, 1.1),
+                                       ("adagrad", 128, 1.1), ("sgd", 3, 1.3), ("ftrl", 260, 1.1),
+                                       ("sum", 1, 1.5)])
+def test_zipf_batches_with_fresh_keys(ps, orc, wl, opt, dim, s):
+    """Exact aggregation in the oracle (float64 sums, rounded once): the kernels add in double
+    precision too, so the tolerance only covers the rounding of the tiles' partial sums."""
+    rng = np.random.default_rng(dim)
+    n_table, n = 50000, 40000 if dim <= 64 else 20000
+    t = ps.Table(dim, capacity=n_table + 3 * n, max_batch=n, **OPTS[opt])
+    r = orc.Oracle(dim, capacity=n_table + 3 * n, **OPTS[opt])
+    fill(t, r, wl, rng, n_table, opt, dim, seed=3)
+    for step in range(3):
+        q = wl.zipf_batch_np(rng, n_table, s, n, seed=3)
+        nf = n // 10
+        q[:nf] = wl.fresh_keys_np(rng, nf)                 # keys the push inserts
+        q[nf:nf + nf // 4] = q[:nf // 4]                    # some of them more than once
+        rng.shuffle(q)
+        g = rng.normal(0, 1e-3, (n, dim)).astype(np.float32)
+        flags = ps.PUSH_NO_INSERT if step == 2 else 0
+        assert t.push(q, g, flags) == 0, t.last_error()
+        assert r.push(q, g, flags | orc.PUSH_EXACT_AGGREGATION) == 0
+        same(t, r, exact=False)
+        assert t.size() == r.size()
+    t.close()
+
+
+@pytest.mark.parametrize("dim", [1, 4, 16, 36])
+def test_integer_gradients_bit_exact(ps, orc, dim):
+    """Integer sums are exact in any order (pico-ps/test/TestOps.h:98-117): heavy repetition, one
+    key that fills a fifth of the batch, keys inserted several times, all bit for bit."""
+    rng = np.random.default_rng(dim + 100)
+    t = ps.Table(dim, capacity=200_000, max_batch=150_000, **OPTS["sum"])
+    r = orc.Oracle(dim, capacity=200_000, **OPTS["sum"])
+    for n in (16384, 16385, 50_000, 150_000):
+        keys = (rng.zipf(1.2, n).astype(np.uint64) * np.uint64(2654435761)) % np.uint64(60_000)
+        keys[rng.integers(0, n, n // 5)] = 424242
+        g = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+        assert t.push(keys, g) == 0 and r.push(keys, g) == 0
+        same(t, r, exact=True)
+    n = 70_000                       # one key only, then two keys
+    for keys in (np.full(n, 7, np.uint64), np.where(np.arange(n) % 3 == 0, 8, 9).astype(np.uint64)):
+        g = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+        assert t.push(keys, g) == 0 and r.push(keys, g) == 0
+        same(t, r, exact=True)
+    t.close()
+
+
+def test_all_keys_distinct_and_all_new(ps, orc, wl):
+    rng = np.random.default_rng(5)
+    n, dim = 100_000, 8
+    t = ps.Table(dim, capacity=2 * n, max_batch=n, **OPTS["adagrad"])
+    r = orc.Oracle(dim, capacity=2 * n, **OPTS["adagrad"])
+    keys = wl.fresh_keys_np(rng, n)
+    g = rng.normal(0, 1e-2, (n, dim)).astype(np.float32)
+    assert t.push(keys, g) == 0 and r.push(keys, g) == 0      # every key inserted by the push
+    same(t, r, exact=True)                                    # nothing to aggregate: bit-exact
+    assert t.push(keys, g) == 0 and r.push(keys, g) == 0      # every key present
+    same(t, r, exact=True)
+    assert t.size() == n
+    t.close()
+
+
+def test_partitions_that_need_several_passes(ps, orc, wl):
+    """With the pass capacity turned down every partition of an ordinary batch takes the path of a
+    partition crowded by hot keys: passes over its entries by hash class."""
+    rng = np.random.default_rng(9)
+    n_table, n, dim = 40000, 60000, 16
+    t = ps.Table(dim, capacity=n_table + n, max_batch=n, **OPTS["sgd"])
+    r = orc.Oracle(dim, capacity=n_table + n, **OPTS["sgd"])
+    fill(t, r, wl, rng, n_table, "sgd", dim, seed=6)
+    q = wl.zipf_batch_np(rng, n_table, 1.05, n, seed=6)
+    q[:3000] = wl.fresh_keys_np(rng, 3000)
+    g = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+    try:
+        ps.debug_part_pass_capacity(256)
+        assert t.push(q, g) == 0 and r.push(q, g) == 0
+    finally:
+        ps.debug_part_pass_capacity(0)
+    same(t, r, exact=True)
+    assert t.size() == r.size()
+    t.close()
+
+
+def test_track_increment_through_the_partitioned_push(ps, orc, wl):
+    rng = np.random.default_rng(13)
+    n_table, n, dim = 30000, 20000, 4
+    t = ps.Table(dim, capacity=n_table + n, max_batch=n, track_increment=True, **OPTS["sgd"])
+    keys = wl.table_keys_np(0, n_table, seed=8)
+    assert t.set(keys, np.zeros((n_table, dim), np.float32)) == 0
+    q = np.concatenate([keys[rng.integers(0, n_table, n - 500)], wl.fresh_keys_np(rng, 500)])
+    g = rng.normal(0, 1, (n, dim)).astype(np.float32)
+    assert t.push(q, g) == 0
+    st, rec = t.take_increment()
+    assert st == 0
+    np.testing.assert_array_equal(np.sort(rec["key"]), np.unique(q))
+    t.close()
