@@ -204,7 +204,7 @@ struct pshbm_table {
     DevBuf ws_slot, ws_row, ws_idx, ws_srow, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wrow, ws_wval, ws_won;
     unsigned won_parity = 0;  // which half of ws_won the next inserting operation counts into
     // scratch of the partitioned push (batches of PART_MIN_KEYS keys and more)
-    DevBuf pt_stage_key, pt_stage_ref, pt_ent_key, pt_ent_ref, pt_counts, pt_starts, pt_blocktot, pt_tile_total,
+    DevBuf pt_stage, pt_ent, pt_counts, pt_starts, pt_blocktot, pt_tile_total,
         pt_pstart, pt_psum, pt_new_slot, pt_new_count, pt_ngrad;
     size_t part_keys = 0;       // batch size those arrays serve
 
@@ -387,10 +387,8 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     if (cap >= PART_MIN_KEYS && part_plan(t->d, std::min(cap, PART_MAX_KEYS), &probe_plan)) {
         const size_t pk = std::min(cap, PART_MAX_KEYS);
         const PartSizes z = part_sizes(t->d.dim, pk);
-        ST_TRY(ensure(t, t->pt_stage_key, z.stage_key));
-        ST_TRY(ensure(t, t->pt_stage_ref, z.stage_ref));
-        ST_TRY(ensure(t, t->pt_ent_key, z.ent_key));
-        ST_TRY(ensure(t, t->pt_ent_ref, z.ent_ref));
+        ST_TRY(ensure(t, t->pt_stage, z.stage));
+        ST_TRY(ensure(t, t->pt_ent, z.ent));
         ST_TRY(ensure(t, t->pt_counts, z.counts));
         ST_TRY(ensure(t, t->pt_starts, z.starts));
         ST_TRY(ensure(t, t->pt_blocktot, z.blocktot));
@@ -565,10 +563,8 @@ Workspace table_workspace(pshbm_table* t) {
     w.won_words = half;
     w.part_keys = t->part_keys;
     if (t->part_keys) {
-        w.part.stage_key = static_cast<uint64_t*>(t->pt_stage_key.p);
-        w.part.stage_ref = static_cast<uint32_t*>(t->pt_stage_ref.p);
-        w.part.ent_key = static_cast<uint64_t*>(t->pt_ent_key.p);
-        w.part.ent_ref = static_cast<uint32_t*>(t->pt_ent_ref.p);
+        w.part.stage = static_cast<uint4*>(t->pt_stage.p);
+        w.part.ent = static_cast<uint4*>(t->pt_ent.p);
         w.part.counts = static_cast<uint32_t*>(t->pt_counts.p);
         w.part.starts = static_cast<uint32_t*>(t->pt_starts.p);
         w.part.blocktot = static_cast<uint32_t*>(t->pt_blocktot.p);
@@ -700,7 +696,7 @@ void destroy_impl(pshbm_table* t) {
     DevBuf* bufs[] = {&t->ws_slot, &t->ws_row, &t->ws_idx,  &t->ws_srow, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
                       &t->ws_pval, &t->ws_wrow, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_raw,
                       &t->ms_dead, &t->ms_tiles, &t->ms_lists, &t->ms_fe,
-                      &t->pt_stage_key, &t->pt_stage_ref, &t->pt_ent_key, &t->pt_ent_ref, &t->pt_counts, &t->pt_starts,
+                      &t->pt_stage, &t->pt_ent, &t->pt_counts, &t->pt_starts,
                       &t->pt_blocktot, &t->pt_tile_total, &t->pt_pstart, &t->pt_psum, &t->pt_new_slot, &t->pt_new_count,
                       &t->pt_ngrad,
                       &t->q_keys,  &t->q_grads};

@@ -21,7 +21,9 @@
 //                           initialises their rows and takes their step.
 // Sums are accumulated in double precision and rounded to fp32 once per tile and once per key: the
 // result does not depend on the order in which a key's rows are met beyond the last bit of a
-// 53-bit sum.
+// 53-bit sum. Loads that a later step needs are never put behind a branch (a lane without work
+// loads element 0 and drops it): the compiler then keeps all of them in flight together, which
+// is what these latency-bound kernels live on.
 #include "table.h"
 #include "probe.h"
 #include "rowops.h"
@@ -32,33 +34,8 @@ namespace {
 
 using u16 = uint16_t;
 
-#ifdef PART_EXPERIMENT
-// Build-time option for the developer: phases switched off by bits of a process-wide word, to see
-// what each costs (results are then wrong).
-#define DBG(flags, bit) (((flags) >> (bit)) & 1u)
-#else
-#define DBG(flags, bit) false
-#endif
-
-#ifdef PART_TIMING
-// Build-time option for the developer: time spent per phase of the tile and apply kernels, summed
-// over the workgroups (ticks of the 100 MHz wall clock), read back by pshbm_debug_part_timing.
-__device__ unsigned long long g_part_ticks[2][16];
-#define TICK_INIT long long tick_last = wall_clock64()
-#define TICK(kernel, phase)                                                                  \
-    do {                                                                                      \
-        if (threadIdx.x == 0) {                                                               \
-            const long long now = wall_clock64();                                             \
-            atomicAdd(&g_part_ticks[kernel][phase], (unsigned long long)(now - tick_last));   \
-            tick_last = now;                                                                  \
-        }                                                                                     \
-    } while (0)
-#else
-#define TICK_INIT
-#define TICK(kernel, phase)
-#endif
-
 constexpr u32 PT_TILE = 4096, PT_BLOCK = 1024, PT_ITEMS = PT_TILE / PT_BLOCK;
+constexpr u32 SC_BLOCK = 1024;                // threads of the scan kernel
 constexpr u32 PT_HT = 2 * PT_TILE;            // slots of a tile's LDS hash table
 constexpr u32 PT_MAX_MULTI = PT_TILE / 2;     // pre-summed rows a tile can produce
 constexpr u32 PT_ACC_DOUBLES = PT_TILE;       // accumulators: the room of the tile's key array (32 KiB)
@@ -142,8 +119,8 @@ struct Acc<float4> {
     }
 };
 
-// Sums of lists of gradient rows, all lists at once: elements [lo, hi) are dealt to the NG lane
-// groups in turn (so a long list is spread over all of them), element e belongs to list lid[e]
+// Sums of lists of gradient rows, all lists at once: elements [lo, hi) are cut into equal runs, one
+// per lane group (so a long list is spread over several groups), element e belongs to list lid[e]
 // (ascending in e) and its row is src(e); a group adds consecutive elements of one list in
 // registers and adds the sum to the list's accumulators in LDS when the list changes.
 // acc[((list - list_base) * units + c) * N + x], double, zero on entry.
@@ -173,28 +150,35 @@ struct ListSum {
     }
 };
 
-// elements first, first + NG, ... below hi
+// elements first, first + 1, ... below last
 template <typename T, typename SRC>
-__device__ __forceinline__ void flat_sum_from(SRC src, const u16* lid, u32 first, u32 hi, u32 NG, u32 c,
-                                              ListSum<T>& ls) {
+__device__ __forceinline__ void flat_sum_from(SRC src, const u16* lid, u32 first, u32 last, u32 c, ListSum<T>& ls) {
     u32 e = first;
-    for (; e + 3 * NG < hi; e += 4 * NG) {  // four rows in flight
-        const u32 l0 = lid[e], l1 = lid[e + NG], l2 = lid[e + 2 * NG], l3 = lid[e + 3 * NG];
-        const T v0 = src(e)[c], v1 = src(e + NG)[c], v2 = src(e + 2 * NG)[c], v3 = src(e + 3 * NG)[c];
+    for (; e + 3 < last; e += 4) {  // four rows in flight
+        const u32 l0 = lid[e], l1 = lid[e + 1], l2 = lid[e + 2], l3 = lid[e + 3];
+        const T v0 = src(e)[c], v1 = src(e + 1)[c], v2 = src(e + 2)[c], v3 = src(e + 3)[c];
         ls.take(l0, v0);
         ls.take(l1, v1);
         ls.take(l2, v2);
         ls.take(l3, v3);
     }
-    for (; e < hi; e += NG) ls.take(lid[e], src(e)[c]);
+    for (; e < last; ++e) ls.take(lid[e], src(e)[c]);
 }
+
+// Lane group g of NG takes the g-th of NG equal runs of consecutive elements: consecutive elements
+// mostly belong to one list, so a group adds to the accumulators about once per list it meets and
+// not once per element (additions of doubles in LDS go one lane at a time).
+__device__ __forceinline__ u32 chunk_len(u32 lo, u32 hi, u32 NG) { return (hi - lo + NG - 1) / NG; }
 
 template <typename T, typename SRC>
 __device__ __forceinline__ void flat_sum(SRC src, const u16* lid, u32 lo, u32 hi, u32 list_base, double* acc,
                                          u32 units, u32 NG, u32 g, u32 c) {
     ListSum<T> ls;
     ls.begin(acc, list_base, units, c);
-    flat_sum_from<T>(src, lid, lo + g, hi, NG, c, ls);
+    const u32 len = chunk_len(lo, hi, NG);
+    const u32 first = lo + g * len < hi ? lo + g * len : hi;
+    const u32 last = first + len < hi ? first + len : hi;
+    flat_sum_from<T>(src, lid, first, last, c, ls);
     ls.flush();
 }
 
@@ -203,7 +187,7 @@ __device__ __forceinline__ u32 partition_of(const TableDev& t, u64 h, u32 part_s
 }
 
 // ---- 1. tile kernel ---------------------------------------------------------------------------
-// LDS (dynamic, 128 KiB): keys of the tile (later the accumulators) | hash table (later the list of
+// LDS (dynamic, 112 KiB + a word per partition): keys of the tile (later the accumulators) | hash table (later the list of
 // keys that repeat) | per-item counts | per-item aux | list of repeating items + their list numbers |
 // partition histogram.
 constexpr u32 PT_OFF_OWNER = PT_TILE * 8;
@@ -213,13 +197,12 @@ constexpr u32 PT_OFF_LIST = PT_OFF_AUX + PT_TILE * 4;
 constexpr u32 PT_OFF_LOWN = PT_OFF_LIST + PT_TILE * 2;
 constexpr u32 PT_OFF_HIST = PT_OFF_LOWN + PT_TILE * 2;
 constexpr u32 PT_MAX_PARTS = 4096;
-constexpr u32 PT_LDS = PT_OFF_HIST + PT_MAX_PARTS * 4;  // 131072
+constexpr u32 PT_LDS_FIXED = PT_OFF_HIST;  // 114688, then one word per partition
 
 template <typename T>
 __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
     TableDev t, const u64* __restrict__ keys, const T* __restrict__ grads, u32 n, u32 P, u32 part_shift,
-    u64* __restrict__ stage_key, u32* __restrict__ stage_ref, u32* __restrict__ counts, u32* __restrict__ starts,
-    u32* __restrict__ blocktot, u32* __restrict__ tile_total, T* __restrict__ psum, u32 units, u32 dbg) {
+    uint4* __restrict__ stage, u32* __restrict__ counts, u32* __restrict__ starts, u32* __restrict__ blocktot, u32* __restrict__ tile_total, T* __restrict__ psum, u32 units) {
     extern __shared__ __align__(16) unsigned char pt_lds[];
     u64* lkey = reinterpret_cast<u64*>(pt_lds);
     u32* owner = reinterpret_cast<u32*>(pt_lds + PT_OFF_OWNER);
@@ -233,16 +216,20 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
     const u32 tid = threadIdx.x;
     const u32 tile = blockIdx.x;
     const u64 tb = (u64)tile * PT_TILE;
-    TICK_INIT;
 
     u64 key[PT_ITEMS], hh[PT_ITEMS];
     bool valid[PT_ITEMS];
     u32 nbad = 0;
 #pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j) {  // no branch around a load: the four stay in flight together
+        const u64 i = tb + j * PT_BLOCK + tid;
+        key[j] = keys[i < n ? i : (u64)n - 1];
+    }
+#pragma unroll
     for (u32 j = 0; j < PT_ITEMS; ++j) {
         const u32 q = j * PT_BLOCK + tid;
         const u64 i = tb + q;
-        key[j] = i < n ? keys[i] : KEY_EMPTY;
+        if (i >= n) key[j] = KEY_EMPTY;
         valid[j] = i < n && key[j] < KEY_DELETED;
         nbad += (i < n && !valid[j]) ? 1u : 0u;
         lkey[q] = key[j];
@@ -253,8 +240,8 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
     for (u32 x = 0; x < PT_HT / PT_BLOCK; ++x) owner[x * PT_BLOCK + tid] = NONE32;
     for (u32 x = tid; x < P; x += PT_BLOCK) hist[x] = 0;
     if (nbad) atomicAdd(&t.counters[CNT_BADKEY], nbad);  // reserved keys are skipped (and rare)
+    if (tile == 0 && tid == 0) t.counters[CNT_ANY_NEW] = 0u;
     __syncthreads();
-    TICK(0, 0);
 
     // the items of one key agree on a representative and number themselves
     u32 rep[PT_ITEMS], arr[PT_ITEMS];
@@ -264,7 +251,6 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
         if (valid[j]) dedupe_insert(key[j], j * PT_BLOCK + tid, hh[j], lkey, owner, cnt, PT_HT - 1, rep[j], arr[j]);
     }
     __syncthreads();
-    TICK(0, 1);
 
     // keys that repeat: a number each (in thread order) and a range of the item list
     u32 m[PT_ITEMS];
@@ -294,7 +280,6 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
             }
     }
     __syncthreads();
-    TICK(0, 2);
 #pragma unroll
     for (u32 j = 0; j < PT_ITEMS; ++j)
         if (valid[j] && m[j] >= 2) {
@@ -311,7 +296,6 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
         prank[j] = isrep[j] ? atomicAdd(&hist[part[j]], 1u) : 0u;
     }
     __syncthreads();
-    TICK(0, 3);
 
     // Pre-summed rows of the keys that repeat, as many lists per round as the accumulators hold
     // (the room of the key array, which nobody reads any more). The rows of the first round are
@@ -323,19 +307,22 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
     const bool on = g < NG;
     const u32 B = PT_ACC_DOUBLES / (units * N);  // lists per round, at least 1
     const T* tile_grads = grads + tb * units;
-    constexpr u32 PF = 4;
+    constexpr u32 PF = 8;
     T pv[PF];
     u32 pl[PF];
     const u32 first_b1 = B < n_multi ? B : n_multi;
     const u32 first_hi = first_b1 < n_multi ? (aux[mrep[first_b1]] & 0xFFFFu) : n_elems;
     for (u32 x = tid; x < first_b1 * units * N; x += PT_BLOCK) acc[x] = 0.0;
+    const u32 first_len = chunk_len(0u, first_hi, NG);
+    const u32 my_first = g * first_len < first_hi ? g * first_len : first_hi;
+    const u32 my_last = my_first + first_len < first_hi ? my_first + first_len : first_hi;
 #pragma unroll
     for (u32 k = 0; k < PF; ++k) {
-        const u32 e = g + k * NG;
-        const bool ok = on && e < first_hi;
+        const u32 e = my_first + k;
+        const bool ok = on && e < my_last;
         pl[k] = ok ? (u32)lown[e] : NONE32;
-        pv[k] = vzero(T());
-        if (ok && !DBG(dbg, 1)) pv[k] = tile_grads[(size_t)list[e] * units + c];
+        const u32 q = ok ? (u32)list[e] : 0u;  // (a lane without an element loads row 0 and drops it)
+        pv[k] = tile_grads[(size_t)q * units + (on ? c : 0u)];
     }
     {
         // thread x owns PP consecutive partitions (P is a power of two, at least 64): their counts,
@@ -367,17 +354,15 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
         }
     }
     __syncthreads();
-    TICK(0, 4);
 #pragma unroll
     for (u32 j = 0; j < PT_ITEMS; ++j)
         if (isrep[j]) {
             const u64 pos = tb + hist[part[j]] + prank[j];
-            stage_key[pos] = key[j];
-            stage_ref[pos] = multi[j] ? (REF_PSUM | (tile * PT_MAX_MULTI + (aux[j * PT_BLOCK + tid] >> 16)))
-                                      : (u32)(tb + j * PT_BLOCK + tid);
+            const u32 ref = multi[j] ? (REF_PSUM | (tile * PT_MAX_MULTI + (aux[j * PT_BLOCK + tid] >> 16)))
+                                     : (u32)(tb + j * PT_BLOCK + tid);
+            stage[pos] = make_uint4((u32)key[j], (u32)(key[j] >> 32), ref, 0u);
         }
-    if (n_multi == 0 || DBG(dbg, 0)) return;  // block-uniform
-    TICK(0, 5);
+    if (n_multi == 0) return;  // block-uniform
 
     for (u32 b0 = 0; b0 < n_multi; b0 += B) {
         const u32 b1 = b0 + B < n_multi ? b0 + B : n_multi;
@@ -391,7 +376,7 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
 #pragma unroll
                 for (u32 k = 0; k < PF; ++k)
                     if (pl[k] != NONE32) ls.take(pl[k], pv[k]);
-                flat_sum_from<T>(row_of, lown, g + PF * NG, hi, NG, c, ls);
+                flat_sum_from<T>(row_of, lown, my_first + PF < my_last ? my_first + PF : my_last, my_last, c, ls);
                 ls.flush();
             }
         } else {
@@ -400,13 +385,11 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
             if (on) flat_sum<T>(row_of, lown, lo, hi, b0, acc, units, NG, g, c);
         }
         __syncthreads();
-        TICK(0, 7);
         if (on)
             for (u32 l = b0 + g; l < b1; l += NG)
                 psum[((size_t)tile * PT_MAX_MULTI + l) * units + c] =
                     Acc<T>::load(acc + ((size_t)(l - b0) * units + c) * N);
         __syncthreads();
-        TICK(0, 8);
     }
 }
 
@@ -417,44 +400,72 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
 // (lane = partition) over all tiles, which its 16 wavefronts split into consecutive parts; what the
 // lower blocks hold it adds up from the per-tile block counts the tile kernel left (no atomic
 // additions anywhere: additions to one address from all over the device are resolved one by one).
-__global__ __launch_bounds__(PT_BLOCK) void part_scan_kernel(u32* __restrict__ counts, const u32* __restrict__ starts,
+__global__ __launch_bounds__(SC_BLOCK) void part_scan_kernel(u32* __restrict__ counts, const u32* __restrict__ starts,
                                                               const u32* __restrict__ blocktot,
                                                               u32* __restrict__ pstart, u32 n_tiles, u32 P) {
-    __shared__ u32 red[PT_BLOCK / 64];
+    __shared__ u32 red[SC_BLOCK / 64];
     __shared__ u32 colbase[64];
-    __shared__ u32 part_sum[PT_BLOCK / 64][64];
+    __shared__ u32 part_sum[SC_BLOCK / 64][64];
+    constexpr u32 WAVES = SC_BLOCK / 64, KEEP = 32;
     const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
     const u32 blk = blockIdx.x, d0 = blk * 64u, NB = P / 64u;
-    // entries of the lower blocks, over all tiles
-    u32 before = 0;
-    for (u32 t0 = tid / 64u; t0 < n_tiles; t0 += PT_BLOCK / 64u)
-        for (u32 x = lane; x < blk; x += 64u) before += blocktot[(size_t)t0 * NB + x];
-    for (u32 off = 32; off >= 1; off >>= 1) before += __shfl_down(before, off);
-    if (lane == 0) red[w] = before;
-    const u32 per = (n_tiles + PT_BLOCK / 64 - 1) / (PT_BLOCK / 64);
+    const u32 per = (n_tiles + WAVES - 1) / WAVES;
     const u32 t0 = w * per < n_tiles ? w * per : n_tiles;
     const u32 t1 = t0 + per < n_tiles ? t0 + per : n_tiles;
     u32* col = counts + d0 + lane;
     const u32* scol = starts + d0 + lane;
+    // all the loads of this workgroup are issued before the first is used: the counts of this
+    // wavefront's tiles (kept in registers when there are few), the block counts of the lower blocks
+    const bool keep = per <= KEEP;
+    u32 v[KEEP], st[KEEP];
     u32 s = 0;
+    if (keep) {
+#pragma unroll
+        for (u32 x = 0; x < KEEP; ++x) {
+            const bool in = t0 + x < t1;
+            v[x] = in ? col[(size_t)(t0 + x) * P] : 0u;
+            st[x] = in ? scol[(size_t)(t0 + x) * P] : 0u;
+        }
+    }
+    u32 before = 0;
     {
+        // (tile, lower block) pairs dealt to the threads, eight loads in flight
+        const u32 pairs = n_tiles * blk;
+        for (u32 i0 = tid; i0 < pairs; i0 += 8 * SC_BLOCK) {
+            u32 bv[8];
+#pragma unroll
+            for (u32 x = 0; x < 8; ++x) {
+                const u32 i = i0 + x * SC_BLOCK;
+                bv[x] = 0;
+                if (i < pairs) bv[x] = blocktot[(size_t)(i / blk) * NB + i % blk];
+            }
+#pragma unroll
+            for (u32 x = 0; x < 8; ++x) before += bv[x];
+        }
+    }
+    if (keep) {
+#pragma unroll
+        for (u32 x = 0; x < KEEP; ++x) s += v[x];
+    } else {
         u32 tt = t0;
         for (; tt + 8 <= t1; tt += 8) {
-            u32 v[8];
+            u32 cv[8];
 #pragma unroll
-            for (u32 x = 0; x < 8; ++x) v[x] = col[(size_t)(tt + x) * P];
+            for (u32 x = 0; x < 8; ++x) cv[x] = col[(size_t)(tt + x) * P];
 #pragma unroll
-            for (u32 x = 0; x < 8; ++x) s += v[x];
+            for (u32 x = 0; x < 8; ++x) s += cv[x];
         }
         for (; tt < t1; ++tt) s += col[(size_t)tt * P];
     }
+    for (u32 off = 32; off >= 1; off >>= 1) before += __shfl_down(before, off);
+    if (lane == 0) red[w] = before;
     part_sum[w][lane] = s;
     __syncthreads();
     if (w == 0) {  // this block's partitions: totals, their exclusive prefix over the lanes
         u32 base = 0;
-        for (u32 x = 0; x < PT_BLOCK / 64; ++x) base += red[x];
+        for (u32 x = 0; x < WAVES; ++x) base += red[x];
         u32 tot = 0;
-        for (u32 x = 0; x < PT_BLOCK / 64; ++x) tot += part_sum[x][lane];
+        for (u32 x = 0; x < WAVES; ++x) tot += part_sum[x][lane];
         u32 incl = tot;
         for (u32 off = 1; off < 64; off <<= 1) {
             const u32 o = __shfl_up(incl, off);
@@ -467,55 +478,60 @@ __global__ __launch_bounds__(PT_BLOCK) void part_scan_kernel(u32* __restrict__ c
     __syncthreads();
     u32 pos = colbase[lane];
     for (u32 x = 0; x < w; ++x) pos += part_sum[x][lane];
-    {
+    if (keep) {
+#pragma unroll
+        for (u32 x = 0; x < KEEP; ++x)
+            if (t0 + x < t1) {
+                col[(size_t)(t0 + x) * P] = pos - st[x];
+                pos += v[x];
+            }
+    } else {
         u32 tt = t0;
         for (; tt + 8 <= t1; tt += 8) {
-            u32 v[8], st[8];
+            u32 cv[8], sv[8];
 #pragma unroll
             for (u32 x = 0; x < 8; ++x) {
-                v[x] = col[(size_t)(tt + x) * P];
-                st[x] = scol[(size_t)(tt + x) * P];
+                cv[x] = col[(size_t)(tt + x) * P];
+                sv[x] = scol[(size_t)(tt + x) * P];
             }
 #pragma unroll
             for (u32 x = 0; x < 8; ++x) {
-                col[(size_t)(tt + x) * P] = pos - st[x];
-                pos += v[x];
+                col[(size_t)(tt + x) * P] = pos - sv[x];
+                pos += cv[x];
             }
         }
         for (; tt < t1; ++tt) {
-            const u32 v = col[(size_t)tt * P];
+            const u32 c = col[(size_t)tt * P];
             col[(size_t)tt * P] = pos - scol[(size_t)tt * P];
-            pos += v;
+            pos += c;
         }
     }
 }
 
 // ---- 3. scatter -----------------------------------------------------------------------------------
-__global__ __launch_bounds__(PT_BLOCK) void part_scatter_kernel(TableDev t, const u64* __restrict__ stage_key,
-                                                                 const u32* __restrict__ stage_ref,
+__global__ __launch_bounds__(PT_BLOCK) void part_scatter_kernel(TableDev t, const uint4* __restrict__ stage,
                                                                  const u32* __restrict__ delta,
                                                                  const u32* __restrict__ tile_total, u32 P,
-                                                                 u32 part_shift, u64* __restrict__ ent_key,
-                                                                 u32* __restrict__ ent_ref) {
+                                                                 u32 part_shift, uint4* __restrict__ ent) {
     const u32 tile = blockIdx.x, tid = threadIdx.x;
     const u64 tb = (u64)tile * PT_TILE;
     const u32 cnt = tile_total[tile];
-    u64 key[PT_ITEMS];
-    u32 ref[PT_ITEMS];
+    uint4 e[PT_ITEMS];
 #pragma unroll
     for (u32 j = 0; j < PT_ITEMS; ++j) {
         const u32 q = j * PT_BLOCK + tid;
-        key[j] = q < cnt ? stage_key[tb + q] : KEY_EMPTY;
-        ref[j] = q < cnt ? stage_ref[tb + q] : 0u;
+        e[j] = stage[tb + (q < cnt ? q : 0u)];
+    }
+    u32 d[PT_ITEMS];
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j) {
+        const u32 p = partition_of(t, hash64(((u64)e[j].y << 32) | e[j].x), part_shift);
+        d[j] = delta[(size_t)tile * P + p];
     }
 #pragma unroll
     for (u32 j = 0; j < PT_ITEMS; ++j) {
         const u32 q = j * PT_BLOCK + tid;
-        if (q >= cnt) continue;
-        const u32 p = partition_of(t, hash64(key[j]), part_shift);
-        const u32 pos = delta[(size_t)tile * P + p] + q;
-        ent_key[pos] = key[j];
-        ent_ref[pos] = ref[j];
+        if (q < cnt) ent[d[j] + q] = e[j];
     }
 }
 
@@ -534,24 +550,23 @@ constexpr u32 PA_OFF_MREP = PA_OFF_UREP + PA_CAP * 2;
 constexpr u32 PA_LDS = PA_OFF_MREP + PA_CAP * 2;  // 75776
 
 struct ApplyArgs {
-    const u64* ent_key;
-    const u32* ent_ref;
+    const uint4* ent;  // {key low, key high, reference, -}
     const u32* pstart;
     u32* new_slot;
     u32* new_count;
     u32 units;
     int insert;
     u32 cap;  // entries a pass holds: PA_CAP, or less when a test wants to see the passes
-    u32 dbg;
 };
 
-// The keys of a pass that have one entry: their gradient row is their sum. Lane group g takes keys
-// g, g + NG, ..., KS of them at a time, so that the loads of KS gradient rows and KS table rows are
-// in flight together.
+// The optimizer step of the distinct keys of a pass: a key with one entry takes its gradient row, a
+// key with several the sum that lies in the accumulators (lists below n_summed; the others are
+// left to later rounds). Lane group g takes keys g, g + NG, ..., KS of them at a time, so that the
+// loads of KS gradient rows and KS table rows are in flight together.
 template <typename T, int KIND, u32 KS>
-__device__ __forceinline__ void apply_singles(const TableDev& t, unsigned char* lds, const T* __restrict__ grads,
-                                              const T* __restrict__ psum, T* __restrict__ ngrad, u32 s, u32 U,
-                                              u32 units, u32 NG, u32 g, u32 c) {
+__device__ __forceinline__ void apply_keys(const TableDev& t, unsigned char* lds, const T* __restrict__ grads,
+                                           const T* __restrict__ psum, T* __restrict__ ngrad, u32 s, u32 U, u32 units,
+                                           u32 NG, u32 g, u32 c, const double* acc, u32 n_summed) {
     constexpr u32 N = sizeof(T) / 4;
     constexpr int STATES = KIND <= 1 ? 0 : KIND - 1;
     const u32* cnt = reinterpret_cast<const u32*>(lds + PA_OFF_CNT);
@@ -573,28 +588,35 @@ __device__ __forceinline__ void apply_singles(const TableDev& t, unsigned char* 
             rowk[k] = ROW_NONE;
             dst[k] = 0;
             gv[k] = vzero(T());
+            u32 ref = 0;          // (a lane with nothing to fetch loads row 0 and drops it:
+            bool summed = false;  // no branch around the loads, so that all of them are in flight)
+            u32 mi = 0;
             if (u < U) {
                 const u32 i = urep[u];
+                const u32 av_ = aux[i];
                 if (cnt[i] == 1) {
                     single[k] = true;
-                    const u32 av_ = aux[i];
+                    ref = list[av_ & 0xFFFFu];
+                } else {
+                    mi = (av_ >> 16) & 0x7FFFu;
+                    summed = mi < n_summed;
+                    single[k] = summed;
+                }
+                if (single[k]) {
                     isnew[k] = (av_ & AUX_NEW) != 0;
-                    const u32 ref = list[av_ & 0xFFFFu];
-                    gv[k] = ((ref & REF_PSUM) ? psum + (size_t)(ref & ~REF_PSUM) * units : grads + (size_t)ref * units)[c];
                     dst[k] = urow[u];
                     if (!isnew[k] && dst[k] < t.max_rows) rowk[k] = dst[k];
                 }
             }
+            gv[k] = ((ref & REF_PSUM) ? psum + (size_t)(ref & ~REF_PSUM) * units : grads + (size_t)ref * units)[c];
+            if (summed) gv[k] = Acc<T>::load(acc + ((size_t)mi * units + c) * N);
         }
 #pragma unroll
         for (u32 k = 0; k < KS; ++k) {
-            wv[k] = vzero(T());
-            if (rowk[k] != ROW_NONE) {
-                const T* r = rows + (size_t)rowk[k] * stride_units + c;
-                wv[k] = r[0];
-                if constexpr (STATES >= 1) av[k] = r[units];
-                if constexpr (STATES >= 2) bv[k] = r[2 * units];
-            }
+            const T* r = rows + (size_t)(rowk[k] != ROW_NONE ? rowk[k] : 0u) * stride_units + c;
+            wv[k] = r[0];
+            if constexpr (STATES >= 1) av[k] = r[units];
+            if constexpr (STATES >= 2) bv[k] = r[2 * units];
         }
 #pragma unroll
         for (u32 k = 0; k < KS; ++k) {
@@ -638,14 +660,12 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
     u16* mrep = reinterpret_cast<u16*>(lds + PA_OFF_MREP);
     const u32 tid = threadIdx.x, lane = tid & 63u;
     const u32 units = a.units;
-    TICK_INIT;
 
 #pragma unroll
     for (u32 x = 0; x < PA_HT / PA_BLOCK; ++x) owner[x * PA_BLOCK + tid] = NONE32;
 #pragma unroll
     for (u32 j = 0; j < PA_ITEMS; ++j) cnt[j * PA_BLOCK + tid] = 0;
     __syncthreads();
-    TICK(1, 0);
 
     u32 rep[PA_ITEMS], arr[PA_ITEMS];
     bool valid[PA_ITEMS];
@@ -660,7 +680,6 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
         }
     }
     __syncthreads();
-    TICK(1, 1);
 
     // distinct keys numbered; the references of the keys with several entries come first in the list
     u32 m[PA_ITEMS];
@@ -696,7 +715,6 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
             }
     }
     __syncthreads();
-    TICK(1, 2);
 #pragma unroll
     for (u32 j = 0; j < PA_ITEMS; ++j)
         if (valid[j]) {
@@ -705,8 +723,22 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
             list[pos] = lref[j * PA_BLOCK + tid];
             lown[pos] = (u16)(av >> 16);
         }
+    // the hash table is done with: its room becomes the accumulators of the keys with several entries,
+    // as many lists as it holds (normally all of them)
+    double* acc = reinterpret_cast<double*>(owner);
+    const u32 B = PA_ACC_DOUBLES / (units * N);
+    const u32 first_b1 = B < n_multi ? B : n_multi;
+    for (u32 x = tid; x < first_b1 * units * N; x += PA_BLOCK) acc[x] = 0.0;
     __syncthreads();
-    TICK(1, 3);
+    const u32 G = units;  // the host admits units <= PA_BLOCK
+    const u32 NG = PA_BLOCK / G;
+    const u32 g = tid / G, c = tid - g * G;
+    const bool on = g < NG;
+    auto src = [&](u32 ref) -> const T* {
+        return (ref & REF_PSUM) ? psum + (size_t)(ref & ~REF_PSUM) * units : grads + (size_t)ref * units;
+    };
+    bool sums_due = n_multi != 0;  // block-uniform
+    const u32 first_hi = first_b1 < n_multi ? (aux[urep[mrep[first_b1]]] & 0xFFFFu) : n_elems;
 
     // One probe per distinct key, four lanes each. A lane group looks at the home buckets of
     // several keys at once (all the loads in flight together); a key that is not in its home
@@ -714,9 +746,7 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
     u32* urow = lref;
     const u32 grp = lane >> 2, sub = lane & 3u;
     constexpr u32 KP = 4, QUADS = PA_BLOCK / 4;
-    if (DBG(a.dbg, 0))
-        for (u32 u = tid; u < U; u += PA_BLOCK) urow[u] = ROW_NONE;
-    for (u32 u0 = 0; u0 < U && !DBG(a.dbg, 0); u0 += QUADS * KP) {
+    for (u32 u0 = 0; u0 < U; u0 += QUADS * KP) {
         u32 uu[KP], ii[KP];
         u64 kk[KP];
         bool act[KP];
@@ -727,8 +757,11 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
             act[k] = uu[k] < U;
             ii[k] = act[k] ? urep[uu[k]] : 0u;
             kk[k] = act[k] ? lkey[ii[k]] : KEY_EMPTY;
-            sv[k] = make_uint4(0u, 0u, 0u, 0u);
-            if (act[k]) sv[k] = t.slots[(u64)((u32)hash64(kk[k]) & t.bucket_mask) * 4 + sub];
+            sv[k] = t.slots[(u64)((u32)hash64(kk[k]) & t.bucket_mask) * 4 + sub];
+        }
+        if (sums_due) {  // while the buckets are on their way: the sums of the keys with several entries
+            if (on) flat_sum<T>([&](u32 e) { return src(list[e]); }, lown, 0u, first_hi, 0u, acc, units, NG, g, c);
+            sums_due = false;
         }
 #pragma unroll
         for (u32 k = 0; k < KP; ++k) {
@@ -768,15 +801,7 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
         }
     }
     __syncthreads();
-    TICK(1, 4);
 
-    const u32 G = units;  // the host admits units <= PA_BLOCK
-    const u32 NG = PA_BLOCK / G;
-    const u32 g = tid / G, c = tid - g * G;
-    const bool on = g < NG;
-    auto src = [&](u32 ref) -> const T* {
-        return (ref & REF_PSUM) ? psum + (size_t)(ref & ~REF_PSUM) * units : grads + (size_t)ref * units;
-    };
     auto apply = [&](u32 u, u32 i, T gv) {
         if (aux[i] & AUX_NEW) {
             ngrad[(size_t)(s + urow[u]) * units + c] = gv;
@@ -785,37 +810,30 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
             if (row != ROW_NONE) finalize<T>(t, row, c, units, gv);
         }
     };
-    // keys with one entry: the gradient row is the sum; several keys per lane group in flight
-    if (on && !DBG(a.dbg, 1)) {
+    // one sweep over the distinct keys: step and store
+    if (on) {
         switch (t.opt.kind) {
-            case 0: apply_singles<T, 0, 4>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c); break;
-            case 1: apply_singles<T, 1, 4>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c); break;
-            case 2: apply_singles<T, 2, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c); break;
-            default: apply_singles<T, 3, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c); break;
+            case 0: apply_keys<T, 0, 4>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
+            case 1: apply_keys<T, 1, 4>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
+            case 2: apply_keys<T, 2, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
+            default: apply_keys<T, 3, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
         }
     }
-    TICK(1, 5);
-    if (n_multi == 0 || DBG(a.dbg, 2)) return;  // block-uniform
-    // keys with several entries: sums in LDS accumulators, as many keys at a time as they hold
-    double* acc = reinterpret_cast<double*>(owner);
-    const u32 B = PA_ACC_DOUBLES / (units * N);
-    for (u32 b0 = 0; b0 < n_multi; b0 += B) {
+    // more lists than the accumulators hold (rows of several KiB): further rounds
+    for (u32 b0 = first_b1; b0 < n_multi; b0 += B) {
         const u32 b1 = b0 + B < n_multi ? b0 + B : n_multi;
         const u32 lo = aux[urep[mrep[b0]]] & 0xFFFFu;
         const u32 hi = b1 < n_multi ? (aux[urep[mrep[b1]]] & 0xFFFFu) : n_elems;
+        __syncthreads();
         for (u32 x = tid; x < (b1 - b0) * units * N; x += PA_BLOCK) acc[x] = 0.0;
         __syncthreads();
-        TICK(1, 6);
         if (on) flat_sum<T>([&](u32 e) { return src(list[e]); }, lown, lo, hi, b0, acc, units, NG, g, c);
         __syncthreads();
-        TICK(1, 7);
         if (on)
             for (u32 l = b0 + g; l < b1; l += NG) {
                 const u32 u = mrep[l];
                 apply(u, urep[u], Acc<T>::load(acc + ((size_t)(l - b0) * units + c) * N));
             }
-        __syncthreads();
-        TICK(1, 8);
     }
 }
 
@@ -825,7 +843,8 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
                                                                ApplyArgs a) {
     extern __shared__ __align__(16) unsigned char pa_lds[];
     __shared__ u64 sums[PA_BLOCK / 64];
-    __shared__ u32 s_nnew, s_sel;
+    __shared__ u32 s_nnew, s_sel, s_sp;
+    __shared__ u32 stk[24];
     u64* lkey = reinterpret_cast<u64*>(pa_lds);
     u32* lref = reinterpret_cast<u32*>(pa_lds + PA_OFF_LREF);
     const u32 tid = threadIdx.x;
@@ -839,42 +858,78 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
         return;
     }
     if (np <= a.cap) {
-        for (u32 i = tid; i < np; i += PA_BLOCK) {
-            lkey[i] = a.ent_key[s + i];
-            lref[i] = a.ent_ref[s + i];
+        uint4 e[PA_ITEMS];
+#pragma unroll
+        for (u32 j = 0; j < PA_ITEMS; ++j) {
+            const u32 i = j * PA_BLOCK + tid;
+            e[j] = a.ent[s + (i < np ? i : 0u)];
+        }
+#pragma unroll
+        for (u32 j = 0; j < PA_ITEMS; ++j) {
+            const u32 i = j * PA_BLOCK + tid;
+            if (i < np) {
+                lkey[i] = ((u64)e[j].y << 32) | e[j].x;
+                lref[i] = e[j].z;
+            }
         }
         __syncthreads();
         apply_pass<T>(t, pa_lds, sums, &s_nnew, grads, psum, ngrad, a, s, np);
     } else {
         // More entries than a pass holds (several keys that are met in most tiles share the
-        // partition): passes over the entries, pass r taking the keys whose hash says r.
-        u32 R = 2;
-        while (np / R > a.cap / 2 && R < 1024u) R <<= 1;
-        for (u32 r = 0; r < R; ++r) {
+        // partition): passes over the entries by hash class. A class that still holds too many is
+        // split in two by the next hash bit, down to 1024 classes; a key has at most one entry per
+        // tile, so only keys that agree in all ten bits could make the last split fail.
+        u32 lgR = 1;
+        while ((np >> lgR) > a.cap / 2 && lgR < 10u) ++lgR;
+        for (u32 r0 = 0; r0 < (1u << lgR); ++r0) {
             __syncthreads();
-            if (tid == 0) s_sel = 0;
+            if (tid == 0) {
+                stk[0] = (lgR << 16) | r0;
+                s_sp = 1;
+            }
             __syncthreads();
-            for (u32 i = tid; i < np; i += PA_BLOCK) {
-                const u64 key = a.ent_key[s + i];
-                if (((u32)(hash64(key) >> 53) & (R - 1u)) == r) {
-                    const u32 pos = atomicAdd(&s_sel, 1u);
-                    if (pos < a.cap) {
-                        lkey[pos] = key;
-                        lref[pos] = a.ent_ref[s + i];
+            while (s_sp) {  // block-uniform: read between barriers
+                const u32 top = stk[s_sp - 1];
+                __syncthreads();
+                if (tid == 0) {
+                    s_sp -= 1;
+                    s_sel = 0;
+                }
+                __syncthreads();
+                const u32 lg = top >> 16, cls = top & 0xFFFFu, mask = (1u << lg) - 1u;
+                for (u32 i = tid; i < np; i += PA_BLOCK) {
+                    const uint4 e = a.ent[s + i];
+                    const u64 key = ((u64)e.y << 32) | e.x;
+                    if (((u32)(hash64(key) >> 53) & mask) == cls) {
+                        const u32 pos = atomicAdd(&s_sel, 1u);
+                        if (pos < a.cap) {
+                            lkey[pos] = key;
+                            lref[pos] = e.z;
+                        }
                     }
                 }
+                __syncthreads();
+                const u32 sel = s_sel;
+                if (sel > a.cap) {
+                    if (lg >= 10u) {  // reported, never silent
+                        if (tid == 0) t.counters[CNT_PART_ERR] = 1u;
+                    } else if (tid == 0) {
+                        stk[s_sp] = ((lg + 1u) << 16) | cls;
+                        stk[s_sp + 1] = ((lg + 1u) << 16) | (cls + (1u << lg));
+                        s_sp += 2;
+                    }
+                } else if (sel) {
+                    apply_pass<T>(t, pa_lds, sums, &s_nnew, grads, psum, ngrad, a, s, sel);
+                }
+                __syncthreads();
             }
-            __syncthreads();
-            const u32 sel = s_sel;
-            if (sel > a.cap) {  // not expected of any hash that spreads keys; reported, never silent
-                if (tid == 0) t.counters[CNT_PART_ERR] = 1u;
-                continue;
-            }
-            if (sel) apply_pass<T>(t, pa_lds, sums, &s_nnew, grads, psum, ngrad, a, s, sel);
         }
     }
     __syncthreads();
-    if (tid == 0) a.new_count[p] = s_nnew;
+    if (tid == 0) {
+        a.new_count[p] = s_nnew;
+        if (s_nnew) t.counters[CNT_ANY_NEW] = 1u;  // (every writer writes the same value)
+    }
 }
 
 // ---- 5. insert ------------------------------------------------------------------------------------
@@ -888,6 +943,10 @@ __global__ __launch_bounds__(PI_BLOCK) void part_insert_kernel(TableDev t, const
     constexpr u32 N = sizeof(T) / 4;
     __shared__ u32 red[PI_BLOCK / 64];
     const u32 p = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    if (!t.counters[CNT_ANY_NEW]) {  // block-uniform: the batch inserted nothing
+        if (p == 0 && tid == 0) publish_rows(t, t.counters[CNT_ENTRY]);
+        return;
+    }
     const u32 mine = new_count[p];
     if (mine == 0 && p != 0) return;  // block-uniform
     const u32 upto = p == 0 ? P : p;
@@ -955,23 +1014,8 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // ---- host side --------------------------------------------------------------------------------
 namespace {
 u32 g_part_cap = PA_CAP;
-u32 g_part_dbg = 0;
 }
-#ifdef PART_TIMING
-extern "C" int32_t pshbm_debug_part_timing(unsigned long long* out) {  // 32 words; the counters restart
-    unsigned long long zero[32] = {};
-    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(g_part_ticks), sizeof zero) != hipSuccess) return 10;
-    if (hipMemcpyToSymbol(HIP_SYMBOL(g_part_ticks), zero, sizeof zero) != hipSuccess) return 10;
-    return 0;
-}
-#endif
-void part_set_pass_capacity(uint32_t entries) {
-#ifdef PART_EXPERIMENT
-    g_part_dbg = entries >> 16;
-    entries &= 0xFFFFu;
-#endif
-    g_part_cap = entries == 0 || entries > PA_CAP ? PA_CAP : entries;
-}
+void part_set_pass_capacity(uint32_t entries) { g_part_cap = entries == 0 || entries > PA_CAP ? PA_CAP : entries; }
 
 bool part_plan(const TableDev& t, size_t n, PartPlan* plan) {
     if (n < PART_MIN_KEYS || n > PART_MAX_KEYS) return false;
@@ -993,10 +1037,8 @@ PartSizes part_sizes(uint32_t dim, size_t n) {
     PartSizes z{};
     const size_t n_tiles = (n + PT_TILE - 1) / PT_TILE;
     const size_t np = n_tiles * PT_TILE;
-    z.stage_key = np * 8;
-    z.stage_ref = np * 4;
-    z.ent_key = np * 8;
-    z.ent_ref = np * 4;
+    z.stage = np * 16;
+    z.ent = np * 16;
     z.counts = n_tiles * PT_MAX_PARTS * 4;
     z.starts = z.counts;
     z.blocktot = n_tiles * (PT_MAX_PARTS / 64) * 4;
@@ -1012,9 +1054,9 @@ PartSizes part_sizes(uint32_t dim, size_t n) {
 hipError_t part_init() {
     hipError_t e;
     if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&part_tile_kernel<float>),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, PT_LDS)) != hipSuccess) return e;
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, PT_LDS_FIXED + PT_MAX_PARTS * 4)) != hipSuccess) return e;
     if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&part_tile_kernel<float4>),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, PT_LDS)) != hipSuccess) return e;
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, PT_LDS_FIXED + PT_MAX_PARTS * 4)) != hipSuccess) return e;
     if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&part_apply_kernel<float>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, PA_LDS)) != hipSuccess) return e;
     if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&part_apply_kernel<float4>),
@@ -1025,33 +1067,31 @@ hipError_t part_init() {
 hipError_t launch_part_tile(const TableDev& t, const PartPlan& pl, const PartBufs& b, const uint64_t* keys,
                             const float* grads, hipStream_t s) {
     if ((t.dim % 4 == 0) && aligned16(grads))
-        part_tile_kernel<float4><<<pl.n_tiles, PT_BLOCK, PT_LDS, s>>>(
-            t, keys, reinterpret_cast<const float4*>(grads), pl.n, pl.P, pl.part_shift, b.stage_key, b.stage_ref,
-            b.counts, b.starts, b.blocktot, b.tile_total, reinterpret_cast<float4*>(b.psum), t.dim / 4, g_part_dbg);
+        part_tile_kernel<float4><<<pl.n_tiles, PT_BLOCK, PT_LDS_FIXED + pl.P * 4, s>>>(
+            t, keys, reinterpret_cast<const float4*>(grads), pl.n, pl.P, pl.part_shift, b.stage, b.counts, b.starts,
+            b.blocktot, b.tile_total, reinterpret_cast<float4*>(b.psum), t.dim / 4);
     else
-        part_tile_kernel<float><<<pl.n_tiles, PT_BLOCK, PT_LDS, s>>>(t, keys, grads, pl.n, pl.P, pl.part_shift,
-                                                                    b.stage_key, b.stage_ref, b.counts, b.starts,
-                                                                    b.blocktot, b.tile_total, b.psum, t.dim,
-                                                                    g_part_dbg);
+        part_tile_kernel<float><<<pl.n_tiles, PT_BLOCK, PT_LDS_FIXED + pl.P * 4, s>>>(t, keys, grads, pl.n, pl.P, pl.part_shift, b.stage,
+                                                                    b.counts, b.starts, b.blocktot, b.tile_total,
+                                                                    b.psum, t.dim);
     return hipGetLastError();
 }
 
 hipError_t launch_part_scan(const PartPlan& pl, const PartBufs& b, hipStream_t s) {
-    part_scan_kernel<<<pl.P / 64, PT_BLOCK, 0, s>>>(b.counts, b.starts, b.blocktot, b.pstart, pl.n_tiles, pl.P);
+    part_scan_kernel<<<pl.P / 64, SC_BLOCK, 0, s>>>(b.counts, b.starts, b.blocktot, b.pstart, pl.n_tiles, pl.P);
     return hipGetLastError();
 }
 
 hipError_t launch_part_scatter(const TableDev& t, const PartPlan& pl, const PartBufs& b, hipStream_t s) {
-    part_scatter_kernel<<<pl.n_tiles, PT_BLOCK, 0, s>>>(t, b.stage_key, b.stage_ref, b.counts, b.tile_total, pl.P,
-                                                        pl.part_shift, b.ent_key, b.ent_ref);
+    part_scatter_kernel<<<pl.n_tiles, PT_BLOCK, 0, s>>>(t, b.stage, b.counts, b.tile_total, pl.P, pl.part_shift, b.ent);
     return hipGetLastError();
 }
 
 hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads, bool insert,
                              hipStream_t s) {
     const bool v4 = (t.dim % 4 == 0) && aligned16(grads);
-    ApplyArgs a{b.ent_key, b.ent_ref, b.pstart, b.new_slot, b.new_count, v4 ? t.dim / 4 : t.dim, insert ? 1 : 0,
-                g_part_cap, g_part_dbg >> 8};
+    ApplyArgs a{b.ent, b.pstart, b.new_slot, b.new_count, v4 ? t.dim / 4 : t.dim, insert ? 1 : 0,
+                g_part_cap};
     if (v4)
         part_apply_kernel<float4><<<pl.P, PA_BLOCK, PA_LDS, s>>>(t, reinterpret_cast<const float4*>(grads),
                                                                  reinterpret_cast<const float4*>(b.psum),

@@ -34,6 +34,7 @@ enum {
     CNT_BADKEY = 4,    // reserved keys met in a batch (skipped)
     CNT_SORT_ERR = 5,  // a sort tile gave up waiting for its predecessor
     CNT_PART_ERR = 6,  // a partition of a push held more entries of one hash class than a pass takes
+    CNT_ANY_NEW = 7,   // the partitioned push that is running has claimed a slot for a new key
     CNT_WORDS = 8
 };
 
@@ -184,19 +185,19 @@ hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long l
 
 // ---- partitioned push (push_part.hip) ---------------------------------------------------------
 // Aggregation and update of a batch of PART_MIN_KEYS .. PART_MAX_KEYS keys without a global sort:
-// tiles of 4096 keys, partitions of about 1024 keys. part_plan says whether a batch qualifies (and
+// tiles of 4096 keys, partitions of about 1024 keys (ranges of home buckets). part_plan says whether a batch qualifies (and
 // how it is cut); part_sizes gives the bytes of each scratch array for batches of up to n keys.
 constexpr size_t PART_MIN_KEYS = 16384, PART_MAX_KEYS = 1u << 22;
 struct PartPlan {
     uint32_t n, n_tiles, P, part_shift;
 };
 struct PartSizes {
-    size_t stage_key, stage_ref, ent_key, ent_ref, counts, starts, blocktot, tile_total, pstart, psum, new_slot,
+    size_t stage, ent, counts, starts, blocktot, tile_total, pstart, psum, new_slot,
         new_count, ngrad;
 };
 struct PartBufs {
-    uint64_t *stage_key, *ent_key;
-    uint32_t *stage_ref, *ent_ref, *counts, *starts, *blocktot, *tile_total, *pstart, *new_slot, *new_count;
+    uint4 *stage, *ent;  // entries {key low, key high, reference, -}: per tile, then per partition
+    uint32_t *counts, *starts, *blocktot, *tile_total, *pstart, *new_slot, *new_count;
     float *psum, *ngrad;
 };
 bool part_plan(const TableDev& t, size_t n, PartPlan* plan);
