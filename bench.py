@@ -6,8 +6,11 @@ through the device-pointer C ABI with every input already resident in HBM. The d
 is the headline configuration ("c2": 100M uint64 keys, dim-16 fp32 rows, plain SGD lr 0.01, 1M-key
 Zipf(1.05) batches, duplicates summed before the update).
 
-Prints ONE JSON line: metric/value (pulled + pushed keys per second), the roofline of the kernel
-that takes the most time, and the same workload timed on the host CPU with the oracle.
+Prints ONE JSON line: metric/value (pulled + pushed keys per second) of the headline
+configuration, the roofline of the kernel that takes the most time per step, the same workload
+timed on the host CPU with the oracle, and -- under "configs" -- the same measurements for the
+other configurations of the benchmark (each on its own table at full size, a shorter run), with
+the load factor and probe-distance histogram of every table.
 """
 import argparse
 import importlib
@@ -48,22 +51,20 @@ KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist"
                    "gather": "gather_slots_kernel", "part_tile": "part_tile_kernel",
                    "part_scan": "part_scan_kernel", "part_scatter": "part_scatter_kernel",
                    "part_apply": "part_apply_kernel", "part_insert": "part_insert_kernel"}
-# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by the factors a plain
-# copy of known size gave), measured on an MI355X; the summaries are under profiles/.
-MEASURED_TRAFFIC_BYTES = {
-    ("c2", "pull"): 191_800_000, ("c2", "locate"): 75_700_000, ("c2", "assign_rows"): 100_000,
-    ("c2", "sort_hist"): 6_400_000, ("c2", "sort_pass"): 26_200_000, ("c2", "segreduce"): 194_800_000,
-    ("c2", "fixup_windows"): 300_000, ("c2", "fixup"): 1_900_000,
-    ("c1", "pull"): 19_200_000,
-    ("c3", "pull"): 694_600_000, ("c3", "locate"): 79_900_000, ("c3", "segreduce"): 739_400_000,
-    ("c4", "pull"): 562_800_000, ("c4", "locate"): 273_200_000, ("c4", "segreduce"): 789_000_000,
-    ("c5", "pull"): 3_185_700_000, ("c5", "segreduce"): 3_744_100_000,
+# HBM bytes per launch as rocprofv3 --pmc counted them on an MI355X (FETCH_SIZE and WRITE_SIZE, each
+# scaled by what the same counter reads for a plain copy of known size): NOT measured by this run.
+# Every figure names the summary under profiles/ it was copied from; a kernel that has changed since
+# must be counted again.
+TRAFFIC_FROM_PROFILES = {
+    # (config, phase): (bytes, summary)
 }
 
 
-def algorithmic_bytes(cfg, phase, k, u):
-    """Bytes of keys, gradients, rows and state one launch must move (probe, sort and scratch
-    traffic excluded): k = keys in the batch, u = distinct keys."""
+def algorithmic_bytes(cfg, phase, k, u, k_alone=None):
+    """Bytes of keys, gradients, rows and state one launch must move (probe, partitioning and
+    scratch traffic excluded): k = keys in the batch, u = distinct keys, k_alone = keys that do
+    not repeat inside their tile of 4096 keys. Over the kernels of a push the figures add up to
+    k * (8 + 4 * dim) + u * 2 * row bytes."""
     d4 = 4 * cfg["dim"]
     r = d4 * STATE_BLOCKS[cfg["opt"]["optimizer"]]
     if phase == "pull":
@@ -72,7 +73,11 @@ def algorithmic_bytes(cfg, phase, k, u):
         return k * 8                        # key read
     if phase == "segreduce":
         return k * d4 + u * 2 * r           # gradient read, row+state read and write
-    return 0                                # sort, fixup: pure overhead
+    if phase == "part_tile":                # keys; the gradient rows of the keys that repeat in their tile
+        return k * 8 + (k - (k_alone if k_alone is not None else k)) * d4
+    if phase == "part_apply":               # the other gradient rows; row+state read and write
+        return (k_alone if k_alone is not None else k) * d4 + u * 2 * r
+    return 0                                # sort, scan, scatter, fix-up, row numbering: pure overhead
 
 
 def build_table(ps, wl, torch, cfg, n_table, seed=0):
@@ -117,15 +122,32 @@ def make_batches(wl, torch, cfg, n_table, n_batches, seed=0):
             pos = torch.randperm(k, device="cuda", generator=gen)[:nf]
             keys[pos] = fresh
         grads = torch.randn(k, cfg["dim"], device="cuda", generator=gen) * cfg["sigma"]
-        out.append((keys.contiguous(), grads.contiguous(), int(torch.unique(keys).numel())))
+        out.append((keys.contiguous(), grads.contiguous(), int(torch.unique(keys).numel()),
+                    keys_alone_in_tile(torch, keys)))
     return out
+
+
+def keys_alone_in_tile(torch, keys, tile=4096):
+    """Keys of the batch that do not repeat inside their tile of `tile` consecutive keys (the
+    partitioned push reads their gradient rows in its apply kernel, the others in its tile kernel)."""
+    k = keys.numel()
+    pad = (-k) % tile
+    x = keys
+    if pad:   # distinct fillers that equal no key of their tile
+        x = torch.cat([keys, torch.arange(pad, device=keys.device, dtype=keys.dtype) - (1 << 62)])
+    x = x.view(-1, tile).sort(dim=1).values
+    same_next = torch.zeros_like(x, dtype=torch.bool)
+    same_next[:, :-1] = x[:, :-1] == x[:, 1:]
+    same_prev = torch.zeros_like(same_next)
+    same_prev[:, 1:] = same_next[:, :-1]
+    return int((~(same_next | same_prev)).sum().item()) - pad
 
 
 def run_steps(t, torch, cfg, batches, out, steps, first=0):
     stream = torch.cuda.current_stream().cuda_stream
     k = cfg["batch"]
     for i in range(first, first + steps):
-        keys, grads, _ = batches[i % len(batches)]
+        keys, grads = batches[i % len(batches)][:2]
         st = t.pull_dev(keys.data_ptr(), k, out.data_ptr(), None, 0, stream)
         if st == 0 and not cfg["pull_only"]:
             st = t.push_dev(keys.data_ptr(), grads.data_ptr(), k, 0, stream)
@@ -231,8 +253,9 @@ def cpu_baseline(cfg, wl, budget_keys):
     o.close()
     return {
         "value": keys_per_step / per_step, "unit": "keys/s", "cores": 1, "kind": "port",
-        "sample": f"{n}-key table (of {cfg['n']}), median of {steps - 1} steps of {k}-key batches, "
-                  f"oracle/ps_oracle.cpp single thread",
+        "sample": f"{n}-key table (of {cfg['n']}: building the full table in a std::unordered_map takes "
+                  f"minutes, this leg is bounded to about 30 s; a smaller table only helps the CPU's caches), "
+                  f"median of {steps - 1} steps of {k}-key batches, oracle/ps_oracle.cpp single thread",
         "sharded": cpu_baseline_sharded(cfg, wl, n, oracle, np),
     }
 
@@ -289,13 +312,132 @@ def cpu_baseline_sharded(cfg, wl, n, oracle, np):
             "sample": f"the same table and batches split over {S} shards by key, one thread per shard"}
 
 
+def table_stats(t):
+    """Load factor and probe-distance histogram of the table (pshbm_get_stats): keys whose bucket
+    lies h buckets past their home bucket, h = 0..14, then 15 and more."""
+    st = t.stats()
+    return {"keys": int(st.size), "slots": int(st.slots), "load_factor": round(st.load_factor, 4),
+            "probe_hist": [int(x) for x in st.probe_hist], "max_probe": int(st.max_probe)}
+
+
+def bulk_slice(ps, t, cfg, max_bytes):
+    """The Dump + Load leg on as large a slice of the table as `max_bytes` of page-locked host memory
+    hold: the first records of the dump sequence (pshbm_iterate) into a pinned buffer, then Load of
+    those records into a second, empty table. Synchronous calls; the rate is record bytes over wall
+    clock, so the whole table would take its record bytes at that rate."""
+    dt = ps.record_dtype(t.value_floats)
+    rows = t.size()
+    n = int(min(rows, max_bytes // dt.itemsize))
+    lib = ps.lib()
+    import ctypes as C
+    rec = ps.pinned_empty(n, dt)                      # page-locking is not timed
+    got = C.c_size_t()
+    t0 = time.perf_counter()
+    st = lib.pshbm_iterate(t._h, 0, n, rec.ctypes.data, C.byref(got))
+    dt_dump = time.perf_counter() - t0
+    assert st == 0 and got.value == n, (st, got.value, t.last_error())
+    t2 = ps.Table(cfg["dim"], capacity=n + 16, max_batch=1 << 20, **cfg["opt"])
+    t0 = time.perf_counter()
+    st = t2.load(rec, ps.LOAD_UNIQUE)
+    dt_load = time.perf_counter() - t0
+    assert st == 0 and t2.size() == n, (st, t2.last_error())
+    t2.close()
+    nbytes = n * dt.itemsize
+    full = rows * dt.itemsize
+    return {"records": n, "of_records": rows, "record_bytes": dt.itemsize, "bytes": nbytes,
+            "dump_ms": round(dt_dump * 1e3, 2), "dump_GBps": round(nbytes / dt_dump / 1e9, 1),
+            "load_ms": round(dt_load * 1e3, 2), "load_GBps": round(nbytes / dt_load / 1e9, 1),
+            "whole_table_dump_s_at_this_rate": round(full / (nbytes / dt_dump), 2),
+            "whole_table_load_s_at_this_rate": round(full / (nbytes / dt_load), 2),
+            "note": "a slice of the table through a page-locked buffer of this size (pshbm_iterate, then "
+                    "pshbm_load into an empty table); PCIe-inclusive by nature, never part of `value`"}
+
+
+def measure(name, args, torch, ps, wl, steps, warmup, headline):
+    """One configuration on its own table at full size: W warm-up steps, K timed steps between two
+    device synchronisations, then the same K steps with HIP events around every kernel launch."""
+    cfg = dict(CONFIGS[name])
+    n_table = (args.table_keys if headline else 0) or cfg["n"]
+    t = build_table(ps, wl, torch, cfg, n_table)
+    batches = make_batches(wl, torch, cfg, n_table, n_batches=8)
+    out = torch.empty(cfg["batch"], cfg["dim"], device="cuda")
+    k = cfg["batch"]
+    keys_per_step = k * (1 if cfg["pull_only"] else 2)
+
+    run_steps(t, torch, cfg, batches, out, warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_steps(t, torch, cfg, batches, out, steps, first=warmup)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / steps
+
+    t.profile_enable(True)
+    run_steps(t, torch, cfg, batches, out, steps, first=warmup)
+    torch.cuda.synchronize()
+    prof = t.profile_read()
+    t.profile_enable(False)
+    u_mean = sum(b[2] for b in batches) / len(batches)
+    alone_mean = sum(b[3] for b in batches) / len(batches)
+    phases = {}
+    for phase, (ms, launches) in prof.items():
+        if launches:
+            avg_ms = ms / launches
+            by = algorithmic_bytes(cfg, phase, k, u_mean, alone_mean)
+            phases[phase] = {"kernel": KERNEL_OF_PHASE[phase], "avg_ms": round(avg_ms, 5), "launches": int(launches),
+                             "ms_per_step": round(ms / steps, 5),
+                             "algorithmic_GBps": round(by / avg_ms / 1e6, 1)}
+    # the kernel that takes the most time per step (all its launches of a step together)
+    dominant = max(phases, key=lambda p: phases[p]["ms_per_step"])
+    achieved = phases[dominant]["algorithmic_GBps"]
+    traffic = TRAFFIC_FROM_PROFILES.get((name, dominant)) if n_table == cfg["n"] else None
+    roofline = {"kernel": KERNEL_OF_PHASE[dominant], "bound": "hbm", "achieved": achieved,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": traffic[0] if traffic else None,
+                "traffic_from_profile": traffic[1] if traffic else None,
+                "avg_ms": phases[dominant]["avg_ms"],
+                "algorithmic_bytes": int(algorithmic_bytes(cfg, dominant, k, u_mean, alone_mean)),
+                "note": "achieved = algorithmic bytes of one launch / its average duration (HIP events on the "
+                        "launch stream, this run); traffic = HBM bytes per launch counted by rocprofv3 --pmc in "
+                        "the run the named summary describes, not in this one"}
+    step_bytes = algorithmic_bytes(cfg, "pull", k, u_mean)
+    if not cfg["pull_only"]:
+        step_bytes += algorithmic_bytes(cfg, "segreduce", k, u_mean) + 8 * k   # = k (8 + 4 dim) + u 2 R
+    res = {
+        "value": keys_per_step * steps / elapsed, "ms_per_step": ms_per_step, "steps": steps, "warmup": warmup,
+        "config": {"workload": cfg["desc"], "table_keys": n_table, "batch": k, "dim": cfg["dim"],
+                   "unique_keys_per_batch": round(u_mean), "keys_alone_in_their_tile": round(alone_mean)},
+        "step_algorithmic_bytes": int(step_bytes),
+        "step_algorithmic_GBps": round(step_bytes / (ms_per_step * 1e6), 1),
+        "step_frac_of_hbm_peak": round(step_bytes / (ms_per_step * 1e6) / HBM_PEAK_GBS, 4),
+        "kernel_ms_per_step": round(sum(p["ms_per_step"] for p in phases.values()), 5),
+        "roofline": roofline,
+        "phases": phases,
+        "table_stats": table_stats(t),
+    }
+    if headline and args.bulk:
+        res["bulk"] = bulk_transfers(ps, t, cfg)
+    if name == "c5" and not args.no_bulk_slice:
+        res["bulk"] = bulk_slice(ps, t, cfg, args.bulk_slice_bytes)
+    if headline and args.scan:
+        res["scan"] = scan_table(ps, t, cfg, n_table)
+    t.close()
+    del out, batches
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
-    ap.add_argument("--table-keys", type=int, default=0, help="override the table size (testing)")
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS),
+                    help="the headline configuration (value, ms_per_step, roofline, cpu_baseline)")
+    ap.add_argument("--only", action="store_true",
+                    help="measure the headline configuration only (profiling runs); by default the other "
+                         "configurations follow, 20 steps each, and are reported under \"configs\"")
+    ap.add_argument("--table-keys", type=int, default=0, help="override the headline table size (testing)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-keys", type=int, default=10_000_000, help="table size of the CPU sample")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -306,8 +448,11 @@ def main():
                          "for-each (count + column sums), for-each under a predicate on a value "
                          "column, erase-if of about a tenth of the keys; reported under \"scan\"")
     ap.add_argument("--bulk", action="store_true",
-                    help="after the steps, also time Dump of the table into page-locked host memory "
-                         "and Load of those records into an empty table; reported under \"bulk\"")
+                    help="after the steps, also time Dump of the whole headline table into page-locked host "
+                         "memory and Load of those records into an empty table; reported under \"bulk\"")
+    ap.add_argument("--bulk-slice-bytes", type=int, default=16 << 30,
+                    help="page-locked bytes of the Dump + Load leg of c5 (a slice of its 215 GB table)")
+    ap.add_argument("--no-bulk-slice", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -316,8 +461,6 @@ def main():
     ps = importlib.import_module("parameter-server_amd")
     wl = importlib.import_module("parameter-server_amd.workload")
     ps.lib()  # fails loudly if the HIP library has not been built
-    cfg = dict(CONFIGS[args.config])
-    n_table = args.table_keys or cfg["n"]
     torch.cuda.set_device(0)
 
     if args.calibration_copy:
@@ -327,69 +470,23 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
-    t = build_table(ps, wl, torch, cfg, n_table)
-    batches = make_batches(wl, torch, cfg, n_table, n_batches=8)
-    out = torch.empty(cfg["batch"], cfg["dim"], device="cuda")
-    k = cfg["batch"]
-    keys_per_step = k * (1 if cfg["pull_only"] else 2)
-
-    # timed region: W warm-up steps, then exactly K steps between two device synchronisations
-    run_steps(t, torch, cfg, batches, out, args.warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_steps(t, torch, cfg, batches, out, args.steps, first=args.warmup)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-    value = keys_per_step * args.steps / elapsed
-
-    # the same K steps again with HIP events around every kernel launch (on the launch stream)
-    t.profile_enable(True)
-    run_steps(t, torch, cfg, batches, out, args.steps, first=args.warmup)
-    torch.cuda.synchronize()
-    prof = t.profile_read()
-    t.profile_enable(False)
-    u_mean = sum(b[2] for b in batches) / len(batches)
-    phases = {}
-    for name, (ms, launches) in prof.items():
-        if launches:
-            avg_ms = ms / launches
-            by = algorithmic_bytes(cfg, name, k, u_mean)
-            phases[name] = {"avg_ms": round(avg_ms, 5), "launches": int(launches),
-                            "algorithmic_GBps": round(by / avg_ms / 1e6, 1)}
-    # the kernel with the longest average launch
-    dominant = max(phases, key=lambda p: phases[p]["avg_ms"])
-    achieved = phases[dominant]["algorithmic_GBps"]
-    roofline = {"kernel": KERNEL_OF_PHASE[dominant], "bound": "hbm", "achieved": achieved,
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dominant)) if not args.table_keys else None,
-                "avg_ms": phases[dominant]["avg_ms"],
-                "algorithmic_bytes": int(algorithmic_bytes(cfg, dominant, k, u_mean))}
-    step_bytes = sum(algorithmic_bytes(cfg, p, k, u_mean) for p in ("pull",) if True)
-    if not cfg["pull_only"]:
-        step_bytes += algorithmic_bytes(cfg, "locate", k, u_mean) + algorithmic_bytes(cfg, "segreduce", k, u_mean)
-
+    head = measure(args.config, args, torch, ps, wl, args.steps, args.warmup, headline=True)
     result = {
         "metric": "pulled+pushed keys/sec on 1 MI355X; achieved HBM GB/s as % of peak",
-        "value": value, "unit": "keys/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "value": head.pop("value"), "unit": "keys/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head.pop("ms_per_step"), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": cfg["desc"], "table_keys": n_table, "batch": k, "dim": cfg["dim"],
-                   "unique_keys_per_batch": round(u_mean)},
-        "step_algorithmic_GBps": round(step_bytes / (ms_per_step * 1e6), 1),
-        "step_frac_of_hbm_peak": round(step_bytes / (ms_per_step * 1e6) / HBM_PEAK_GBS, 4),
-        "roofline": roofline,
-        "phases": phases,
     }
-    if args.bulk:
-        result["bulk"] = bulk_transfers(ps, t, cfg)
-    if args.scan:
-        result["scan"] = scan_table(ps, t, cfg, n_table)
-    t.close()
-    del out, batches
-    torch.cuda.empty_cache()
+    head.pop("steps"), head.pop("warmup")
+    result.update(head)
+    if not args.only:
+        result["configs"] = {}
+        for other in sorted(CONFIGS):
+            if other != args.config:
+                result["configs"][other] = measure(other, args, torch, ps, wl, min(args.steps, 20),
+                                                   min(args.warmup, 3), headline=False)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cfg, wl, args.cpu_keys)
+        result["cpu_baseline"] = cpu_baseline(dict(CONFIGS[args.config]), wl, args.cpu_keys)
     print(json.dumps(result))
 
 
