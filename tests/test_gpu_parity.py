@@ -177,28 +177,31 @@ def test_aggregation_exact_large_batch(ps, orc, n):
     t.close()
 
 
-LOW_MULTIPLICITY = 32
-
-
-def assert_push_parity(gpu, seq, exact, multiplicity):
+def assert_push_parity(gpu, seq, exact, multiplicity=None, report=None):
     """gpu / seq / exact: key-sorted dumps after the same push from the same state, through the
-    kernels, the oracle (sums duplicates sequentially in fp32, the reference's order) and the
-    oracle with exactly rounded sums. Every value must be within RTOL/ATOL of the reference-order
-    result. The one excuse: a key repeated more than LOW_MULTIPLICITY times in the batch, where
-    the order of the fp32 additions alone moves the sum by more than the tolerance (the
-    sequential sum of thousands of terms is itself that far from the exact sum); such a value
-    must then be at least as close to the exactly rounded result as the reference-order one."""
+    kernels, the oracle (sums duplicates sequentially in fp32, the reference's order:
+    pico-ps/operator/SparsePushOperator.h:134-141) and the oracle with exactly rounded sums.
+    Every value must be within RTOL/ATOL of the reference-order result or of the exactly rounded
+    one: the sequential fp32 sum of thousands of terms is itself further than the tolerance from
+    the exact sum, and an implementation that adds in another order cannot (and should not)
+    follow it there. No value is excused. `report` collects how many values needed the second
+    clause and how far both implementations are from the exact result."""
     np.testing.assert_array_equal(gpu["key"], seq["key"])
     np.testing.assert_array_equal(gpu["key"], exact["key"])
     g, s, e = (x["value"].astype(np.float64) for x in (gpu, seq, exact))
-    ok = np.abs(g - s) <= ATOL + RTOL * np.abs(s)
-    if ok.all():
-        return
-    bad_rows = np.unique(np.nonzero(~ok)[0])
-    assert (multiplicity[bad_rows] > LOW_MULTIPLICITY).all(), \
-        "a key of low multiplicity misses the tolerance"
-    closer = np.abs(g - e) <= np.abs(s - e) + ATOL + RTOL * np.abs(e)
-    assert (ok | closer).all(), "a heavily repeated key is further from the exact sum than the reference order"
+    near_seq = np.abs(g - s) <= ATOL + RTOL * np.abs(s)
+    near_exact = np.abs(g - e) <= ATOL + RTOL * np.abs(e)
+    if report is not None:
+        report["values"] = report.get("values", 0) + g.size
+        report["beyond_reference_order_tolerance"] = report.get("beyond_reference_order_tolerance", 0) + int((~near_seq).sum())
+        report["worst_gpu_minus_exact"] = max(report.get("worst_gpu_minus_exact", 0.0), float(np.abs(g - e).max()))
+        report["worst_reference_minus_exact"] = max(report.get("worst_reference_minus_exact", 0.0), float(np.abs(s - e).max()))
+        if multiplicity is not None and (~near_seq).any():
+            rows = np.unique(np.nonzero(~near_seq)[0])
+            report["least_multiplicity_beyond"] = min(report.get("least_multiplicity_beyond", 1 << 60),
+                                                      int(multiplicity[rows].min()))
+    assert (near_seq | near_exact).all(), \
+        "a pushed value is within the tolerance of neither the reference-order nor the exact result"
 
 
 @pytest.mark.parametrize("opt", ["sgd", "adagrad", "ftrl"])
@@ -234,6 +237,8 @@ def test_push_zipf_within_tolerance(ps, orc, wl, opt, dim, s, batch):
         mult = np.zeros(a.size, np.int64)
         mult[np.searchsorted(a["key"], uk)] = cnt
         assert_push_parity(a, b, c, mult)
+        # whatever the multiplicity, the kernels stay within the tolerance of the exact result
+        np.testing.assert_allclose(a["value"], c["value"], rtol=RTOL, atol=ATOL)
         # next step: everyone restarts from the reference-order state
         assert t.set(b["key"], b["value"]) == 0, t.last_error()
         assert x.set(b["key"], b["value"]) == 0
@@ -857,4 +862,41 @@ def test_sort_that_gives_up_applies_nothing(ps, orc, wl):
     assert t.set(keys, vals) == 0 and t.push(q, g) == 0 and t.size() == n_table
     st, rows, hit = t.pull(keys)
     assert not np.array_equal(rows, vals)
+    t.close()
+
+
+def test_c2_shaped_push_against_reference_order_and_exact_sums(ps, orc, wl, capsys):
+    """The headline workload at a table size the oracle reaches: 1M-key Zipf(1.05) batches (the
+    hottest key repeats about 100,000 times) over 10M keys, dim 16, SGD, gradients N(0, 1e-3).
+    Every value must be within 1e-6 / 1e-7 of the exactly rounded result; the report says how many
+    are further than that from the reference-order result, which drifts from the exact one itself."""
+    rng = np.random.default_rng(17)
+    n_table, n, dim = 10_000_000, 1_000_000, 16
+    t = ps.Table(dim, capacity=n_table + 16, max_batch=n, **OPTS["sgd"])
+    r = orc.Oracle(dim, capacity=n_table + 16, **OPTS["sgd"])
+    x = orc.Oracle(dim, capacity=n_table + 16, **OPTS["sgd"])
+    chunk = 1_000_000
+    for start in range(0, n_table, chunk):
+        keys = wl.table_keys_np(start, chunk, seed=11)
+        vals = rng.normal(0, 0.01, (chunk, dim)).astype(np.float32)
+        for b in (t, r, x):
+            assert b.set(keys, vals) == 0
+    report = {}
+    for step in range(2):
+        q = wl.zipf_batch_np(rng, n_table, 1.05, n, seed=11)
+        g = rng.normal(0, 1e-3, (n, dim)).astype(np.float32)
+        assert t.push(q, g) == 0 and r.push(q, g) == 0
+        assert x.push(q, g, orc.PUSH_EXACT_AGGREGATION) == 0
+        uk, cnt = np.unique(q, return_counts=True)
+        # compare the rows the batch touched (the others are bit-identical by construction)
+        a, b, c = (bb.pull(uk)[1] for bb in (t, r, x))
+        dt = np.dtype([("key", "<u8"), ("value", "<f4", (dim,))])
+        pack = lambda rows: np.rec.fromarrays([uk, rows], dtype=dt)
+        assert_push_parity(pack(a), pack(b), pack(c), cnt, report)
+        np.testing.assert_allclose(a, c, rtol=RTOL, atol=ATOL)
+        report["top_multiplicity"] = max(report.get("top_multiplicity", 0), int(cnt.max()))
+        # both oracles restart from the reference-order state, as the table does
+        assert t.set(uk, b) == 0 and x.set(uk, b) == 0
+    with capsys.disabled():
+        print("\nC2-shaped push parity report:", report)
     t.close()
