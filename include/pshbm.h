@@ -63,6 +63,11 @@ extern "C" {
 #define PSHBM_OPT_SGD 1
 #define PSHBM_OPT_ADAGRAD 2
 #define PSHBM_OPT_FTRL 3
+/* The rule of parameter-server_amd/csrc/user_opt.h, compiled into the library: the place of a
+ * maintainer's own init_store_value / store_push_value (SparsePushOperator.h:434-448). The file
+ * declares the state blocks a key carries, their initial value and the step of one element; as
+ * shipped it is SGD with momentum, v = beta*v + g; w -= lr*v (one state block, zero at insertion). */
+#define PSHBM_OPT_USER 4
 
 typedef struct pshbm_config {
     uint32_t struct_size;        /* sizeof(pshbm_config), for forward compatibility */

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libps_oracle.so")
 
 OK, INVALID_CONFIG, OUT_OF_MEMORY, ERROR = 0, 1, 3, 10
-OPT_SUM, OPT_SGD, OPT_ADAGRAD, OPT_FTRL = 0, 1, 2, 3
+OPT_SUM, OPT_SGD, OPT_ADAGRAD, OPT_FTRL, OPT_USER = 0, 1, 2, 3, 4
 PULL_INSERT_ON_MISS = 1
 PUSH_NO_INSERT = 1
 PUSH_EXACT_AGGREGATION = 0x100  # oracle only: float64 sums, rounded once

@@ -67,7 +67,7 @@ constexpr uint64_t KEY_EMPTY = 0xFFFFFFFFFFFFFFFFull;
 constexpr uint64_t KEY_DELETED = 0xFFFFFFFFFFFFFFFEull;
 
 enum { ST_OK = 0, ST_INVALID_CONFIG = 1, ST_OOM = 3, ST_ERROR = 10 };  // Status.h:15-29
-enum { OPT_SUM = 0, OPT_SGD = 1, OPT_ADAGRAD = 2, OPT_FTRL = 3 };
+enum { OPT_SUM = 0, OPT_SGD = 1, OPT_ADAGRAD = 2, OPT_FTRL = 3, OPT_USER = 4 };
 enum { PULL_INSERT_ON_MISS = 1u, PUSH_NO_INSERT = 1u, LOAD_UNIQUE = 1u };
 // Oracle-only push flag: sum duplicates in float64 and round once. This is not what the reference
 // computes; it is the exactly rounded sum, against which tests judge which of two fp32 summation
@@ -106,6 +106,7 @@ uint32_t value_floats(uint32_t dim, int32_t opt) {
         case OPT_SGD: return dim;
         case OPT_ADAGRAD: return 2 * dim;
         case OPT_FTRL: return 3 * dim;
+        case OPT_USER: return 2 * dim;  // the rule shipped in parameter-server_amd/csrc/user_opt.h: one state block
     }
     return 0;
 }
@@ -138,6 +139,8 @@ void init_value(const Config& c, uint64_t key, float* v) {
         for (uint32_t j = 0; j < d; ++j) v[d + j] = c.init_acc;
     if (c.optimizer == OPT_FTRL)
         for (uint32_t j = 0; j < 2 * d; ++j) v[d + j] = 0.0f;
+    if (c.optimizer == OPT_USER)  // momentum starts at rest
+        for (uint32_t j = 0; j < d; ++j) v[d + j] = 0.0f;
 }
 
 // store_push_value (SparsePushOperator.h:448) for the optimizers this repository defines.
@@ -184,6 +187,16 @@ void apply_update(const Config& c, const float* g, float* v) {
                 v[j] = w_new;
                 v[d + j] = z;
                 v[2 * d + j] = n_new;
+            }
+            break;
+        case OPT_USER:  // mirror of the rule shipped as the library's user hook: SGD with momentum,
+                        // v = beta * v + g; w = w - lr * v (heavy ball, Polyak 1964), one state block
+            for (uint32_t j = 0; j < d; ++j) {
+                float carried = c.beta * v[d + j];
+                float vel = carried + g[j];
+                float delta = c.lr * vel;
+                v[d + j] = vel;
+                v[j] = v[j] - delta;
             }
             break;
     }

@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(_HERE, "libpshbm.so")
 CSRC = os.path.join(_HERE, "csrc")
 
 OK, INVALID_CONFIG, INVALID_ID, OUT_OF_MEMORY, ERROR, FATAL = 0, 1, 2, 3, 10, 11
-OPT_SUM, OPT_SGD, OPT_ADAGRAD, OPT_FTRL = 0, 1, 2, 3
+OPT_SUM, OPT_SGD, OPT_ADAGRAD, OPT_FTRL, OPT_USER = 0, 1, 2, 3, 4
 PULL_INSERT_ON_MISS = 1
 PUSH_NO_INSERT = 1
 PUSH_ASSUME_UNIQUE = 2

@@ -17,6 +17,7 @@
 #include <vector>
 
 #include "table.h"
+#include "user_opt.h"
 
 using namespace pshbm;
 
@@ -807,6 +808,7 @@ uint32_t pshbm_value_floats(uint32_t dim, int32_t optimizer) {
         case PSHBM_OPT_SGD: return dim;
         case PSHBM_OPT_ADAGRAD: return 2 * dim;
         case PSHBM_OPT_FTRL: return 3 * dim;
+        case PSHBM_OPT_USER: return (1 + pshbm_user::STATE_BLOCKS) * dim;
     }
     return 0;
 }
@@ -878,8 +880,8 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     d.dim = cfg->dim;
     d.vf = vf;
     d.stride_f = (uint32_t)round_up(vf, 4);
-    d.opt = OptParams{cfg->optimizer, cfg->lr, cfg->init_acc, cfg->alpha, cfg->beta, cfg->l1, cfg->l2,
-                      cfg->init_range};
+    d.opt = OptParams{cfg->optimizer, (int32_t)(vf / cfg->dim) - 1, cfg->lr, cfg->init_acc, cfg->alpha, cfg->beta,
+                      cfg->l1, cfg->l2, cfg->init_range};
     t->slots_bytes = nb * 64;
     t->rows_bytes = max_rows * d.stride_f * 4;
     t->keys_bytes = max_rows * 8;
@@ -1743,7 +1745,7 @@ int32_t pshbm_set_hyperparameters(pshbm_table* t, const pshbm_hyperparameters* h
     t->cfg.beta = hp->beta;
     t->cfg.l1 = hp->l1;
     t->cfg.l2 = hp->l2;
-    t->d.opt = OptParams{t->cfg.optimizer, hp->lr, hp->init_acc, hp->alpha, hp->beta, hp->l1, hp->l2,
+    t->d.opt = OptParams{t->cfg.optimizer, t->d.opt.states, hp->lr, hp->init_acc, hp->alpha, hp->beta, hp->l1, hp->l2,
                          t->cfg.init_range};
     return PSHBM_OK;
 }

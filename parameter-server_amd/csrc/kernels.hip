@@ -296,7 +296,7 @@ __device__ __forceinline__ void apply_runs(const TableDev& t, const T* s_val, co
                                            u32 g, u32 c, bool lane_on, u32 lp_full, u32 units,
                                            u32 col) {
     constexpr int N = sizeof(T) / 4;
-    constexpr int STATES = KIND <= 1 ? 0 : KIND - 1;
+    constexpr int STATES = states_of<KIND>();
     T* rows = reinterpret_cast<T*>(t.rows);
     const u32 stride_units = t.stride_f / N;
     for (u32 j0 = 0; j0 < nruns; j0 += FB * P) {
@@ -494,8 +494,12 @@ __global__ __launch_bounds__(SEG_BLOCK) void segreduce_kernel(
             apply_runs<T, 2, SEG_ROUNDS / 2>(t, s_val, s_row, s_aux, s_start, nruns, P, g, c, lane_on,
                                              lp_full, units, col);
             break;
-        default:
+        case 3:
             apply_runs<T, 3, SEG_ROUNDS / 4>(t, s_val, s_row, s_aux, s_start, nruns, P, g, c, lane_on,
+                                             lp_full, units, col);
+            break;
+        default:
+            apply_runs<T, 4, SEG_ROUNDS / 4>(t, s_val, s_row, s_aux, s_start, nruns, P, g, c, lane_on,
                                              lp_full, units, col);
             break;
     }

@@ -568,7 +568,7 @@ __device__ __forceinline__ void apply_keys(const TableDev& t, unsigned char* lds
                                            const T* __restrict__ psum, T* __restrict__ ngrad, u32 s, u32 U, u32 units,
                                            u32 NG, u32 g, u32 c, const double* acc, u32 n_summed) {
     constexpr u32 N = sizeof(T) / 4;
-    constexpr int STATES = KIND <= 1 ? 0 : KIND - 1;
+    constexpr int STATES = states_of<KIND>();
     const u32* cnt = reinterpret_cast<const u32*>(lds + PA_OFF_CNT);
     const u32* aux = reinterpret_cast<const u32*>(lds + PA_OFF_AUX);
     const u32* urow = reinterpret_cast<const u32*>(lds + PA_OFF_LREF);
@@ -816,7 +816,8 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
             case 0: apply_keys<T, 0, 4>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
             case 1: apply_keys<T, 1, 4>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
             case 2: apply_keys<T, 2, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
-            default: apply_keys<T, 3, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
+            case 3: apply_keys<T, 3, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
+            default: apply_keys<T, 4, 2>(t, lds, grads, psum, ngrad, s, U, units, NG, g, c, acc, first_b1); break;
         }
     }
     // more lists than the accumulators hold (rows of several KiB): further rounds
@@ -1001,8 +1002,8 @@ __global__ __launch_bounds__(PI_BLOCK) void part_insert_kernel(TableDev t, const
             }
             opt_step_n<(int)N>(t.opt, gp, wp, ap, bp);
             r[c] = wv;
-            if (t.opt.kind >= 2) r[units + c] = av;
-            if (t.opt.kind == 3) r[2 * units + c] = bv;
+            if (t.opt.states >= 1) r[units + c] = av;
+            if (t.opt.states >= 2) r[2 * units + c] = bv;
         }
     }
 }

@@ -5,6 +5,7 @@
 
 #include "table.h"
 #include "probe.h"
+#include "user_opt.h"
 
 namespace pshbm {
 
@@ -32,10 +33,21 @@ __device__ __forceinline__ void publish_rows(const TableDev& t, u32 rows) {
                            __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// state blocks of each optimizer, for code specialised by KIND
+template <int KIND>
+__host__ __device__ constexpr int states_of() {
+    return KIND <= 1 ? 0 : KIND == 2 ? 1 : KIND == 3 ? 2 : pshbm_user::STATE_BLOCKS;
+}
+__device__ __forceinline__ pshbm_user::Hyper user_hyper(const OptParams& o) {
+    return pshbm_user::Hyper{o.lr, o.init_acc, o.alpha, o.beta, o.l1, o.l2};
+}
+
 // float f of the value a key starts with: weights, then optimizer state
 __device__ __forceinline__ float init_float(const TableDev& t, u64 key, u32 f) {
     if (f < t.dim) return t.opt.init_range != 0.0f ? init_weight(t.opt.init_range, key, f) : 0.0f;
-    return t.opt.kind == 2 /*ADAGRAD*/ ? t.opt.init_acc : 0.0f;
+    if (t.opt.kind == 2 /*ADAGRAD*/) return t.opt.init_acc;
+    if (t.opt.kind == 4 /*USER*/) return pshbm_user::init_state(user_hyper(t.opt), (int)(f / t.dim) - 1);
+    return 0.0f;
 }
 // the weights a pull answers for a key that is not stored (init_store_value + fetch_pull_value of
 // pico-ps/operator/SparsePullOperator.h:217,226), column unit c of T
@@ -65,6 +77,8 @@ __device__ __forceinline__ void opt_step(const OptParams& o, float g, float& w, 
         float step = num / sqrtf(nn);
         s1 = nn;
         w = w - step;
+    } else if constexpr (KIND == 4) {  // USER: user_opt.h
+        pshbm_user::step(user_hyper(o), g, w, s1, s2);
     } else {  // FTRL: s1 = z, s2 = n
         float gg = g * g;
         float n_new = s2 + gg;
@@ -103,9 +117,13 @@ __device__ __forceinline__ void opt_step_n(const OptParams& o, const float* g, f
 #pragma unroll
             for (int e = 0; e < N; ++e) opt_step<2>(o, g[e], w[e], s1[e], s2[e]);
             break;
-        default:
+        case 3:
 #pragma unroll
             for (int e = 0; e < N; ++e) opt_step<3>(o, g[e], w[e], s1[e], s2[e]);
+            break;
+        default:
+#pragma unroll
+            for (int e = 0; e < N; ++e) opt_step<4>(o, g[e], w[e], s1[e], s2[e]);
             break;
     }
 }
@@ -116,11 +134,11 @@ __device__ __forceinline__ void finalize(const TableDev& t, u32 row, u32 col, u3
     constexpr int N = sizeof(T) / 4;
     if (row >= t.max_rows) return;
     T* r = reinterpret_cast<T*>(t.rows + (u64)row * t.stride_f);
-    const int kind = t.opt.kind;
+    const int states = t.opt.states;
     T wv = r[col];
     T av = vzero(T()), bv = vzero(T());
-    if (kind >= 2) av = r[units + col];
-    if (kind == 3) bv = r[2 * units + col];
+    if (states >= 1) av = r[units + col];
+    if (states >= 2) bv = r[2 * units + col];
     float* gp = reinterpret_cast<float*>(&g);
     float* wp = reinterpret_cast<float*>(&wv);
     float* ap = reinterpret_cast<float*>(&av);
@@ -128,8 +146,8 @@ __device__ __forceinline__ void finalize(const TableDev& t, u32 row, u32 col, u3
     opt_step_n<N>(t.opt, gp, wp, ap, bp);
     if (t.dirty && col == 0) t.dirty[row] = 1;
     r[col] = wv;
-    if (kind >= 2) r[units + col] = av;
-    if (kind == 3) r[2 * units + col] = bv;
+    if (states >= 1) r[units + col] = av;
+    if (states >= 2) r[2 * units + col] = bv;
 }
 
 }  // namespace pshbm

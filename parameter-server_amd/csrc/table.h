@@ -39,7 +39,8 @@ enum {
 };
 
 struct OptParams {
-    int32_t kind;  // PSHBM_OPT_*
+    int32_t kind;    // PSHBM_OPT_*
+    int32_t states;  // blocks of dim floats after the weights: 0 SUM / SGD, 1 ADAGRAD, 2 FTRL, USER as user_opt.h says
     float lr, init_acc, alpha, beta, l1, l2;
     float init_range;  // weights of a new key: 0, or uniform in [-init_range, init_range) by init_weight()
 };

@@ -31,7 +31,7 @@
 
 namespace pshbm_host {
 
-// op_config keys of an HBM table: dim, optimizer (sum|sgd|adagrad|ftrl), lr, init_acc, alpha, beta,
+// op_config keys of an HBM table: dim, optimizer (sum|sgd|adagrad|ftrl|user), lr, init_acc, alpha, beta,
 // l1, l2, hbm_table.expected_max_items, hbm_table.grow_limit, hbm_table.max_load_factor,
 // hbm_table.max_batch, hbm_table.track_increment, hbm_table.init_range, read_only, device. The learning rate lives in the operator config, as pico-ps/operator/Operator.h:55 expects.
 inline pshbm_config table_config(const Configure& c) {
@@ -41,7 +41,8 @@ inline pshbm_config table_config(const Configure& c) {
     cfg.dim = (uint32_t)c.number("dim", 0);
     const std::string opt = c.str("optimizer", "sum");
     cfg.optimizer = opt == "sgd" ? PSHBM_OPT_SGD : opt == "adagrad" ? PSHBM_OPT_ADAGRAD
-                  : opt == "ftrl" ? PSHBM_OPT_FTRL : opt == "sum" ? PSHBM_OPT_SUM : -1;
+                  : opt == "ftrl" ? PSHBM_OPT_FTRL : opt == "user" ? PSHBM_OPT_USER
+                  : opt == "sum" ? PSHBM_OPT_SUM : -1;
     cfg.lr = (float)c.number("lr", 0.0);
     cfg.init_acc = (float)c.number("init_acc", 0.0);
     cfg.alpha = (float)c.number("alpha", 0.0);

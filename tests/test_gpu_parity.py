@@ -18,6 +18,7 @@ OPTS = {
     "sgd": dict(optimizer=1, lr=0.01),
     "adagrad": dict(optimizer=2, lr=0.05, init_acc=0.1),
     "ftrl": dict(optimizer=3, alpha=0.05, beta=1.0, l1=1e-4, l2=1e-5),
+    "user": dict(optimizer=4, lr=0.05, beta=0.9),   # the rule of csrc/user_opt.h: SGD with momentum
 }
 
 
@@ -108,7 +109,7 @@ def test_pull_insert_on_miss(ps, orc, wl, dim):
     t.close(), t2.close()
 
 
-@pytest.mark.parametrize("opt", ["sum", "sgd", "adagrad", "ftrl"])
+@pytest.mark.parametrize("opt", ["sum", "sgd", "adagrad", "ftrl", "user"])
 @pytest.mark.parametrize("dim", [1, 3, 8, 16, 64, 128, 260])
 def test_push_unique_keys_bit_exact(ps, orc, wl, opt, dim):
     """With distinct keys there is nothing to aggregate: every value must match bit for bit."""
@@ -204,7 +205,7 @@ def assert_push_parity(gpu, seq, exact, multiplicity=None, report=None):
         "a pushed value is within the tolerance of neither the reference-order nor the exact result"
 
 
-@pytest.mark.parametrize("opt", ["sgd", "adagrad", "ftrl"])
+@pytest.mark.parametrize("opt", ["sgd", "adagrad", "ftrl", "user"])
 @pytest.mark.parametrize("dim,s", [(16, 1.05), (64, 1.2), (8, 1.1), (128, 1.1)])
 @pytest.mark.parametrize("batch", [30000, 800, 450])  # 450: the one-launch push
 def test_push_zipf_within_tolerance(ps, orc, wl, opt, dim, s, batch):

@@ -12,6 +12,7 @@ OPTS = {
     "sgd": dict(optimizer=1, lr=0.01),
     "adagrad": dict(optimizer=2, lr=0.05, init_acc=0.1),
     "ftrl": dict(optimizer=3, alpha=0.05, beta=1.0, l1=1e-4, l2=1e-5),
+    "user": dict(optimizer=4, lr=0.05, beta=0.9),   # the rule of csrc/user_opt.h: SGD with momentum
 }
 
 
@@ -41,9 +42,13 @@ def fill(t, r, wl, rng, n_table, opt, dim, seed):
     return keys
 
 
+def test_value_floats_of_the_user_rule(ps, orc):
+    assert ps.value_floats(8, ps.OPT_USER) == orc.lib().pso_value_floats(8, orc.OPT_USER) == 16
+
+
 @pytest.mark.parametrize("opt,dim,s", [("sgd", 16, 1.05), ("adagrad", 64, 1.2), ("ftrl", 8, 1.1),
                                        ("adagrad", 128, 1.1), ("sgd", 3, 1.3), ("ftrl", 260, 1.1),
-                                       ("sum", 1, 1.5)])
+                                       ("sum", 1, 1.5), ("user", 16, 1.1), ("user", 6, 1.2)])
 def test_zipf_batches_with_fresh_keys(ps, orc, wl, opt, dim, s):
     """Exact aggregation in the oracle (float64 sums, rounded once): the kernels add in double
     precision too, so the tolerance only covers the rounding of the tiles' partial sums."""

@@ -141,3 +141,29 @@ def test_aggregation_is_sequential_input_order_sum(orc):
     uk, us = orc.aggregate(2, keys, grads)
     np.testing.assert_array_equal(us[:, 0], uk.astype(np.float32) * 3)
     np.testing.assert_array_equal(us[:, 1], 3)
+
+
+def test_user_rule_momentum_hand_computed(orc):
+    """The rule shipped as the library's user hook (parameter-server_amd/csrc/user_opt.h), which the
+    oracle mirrors: SGD with momentum, v = beta * v + g; w = w - lr * v. Parity unpinned by the
+    reference (its update rule is user code); pinned by hand-computed steps, the closed form of a
+    constant gradient, and the identity beta = 0 => plain SGD."""
+    kw = dict(lr=0.1, beta=0.9)
+    v = one(orc, orc.OPT_USER, 1.0, 0.5, state=[0.25], **kw)
+    assert v[1] == pytest.approx(0.9 * 0.25 + 0.5, rel=1e-7)           # v = 0.725
+    assert v[0] == pytest.approx(1.0 - 0.1 * 0.725, rel=1e-7)          # w = 0.9275
+    # a fresh key starts at rest; n pushes of a constant g: v_n = g (1 - beta^n) / (1 - beta)
+    o = orc.Oracle(1, orc.OPT_USER, capacity=4, **kw)
+    w, vel = 0.0, 0.0
+    for n in range(1, 6):
+        assert o.push(K, np.array([[0.2]], np.float32)) == 0
+        vel = 0.9 * vel + 0.2
+        w -= 0.1 * vel
+        got = o.dump()[1]["value"][0]
+        assert got[1] == pytest.approx(0.2 * (1 - 0.9 ** n) / (1 - 0.9), rel=1e-6)
+        assert got[0] == pytest.approx(w, rel=1e-6)
+    # beta = 0: the weight follows plain SGD bit for bit
+    a = one(orc, orc.OPT_USER, 0.3, -0.7, state=[123.0], lr=0.05, beta=0.0)
+    b = one(orc, orc.OPT_SGD, 0.3, -0.7, lr=0.05)
+    assert a[0] == b[0] and a[1] == np.float32(-0.7)
+    assert orc.lib().pso_value_floats(8, orc.OPT_USER) == 16
