@@ -49,7 +49,6 @@ KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist"
                    "assign_rows": "assign_rows_kernel", "update_unique": "update_unique_kernel",
                    "push_small": "push_small_kernel",
                    "gather": "gather_slots_kernel", "part_tile": "part_tile_kernel",
-                   "part_scan": "part_scan_kernel", "part_scatter": "part_scatter_kernel",
                    "part_apply": "part_apply_kernel", "part_insert": "part_insert_kernel"}
 # HBM bytes per launch as rocprofv3 --pmc counted them on an MI355X (FETCH_SIZE and WRITE_SIZE, each
 # scaled by what the same counter reads for a plain copy of known size): NOT measured by this run.

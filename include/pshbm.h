@@ -373,11 +373,9 @@ int32_t pshbm_get_stats(pshbm_table* t, pshbm_stats* out);
 #define PSHBM_PHASE_ASSIGN_ROWS 9   /* rows for the slots an inserting operation claimed */
 #define PSHBM_PHASE_PUSH_SMALL 10   /* a whole push of a small batch in one launch */
 #define PSHBM_PHASE_PART_TILE 11    /* partitioned push: repeats inside a tile pre-summed, entries staged */
-#define PSHBM_PHASE_PART_SCAN 12    /* partitioned push: where each tile's entries go */
-#define PSHBM_PHASE_PART_SCATTER 13 /* partitioned push: entries moved into partition order */
-#define PSHBM_PHASE_PART_APPLY 14   /* partitioned push: one probe, sum and update per distinct key */
-#define PSHBM_PHASE_PART_INSERT 15  /* partitioned push: rows for the keys it inserted */
-#define PSHBM_PHASES 16
+#define PSHBM_PHASE_PART_APPLY 12   /* partitioned push: one probe, sum and update per distinct key */
+#define PSHBM_PHASE_PART_INSERT 13  /* partitioned push: rows for the keys it inserted */
+#define PSHBM_PHASES 14
 typedef struct pshbm_profile {
     double ms[PSHBM_PHASES];
     uint64_t launches[PSHBM_PHASES];

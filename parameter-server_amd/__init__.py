@@ -37,8 +37,7 @@ SYMBOLS = [
     "pshbm_push_dev_noalloc", "pshbm_debug_sort_spin_limit", "pshbm_debug_part_pass_capacity",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
-          "fixup_windows", "assign_rows", "push_small", "part_tile", "part_scan", "part_scatter", "part_apply",
-          "part_insert"]
+          "fixup_windows", "assign_rows", "push_small", "part_tile", "part_apply", "part_insert"]
 
 
 class Config(C.Structure):
@@ -133,7 +132,7 @@ def update(op, first_column, n_columns, a, b):
 
 
 class Profile(C.Structure):
-    _fields_ = [("ms", C.c_double * 16), ("launches", C.c_uint64 * 16)]
+    _fields_ = [("ms", C.c_double * len(PHASES)), ("launches", C.c_uint64 * len(PHASES))]
 
 
 class PshbmError(RuntimeError):

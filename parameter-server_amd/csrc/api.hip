@@ -205,8 +205,7 @@ struct pshbm_table {
     DevBuf ws_slot, ws_row, ws_idx, ws_srow, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wrow, ws_wval, ws_won;
     unsigned won_parity = 0;  // which half of ws_won the next inserting operation counts into
     // scratch of the partitioned push (batches of PART_MIN_KEYS keys and more)
-    DevBuf pt_stage, pt_ent, pt_counts, pt_starts, pt_blocktot, pt_tile_total,
-        pt_pstart, pt_psum, pt_new_slot, pt_new_count, pt_ngrad;
+    DevBuf pt_stage, pt_starts, pt_pstart, pt_psum, pt_new_slot, pt_new_count, pt_ngrad;
     size_t part_keys = 0;       // batch size those arrays serve
 
     // staging of the host-pointer entry points
@@ -389,11 +388,7 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
         const size_t pk = std::min(cap, PART_MAX_KEYS);
         const PartSizes z = part_sizes(t->d.dim, pk);
         ST_TRY(ensure(t, t->pt_stage, z.stage));
-        ST_TRY(ensure(t, t->pt_ent, z.ent));
-        ST_TRY(ensure(t, t->pt_counts, z.counts));
         ST_TRY(ensure(t, t->pt_starts, z.starts));
-        ST_TRY(ensure(t, t->pt_blocktot, z.blocktot));
-        ST_TRY(ensure(t, t->pt_tile_total, z.tile_total));
         ST_TRY(ensure(t, t->pt_pstart, z.pstart));
         ST_TRY(ensure(t, t->pt_psum, z.psum));
         ST_TRY(ensure(t, t->pt_new_slot, z.new_slot));
@@ -565,11 +560,7 @@ Workspace table_workspace(pshbm_table* t) {
     w.part_keys = t->part_keys;
     if (t->part_keys) {
         w.part.stage = static_cast<uint4*>(t->pt_stage.p);
-        w.part.ent = static_cast<uint4*>(t->pt_ent.p);
-        w.part.counts = static_cast<uint32_t*>(t->pt_counts.p);
         w.part.starts = static_cast<uint32_t*>(t->pt_starts.p);
-        w.part.blocktot = static_cast<uint32_t*>(t->pt_blocktot.p);
-        w.part.tile_total = static_cast<uint32_t*>(t->pt_tile_total.p);
         w.part.pstart = static_cast<uint32_t*>(t->pt_pstart.p);
         w.part.psum = static_cast<float*>(t->pt_psum.p);
         w.part.new_slot = static_cast<uint32_t*>(t->pt_new_slot.p);
@@ -603,8 +594,6 @@ int32_t push_with(pshbm_table* t, const Workspace& w, const uint64_t* d_keys, co
     if (!unique && !checked && n <= w.part_keys && part_plan(t->d, n, &pl)) {
         *used_part = true;
         HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_TILE, launch_part_tile(t->d, pl, w.part, d_keys, d_grads, s));
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_SCAN, launch_part_scan(pl, w.part, s));
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_SCATTER, launch_part_scatter(t->d, pl, w.part, s));
         HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_APPLY, launch_part_apply(t->d, pl, w.part, d_grads, insert, s));
         if (insert) HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_INSERT, launch_part_insert(t->d, pl, w.part, d_grads, s));
         return PSHBM_OK;
@@ -697,8 +686,7 @@ void destroy_impl(pshbm_table* t) {
     DevBuf* bufs[] = {&t->ws_slot, &t->ws_row, &t->ws_idx,  &t->ws_srow, &t->ws_sidx, &t->ws_sort, &t->ws_hdr,
                       &t->ws_pval, &t->ws_wrow, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_raw,
                       &t->ms_dead, &t->ms_tiles, &t->ms_lists, &t->ms_fe,
-                      &t->pt_stage, &t->pt_ent, &t->pt_counts, &t->pt_starts,
-                      &t->pt_blocktot, &t->pt_tile_total, &t->pt_pstart, &t->pt_psum, &t->pt_new_slot, &t->pt_new_count,
+                      &t->pt_stage, &t->pt_starts, &t->pt_pstart, &t->pt_psum, &t->pt_new_slot, &t->pt_new_count,
                       &t->pt_ngrad,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)

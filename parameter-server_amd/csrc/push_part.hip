@@ -3,21 +3,23 @@
 // of :245-268).
 //
 // The batch is cut into tiles of 4096 keys and the key space into P partitions, a partition being a
-// range of home buckets of the hash array. Five launches:
+// range of home buckets of the hash array. Three launches:
 //   1. part_tile_kernel     a workgroup per tile: finds the keys that repeat inside the tile (a hash
 //                           table in LDS), adds up their gradient rows into one pre-summed row per
 //                           key, and leaves one entry {key, reference} per distinct key of the tile,
-//                           grouped by partition, in the tile's staging block; a reference is the
-//                           batch index of the gradient row or the number of a pre-summed row.
-//   2. part_scan_kernel     where each (tile, partition) segment goes in the partitioned entry array.
-//   3. part_scatter_kernel  moves the entries there.
-//   4. part_apply_kernel    a workgroup per partition: groups the partition's entries by key (LDS hash
-//                           table again; a key has at most one entry per tile, so the hottest key of
-//                           a batch is a list of a few hundred references, not of a hundred thousand),
-//                           probes the table ONCE per distinct key, adds up each key's rows and takes
-//                           the optimizer step. A key that is not stored claims a slot; its summed
-//                           gradient is parked for the last launch.
-//   5. part_insert_kernel   numbers the new keys densely (prefix over the partitions' counts),
+//                           grouped by partition, in the tile's staging block, with the place where
+//                           each partition's entries start in the block; a reference is the batch
+//                           index of the gradient row or the number of a pre-summed row.
+//   2. part_apply_kernel    a workgroup per partition: collects the partition's entries from the
+//                           staging blocks of all tiles (the tiles' start words of its partition and
+//                           of the next give every segment, and their sum the number of entries in
+//                           lower partitions: no scan launch, no copy into partition order), groups
+//                           them by key (LDS hash table again; a key has at most one entry per tile,
+//                           so the hottest key of a batch is a list of a few hundred references, not
+//                           of a hundred thousand), probes the table ONCE per distinct key, adds up
+//                           each key's rows and takes the optimizer step. A key that is not stored
+//                           claims a slot; its summed gradient is parked for the last launch.
+//   3. part_insert_kernel   numbers the new keys densely (prefix over the partitions' counts),
 //                           initialises their rows and takes their step.
 // Sums are accumulated in double precision and rounded to fp32 once per tile and once per key: the
 // result does not depend on the order in which a key's rows are met beyond the last bit of a
@@ -35,10 +37,10 @@ namespace {
 using u16 = uint16_t;
 
 constexpr u32 PT_TILE = 4096, PT_BLOCK = 1024, PT_ITEMS = PT_TILE / PT_BLOCK;
-constexpr u32 SC_BLOCK = 1024;                // threads of the scan kernel
 constexpr u32 PT_HT = 2 * PT_TILE;            // slots of a tile's LDS hash table
 constexpr u32 PT_MAX_MULTI = PT_TILE / 2;     // pre-summed rows a tile can produce
-constexpr u32 PT_ACC_DOUBLES = PT_TILE;       // accumulators: the room of the tile's key array (32 KiB)
+// accumulators: the room of the tile's key array, of its hash table and of half its counts (72 KiB)
+constexpr u32 PT_ACC_DOUBLES = (PT_TILE * 8 + PT_HT * 4 + (PT_TILE - PT_MAX_MULTI) * 4) / 8;
 constexpr u32 REF_PSUM = 0x80000000u;         // reference to a pre-summed row
 constexpr u32 NONE32 = 0xFFFFFFFFu;
 constexpr u32 PA_BLOCK = 512, PA_ITEMS = 4, PA_CAP = PA_BLOCK * PA_ITEMS;  // entries a partition pass holds
@@ -202,7 +204,7 @@ constexpr u32 PT_LDS_FIXED = PT_OFF_HIST;  // 114688, then one word per partitio
 template <typename T>
 __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
     TableDev t, const u64* __restrict__ keys, const T* __restrict__ grads, u32 n, u32 P, u32 part_shift,
-    uint4* __restrict__ stage, u32* __restrict__ counts, u32* __restrict__ starts, u32* __restrict__ blocktot, u32* __restrict__ tile_total, T* __restrict__ psum, u32 units) {
+    uint4* __restrict__ stage, u32* __restrict__ starts, T* __restrict__ psum, u32 units) {
     extern __shared__ __align__(16) unsigned char pt_lds[];
     u64* lkey = reinterpret_cast<u64*>(pt_lds);
     u32* owner = reinterpret_cast<u32*>(pt_lds + PT_OFF_OWNER);
@@ -267,7 +269,7 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
     u64 tot = 0;
     const u64 ex = block_scan_excl<PT_BLOCK>(((u64)my_len << 32) | my_multi, tid, sums, &tot);
     const u32 n_multi = (u32)tot, n_elems = (u32)(tot >> 32);
-    u32* mrep = owner;  // the hash table is done with
+    u32* mrep = cnt + (PT_TILE - PT_MAX_MULTI);  // (the counts have been read: barriers of the scan since)
     {
         u32 mr = (u32)ex, lo = (u32)(ex >> 32);
 #pragma unroll
@@ -298,7 +300,8 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
     __syncthreads();
 
     // Pre-summed rows of the keys that repeat, as many lists per round as the accumulators hold
-    // (the room of the key array, which nobody reads any more). The rows of the first round are
+    // (the room of the key array, the hash table and the first half of the counts, which nobody
+    // reads any more). The rows of the first round are
     // requested now and added up after the staging block is written: their latency covers that.
     double* acc = reinterpret_cast<double*>(pt_lds);
     const u32 G = units;  // lanes per row (the host admits units <= PT_BLOCK)
@@ -325,8 +328,9 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
         pv[k] = tile_grads[(size_t)q * units + (on ? c : 0u)];
     }
     {
-        // thread x owns PP consecutive partitions (P is a power of two, at least 64): their counts,
-        // where their entries start in the staging block, and the count of each block of 64
+        // thread x owns PP consecutive partitions (P is a power of two, at least 64): where their
+        // entries start in the staging block -- starts[tile][p], P + 1 words per tile, the last one
+        // the tile's entry count
         const u32 PP = P > PT_BLOCK ? P / PT_BLOCK : 1u;
         u32 cc[PT_MAX_PARTS / PT_BLOCK];
         u32 local = 0;
@@ -338,17 +342,14 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
         }
         u64 all = 0;
         u32 run = (u32)block_scan_excl<PT_BLOCK>(local, tid, sums, &all);
-        if (tid == 0) tile_total[tile] = (u32)all;
-        u32 blk = local;
-        for (u32 off = 1; off < 64u / PP; off <<= 1) blk += __shfl_xor(blk, (int)off);
-        if ((tid & (64u / PP - 1u)) == 0 && tid * PP < P) blocktot[(size_t)tile * (P / 64u) + tid * PP / 64u] = blk;
+        u32* my_starts = starts + (size_t)tile * (P + 1u);
+        if (tid == 0) my_starts[P] = (u32)all;
 #pragma unroll
         for (u32 x = 0; x < PT_MAX_PARTS / PT_BLOCK; ++x) {
             const u32 p = tid * PP + x;
             if (x < PP && p < P) {
                 hist[p] = run;
-                counts[(size_t)tile * P + p] = cc[x];
-                starts[(size_t)tile * P + p] = run;
+                my_starts[p] = run;
                 run += cc[x];
             }
         }
@@ -393,149 +394,7 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
     }
 }
 
-// ---- 2. scan ------------------------------------------------------------------------------------
-// counts[tile][p] becomes delta[tile][p] = (position of the tile's first entry of partition p in the
-// partitioned array) - starts[tile][p], so that entry j of the tile's staging block goes to
-// delta + j; pstart[p] = first entry of partition p. A workgroup owns a block of 64 partitions
-// (lane = partition) over all tiles, which its 16 wavefronts split into consecutive parts; what the
-// lower blocks hold it adds up from the per-tile block counts the tile kernel left (no atomic
-// additions anywhere: additions to one address from all over the device are resolved one by one).
-__global__ __launch_bounds__(SC_BLOCK) void part_scan_kernel(u32* __restrict__ counts, const u32* __restrict__ starts,
-                                                              const u32* __restrict__ blocktot,
-                                                              u32* __restrict__ pstart, u32 n_tiles, u32 P) {
-    __shared__ u32 red[SC_BLOCK / 64];
-    __shared__ u32 colbase[64];
-    __shared__ u32 part_sum[SC_BLOCK / 64][64];
-    constexpr u32 WAVES = SC_BLOCK / 64, KEEP = 32;
-    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
-    const u32 blk = blockIdx.x, d0 = blk * 64u, NB = P / 64u;
-    const u32 per = (n_tiles + WAVES - 1) / WAVES;
-    const u32 t0 = w * per < n_tiles ? w * per : n_tiles;
-    const u32 t1 = t0 + per < n_tiles ? t0 + per : n_tiles;
-    u32* col = counts + d0 + lane;
-    const u32* scol = starts + d0 + lane;
-    // all the loads of this workgroup are issued before the first is used: the counts of this
-    // wavefront's tiles (kept in registers when there are few), the block counts of the lower blocks
-    const bool keep = per <= KEEP;
-    u32 v[KEEP], st[KEEP];
-    u32 s = 0;
-    if (keep) {
-#pragma unroll
-        for (u32 x = 0; x < KEEP; ++x) {
-            const bool in = t0 + x < t1;
-            v[x] = in ? col[(size_t)(t0 + x) * P] : 0u;
-            st[x] = in ? scol[(size_t)(t0 + x) * P] : 0u;
-        }
-    }
-    u32 before = 0;
-    {
-        // (tile, lower block) pairs dealt to the threads, eight loads in flight
-        const u32 pairs = n_tiles * blk;
-        for (u32 i0 = tid; i0 < pairs; i0 += 8 * SC_BLOCK) {
-            u32 bv[8];
-#pragma unroll
-            for (u32 x = 0; x < 8; ++x) {
-                const u32 i = i0 + x * SC_BLOCK;
-                bv[x] = 0;
-                if (i < pairs) bv[x] = blocktot[(size_t)(i / blk) * NB + i % blk];
-            }
-#pragma unroll
-            for (u32 x = 0; x < 8; ++x) before += bv[x];
-        }
-    }
-    if (keep) {
-#pragma unroll
-        for (u32 x = 0; x < KEEP; ++x) s += v[x];
-    } else {
-        u32 tt = t0;
-        for (; tt + 8 <= t1; tt += 8) {
-            u32 cv[8];
-#pragma unroll
-            for (u32 x = 0; x < 8; ++x) cv[x] = col[(size_t)(tt + x) * P];
-#pragma unroll
-            for (u32 x = 0; x < 8; ++x) s += cv[x];
-        }
-        for (; tt < t1; ++tt) s += col[(size_t)tt * P];
-    }
-    for (u32 off = 32; off >= 1; off >>= 1) before += __shfl_down(before, off);
-    if (lane == 0) red[w] = before;
-    part_sum[w][lane] = s;
-    __syncthreads();
-    if (w == 0) {  // this block's partitions: totals, their exclusive prefix over the lanes
-        u32 base = 0;
-        for (u32 x = 0; x < WAVES; ++x) base += red[x];
-        u32 tot = 0;
-        for (u32 x = 0; x < WAVES; ++x) tot += part_sum[x][lane];
-        u32 incl = tot;
-        for (u32 off = 1; off < 64; off <<= 1) {
-            const u32 o = __shfl_up(incl, off);
-            if (lane >= off) incl += o;
-        }
-        colbase[lane] = base + incl - tot;
-        pstart[d0 + lane] = base + incl - tot;
-        if (blk + 1 == NB && lane == 63) pstart[P] = base + incl;
-    }
-    __syncthreads();
-    u32 pos = colbase[lane];
-    for (u32 x = 0; x < w; ++x) pos += part_sum[x][lane];
-    if (keep) {
-#pragma unroll
-        for (u32 x = 0; x < KEEP; ++x)
-            if (t0 + x < t1) {
-                col[(size_t)(t0 + x) * P] = pos - st[x];
-                pos += v[x];
-            }
-    } else {
-        u32 tt = t0;
-        for (; tt + 8 <= t1; tt += 8) {
-            u32 cv[8], sv[8];
-#pragma unroll
-            for (u32 x = 0; x < 8; ++x) {
-                cv[x] = col[(size_t)(tt + x) * P];
-                sv[x] = scol[(size_t)(tt + x) * P];
-            }
-#pragma unroll
-            for (u32 x = 0; x < 8; ++x) {
-                col[(size_t)(tt + x) * P] = pos - sv[x];
-                pos += cv[x];
-            }
-        }
-        for (; tt < t1; ++tt) {
-            const u32 c = col[(size_t)tt * P];
-            col[(size_t)tt * P] = pos - scol[(size_t)tt * P];
-            pos += c;
-        }
-    }
-}
-
-// ---- 3. scatter -----------------------------------------------------------------------------------
-__global__ __launch_bounds__(PT_BLOCK) void part_scatter_kernel(TableDev t, const uint4* __restrict__ stage,
-                                                                 const u32* __restrict__ delta,
-                                                                 const u32* __restrict__ tile_total, u32 P,
-                                                                 u32 part_shift, uint4* __restrict__ ent) {
-    const u32 tile = blockIdx.x, tid = threadIdx.x;
-    const u64 tb = (u64)tile * PT_TILE;
-    const u32 cnt = tile_total[tile];
-    uint4 e[PT_ITEMS];
-#pragma unroll
-    for (u32 j = 0; j < PT_ITEMS; ++j) {
-        const u32 q = j * PT_BLOCK + tid;
-        e[j] = stage[tb + (q < cnt ? q : 0u)];
-    }
-    u32 d[PT_ITEMS];
-#pragma unroll
-    for (u32 j = 0; j < PT_ITEMS; ++j) {
-        const u32 p = partition_of(t, hash64(((u64)e[j].y << 32) | e[j].x), part_shift);
-        d[j] = delta[(size_t)tile * P + p];
-    }
-#pragma unroll
-    for (u32 j = 0; j < PT_ITEMS; ++j) {
-        const u32 q = j * PT_BLOCK + tid;
-        if (q < cnt) ent[d[j] + q] = e[j];
-    }
-}
-
-// ---- 4. apply -------------------------------------------------------------------------------------
+// ---- 2. apply -------------------------------------------------------------------------------------
 // LDS (dynamic, 72 KiB): entry keys | hash table (later the accumulators) | counts | aux |
 // entry references (later the rows of the distinct keys) | references grouped by key | list numbers |
 // distinct keys | keys with more than one entry.
@@ -550,8 +409,11 @@ constexpr u32 PA_OFF_MREP = PA_OFF_UREP + PA_CAP * 2;
 constexpr u32 PA_LDS = PA_OFF_MREP + PA_CAP * 2;  // 75776
 
 struct ApplyArgs {
-    const uint4* ent;  // {key low, key high, reference, -}
-    const u32* pstart;
+    const uint4* stage;  // {key low, key high, reference, -}, a block of PT_TILE per tile
+    const u32* starts;   // [tile][P + 1]: where each partition's entries start in the tile's block
+    u32* pstart;         // out: entries in lower partitions (where the partition parks its new keys)
+    u32 n_tiles, P;
+    u32 search_step;     // half the power of two that n_tiles rounds up to
     u32* new_slot;
     u32* new_count;
     u32 units;
@@ -838,6 +700,41 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
     }
 }
 
+// The partition's segments in the staging blocks: tile x holds entries [ta[x], ta[x] + count) of its
+// block, and they are entries toff[x] .. of the partition (toff is filled for all PA_TILES_MAX
+// numbers, with the partition's entry count beyond the last tile). A thread takes two tiles; the
+// loads are issued before anything waits. Returns {entries of the partition, entries in lower
+// partitions}. All threads call it.
+constexpr u32 PA_TILES_MAX = 2 * PA_BLOCK;
+static_assert(PART_MAX_KEYS / PT_TILE <= PA_TILES_MAX, "two tiles per thread cover the largest batch");
+static_assert(2 * PA_TILES_MAX <= PA_CAP, "the offsets fit the room of the reference list");
+
+__device__ __forceinline__ u64 tile_segments(const ApplyArgs& a, u32 p, u32 tid, u64* sums, u32* toff, u32* ta) {
+    const u32 x0 = 2u * tid, x1 = x0 + 1u;
+    const size_t stride = (size_t)a.P + 1u;
+    const u32* c0 = a.starts + (size_t)(x0 < a.n_tiles ? x0 : 0u) * stride + p;
+    const u32* c1 = a.starts + (size_t)(x1 < a.n_tiles ? x1 : 0u) * stride + p;
+    u32 a0 = c0[0], b0 = c0[1], a1 = c1[0], b1 = c1[1];
+    if (x0 >= a.n_tiles) a0 = b0 = 0u;
+    if (x1 >= a.n_tiles) a1 = b1 = 0u;
+    const u32 n0 = b0 - a0, n1 = b1 - a1;
+    u64 tot = 0;
+    const u64 ex = block_scan_excl<PA_BLOCK>((u64)(n0 + n1) | ((u64)(a0 + a1) << 32), tid, sums, &tot);
+    toff[x0] = (u32)ex;
+    toff[x1] = (u32)ex + n0;
+    ta[x0] = a0;
+    ta[x1] = a1;
+    return tot;
+}
+
+// entry i of the partition (tile_segments() has run, a barrier since)
+__device__ __forceinline__ uint4 partition_entry(const ApplyArgs& a, const u32* toff, const u32* ta, u32 i) {
+    u32 x = 0;
+    for (u32 step = a.search_step; step; step >>= 1)
+        if (toff[x + step] <= i) x += step;  // the last tile that starts at or before entry i
+    return a.stage[(size_t)x * PT_TILE + ta[x] + (i - toff[x])];
+}
+
 template <typename T>
 __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, const T* __restrict__ grads,
                                                                const T* __restrict__ psum, T* __restrict__ ngrad,
@@ -848,22 +745,31 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
     __shared__ u32 stk[24];
     u64* lkey = reinterpret_cast<u64*>(pa_lds);
     u32* lref = reinterpret_cast<u32*>(pa_lds + PA_OFF_LREF);
+    u32* toff = reinterpret_cast<u32*>(pa_lds + PA_OFF_LIST);  // (the reference list is written later)
+    u32* ta = toff + PA_TILES_MAX;
     const u32 tid = threadIdx.x;
-    const u32 p = blockIdx.x;
-    const u32 s = a.pstart[p], np = a.pstart[p + 1] - s;
+    // Workgroups are dealt to the eight XCDs in turn: each XCD takes a run of consecutive partitions,
+    // whose start words and staging segments share cache lines, into its own L2.
+    const u32 p = (blockIdx.x & 7u) * (a.P >> 3) + (blockIdx.x >> 3);
+    const u64 seg = tile_segments(a, p, tid, sums, toff, ta);
+    const u32 np = (u32)seg, s = (u32)(seg >> 32);
     // the row count as it is when this operation begins (this launch hands out no rows)
     if (p == 0 && tid == 0) t.counters[CNT_ENTRY] = t.counters[CNT_ROWS];
-    if (tid == 0) s_nnew = 0;
+    if (tid == 0) {
+        s_nnew = 0;
+        a.pstart[p] = s;
+    }
     if (np == 0) {
         if (tid == 0) a.new_count[p] = 0;
         return;
     }
+    __syncthreads();
     if (np <= a.cap) {
         uint4 e[PA_ITEMS];
 #pragma unroll
         for (u32 j = 0; j < PA_ITEMS; ++j) {
             const u32 i = j * PA_BLOCK + tid;
-            e[j] = a.ent[s + (i < np ? i : 0u)];
+            e[j] = partition_entry(a, toff, ta, i < np ? i : 0u);
         }
 #pragma unroll
         for (u32 j = 0; j < PA_ITEMS; ++j) {
@@ -898,8 +804,10 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
                 }
                 __syncthreads();
                 const u32 lg = top >> 16, cls = top & 0xFFFFu, mask = (1u << lg) - 1u;
+                tile_segments(a, p, tid, sums, toff, ta);  // (a pass overwrites them)
+                __syncthreads();
                 for (u32 i = tid; i < np; i += PA_BLOCK) {
-                    const uint4 e = a.ent[s + i];
+                    const uint4 e = partition_entry(a, toff, ta, i);
                     const u64 key = ((u64)e.y << 32) | e.x;
                     if (((u32)(hash64(key) >> 53) & mask) == cls) {
                         const u32 pos = atomicAdd(&s_sel, 1u);
@@ -933,7 +841,7 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
     }
 }
 
-// ---- 5. insert ------------------------------------------------------------------------------------
+// ---- 3. insert ------------------------------------------------------------------------------------
 constexpr u32 PI_BLOCK = 256;
 
 template <typename T>
@@ -1039,11 +947,7 @@ PartSizes part_sizes(uint32_t dim, size_t n) {
     const size_t n_tiles = (n + PT_TILE - 1) / PT_TILE;
     const size_t np = n_tiles * PT_TILE;
     z.stage = np * 16;
-    z.ent = np * 16;
-    z.counts = n_tiles * PT_MAX_PARTS * 4;
-    z.starts = z.counts;
-    z.blocktot = n_tiles * (PT_MAX_PARTS / 64) * 4;
-    z.tile_total = n_tiles * 4;
+    z.starts = n_tiles * (PT_MAX_PARTS + 1) * 4;
     z.pstart = (PT_MAX_PARTS + 1) * 4;
     z.psum = n_tiles * PT_MAX_MULTI * (size_t)dim * 4;
     z.new_slot = np * 4;
@@ -1069,30 +973,21 @@ hipError_t launch_part_tile(const TableDev& t, const PartPlan& pl, const PartBuf
                             const float* grads, hipStream_t s) {
     if ((t.dim % 4 == 0) && aligned16(grads))
         part_tile_kernel<float4><<<pl.n_tiles, PT_BLOCK, PT_LDS_FIXED + pl.P * 4, s>>>(
-            t, keys, reinterpret_cast<const float4*>(grads), pl.n, pl.P, pl.part_shift, b.stage, b.counts, b.starts,
-            b.blocktot, b.tile_total, reinterpret_cast<float4*>(b.psum), t.dim / 4);
+            t, keys, reinterpret_cast<const float4*>(grads), pl.n, pl.P, pl.part_shift, b.stage, b.starts,
+            reinterpret_cast<float4*>(b.psum), t.dim / 4);
     else
-        part_tile_kernel<float><<<pl.n_tiles, PT_BLOCK, PT_LDS_FIXED + pl.P * 4, s>>>(t, keys, grads, pl.n, pl.P, pl.part_shift, b.stage,
-                                                                    b.counts, b.starts, b.blocktot, b.tile_total,
-                                                                    b.psum, t.dim);
-    return hipGetLastError();
-}
-
-hipError_t launch_part_scan(const PartPlan& pl, const PartBufs& b, hipStream_t s) {
-    part_scan_kernel<<<pl.P / 64, SC_BLOCK, 0, s>>>(b.counts, b.starts, b.blocktot, b.pstart, pl.n_tiles, pl.P);
-    return hipGetLastError();
-}
-
-hipError_t launch_part_scatter(const TableDev& t, const PartPlan& pl, const PartBufs& b, hipStream_t s) {
-    part_scatter_kernel<<<pl.n_tiles, PT_BLOCK, 0, s>>>(t, b.stage, b.counts, b.tile_total, pl.P, pl.part_shift, b.ent);
+        part_tile_kernel<float><<<pl.n_tiles, PT_BLOCK, PT_LDS_FIXED + pl.P * 4, s>>>(
+            t, keys, grads, pl.n, pl.P, pl.part_shift, b.stage, b.starts, b.psum, t.dim);
     return hipGetLastError();
 }
 
 hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads, bool insert,
                              hipStream_t s) {
     const bool v4 = (t.dim % 4 == 0) && aligned16(grads);
-    ApplyArgs a{b.ent, b.pstart, b.new_slot, b.new_count, v4 ? t.dim / 4 : t.dim, insert ? 1 : 0,
-                g_part_cap};
+    u32 pow2 = 1;
+    while (pow2 < pl.n_tiles) pow2 <<= 1;
+    ApplyArgs a{b.stage, b.starts, b.pstart, pl.n_tiles, pl.P, pow2 / 2, b.new_slot, b.new_count,
+                v4 ? t.dim / 4 : t.dim, insert ? 1 : 0, g_part_cap};
     if (v4)
         part_apply_kernel<float4><<<pl.P, PA_BLOCK, PA_LDS, s>>>(t, reinterpret_cast<const float4*>(grads),
                                                                  reinterpret_cast<const float4*>(b.psum),

@@ -193,12 +193,11 @@ struct PartPlan {
     uint32_t n, n_tiles, P, part_shift;
 };
 struct PartSizes {
-    size_t stage, ent, counts, starts, blocktot, tile_total, pstart, psum, new_slot,
-        new_count, ngrad;
+    size_t stage, starts, pstart, psum, new_slot, new_count, ngrad;
 };
 struct PartBufs {
-    uint4 *stage, *ent;  // entries {key low, key high, reference, -}: per tile, then per partition
-    uint32_t *counts, *starts, *blocktot, *tile_total, *pstart, *new_slot, *new_count;
+    uint4* stage;  // entries {key low, key high, reference, -}: a block per tile, grouped by partition
+    uint32_t *starts, *pstart, *new_slot, *new_count;
     float *psum, *ngrad;
 };
 bool part_plan(const TableDev& t, size_t n, PartPlan* plan);
@@ -206,8 +205,6 @@ PartSizes part_sizes(uint32_t dim, size_t n);
 hipError_t part_init();  // once per device, before the first launch
 hipError_t launch_part_tile(const TableDev& t, const PartPlan& pl, const PartBufs& b, const uint64_t* keys,
                             const float* grads, hipStream_t s);
-hipError_t launch_part_scan(const PartPlan& pl, const PartBufs& b, hipStream_t s);
-hipError_t launch_part_scatter(const TableDev& t, const PartPlan& pl, const PartBufs& b, hipStream_t s);
 hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads, bool insert,
                              hipStream_t s);
 hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads,
