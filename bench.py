@@ -142,14 +142,23 @@ def keys_alone_in_tile(torch, keys, tile=4096):
     return int((~(same_next | same_prev)).sum().item()) - pad
 
 
-def run_steps(t, torch, cfg, batches, out, steps, first=0):
+def run_steps(t, torch, cfg, batches, out, steps, first=0, handles=None):
+    """`steps` steps: the pull of a batch, then the push of gradients for the same keys. With
+    `handles` (a device array of one word per key) the pull tells the push where the rows lie
+    (pshbm_pull_dev_handles / pshbm_push_dev_handles), so that the push does not look the keys up
+    a second time; without, the plain pshbm_pull_dev / pshbm_push_dev."""
     stream = torch.cuda.current_stream().cuda_stream
     k = cfg["batch"]
     for i in range(first, first + steps):
         keys, grads = batches[i % len(batches)][:2]
-        st = t.pull_dev(keys.data_ptr(), k, out.data_ptr(), None, 0, stream)
-        if st == 0 and not cfg["pull_only"]:
-            st = t.push_dev(keys.data_ptr(), grads.data_ptr(), k, 0, stream)
+        if handles is None or cfg["pull_only"]:
+            st = t.pull_dev(keys.data_ptr(), k, out.data_ptr(), None, 0, stream)
+            if st == 0 and not cfg["pull_only"]:
+                st = t.push_dev(keys.data_ptr(), grads.data_ptr(), k, 0, stream)
+        else:
+            st, epoch = t.pull_dev_handles(keys.data_ptr(), k, out.data_ptr(), handles.data_ptr(), None, 0, stream)
+            if st == 0:
+                st = t.push_dev_handles(keys.data_ptr(), grads.data_ptr(), handles.data_ptr(), epoch, k, 0, stream)
         if st != 0:
             raise RuntimeError(f"step {i} failed: {st} {t.last_error()}")
 
@@ -362,17 +371,18 @@ def measure(name, args, torch, ps, wl, steps, warmup, headline):
     out = torch.empty(cfg["batch"], cfg["dim"], device="cuda")
     k = cfg["batch"]
     keys_per_step = k * (1 if cfg["pull_only"] else 2)
+    handles = None if args.no_handles else torch.empty(k, dtype=torch.int32, device="cuda")
 
-    run_steps(t, torch, cfg, batches, out, warmup)
+    run_steps(t, torch, cfg, batches, out, warmup, handles=handles)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    run_steps(t, torch, cfg, batches, out, steps, first=warmup)
+    run_steps(t, torch, cfg, batches, out, steps, first=warmup, handles=handles)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / steps
 
     t.profile_enable(True)
-    run_steps(t, torch, cfg, batches, out, steps, first=warmup)
+    run_steps(t, torch, cfg, batches, out, steps, first=warmup, handles=handles)
     torch.cuda.synchronize()
     prof = t.profile_read()
     t.profile_enable(False)
@@ -405,7 +415,8 @@ def measure(name, args, torch, ps, wl, steps, warmup, headline):
     res = {
         "value": keys_per_step * steps / elapsed, "ms_per_step": ms_per_step, "steps": steps, "warmup": warmup,
         "config": {"workload": cfg["desc"], "table_keys": n_table, "batch": k, "dim": cfg["dim"],
-                   "unique_keys_per_batch": round(u_mean), "keys_alone_in_their_tile": round(alone_mean)},
+                   "unique_keys_per_batch": round(u_mean), "keys_alone_in_their_tile": round(alone_mean),
+                   "row_handles": handles is not None and not cfg["pull_only"]},
         "step_algorithmic_bytes": int(step_bytes),
         "step_algorithmic_GBps": round(step_bytes / (ms_per_step * 1e6), 1),
         "step_frac_of_hbm_peak": round(step_bytes / (ms_per_step * 1e6) / HBM_PEAK_GBS, 4),
@@ -438,6 +449,9 @@ def main():
                          "configurations follow, 20 steps each, and are reported under \"configs\"")
     ap.add_argument("--table-keys", type=int, default=0, help="override the headline table size (testing)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-handles", action="store_true",
+                    help="plain pshbm_pull_dev / pshbm_push_dev: the push looks every key up again instead of "
+                         "taking the rows the pull of the same batch found")
     ap.add_argument("--cpu-keys", type=int, default=10_000_000, help="table size of the CPU sample")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device copy, a kernel of known HBM traffic that "

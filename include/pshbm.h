@@ -107,6 +107,7 @@ typedef struct pshbm_table pshbm_table;
 #define PSHBM_PUSH_NO_INSERT 1u      /* init_store_value returns false, item dropped: SparsePushOperator.h:250-251 */
 #define PSHBM_PUSH_ASSUME_UNIQUE 2u  /* caller guarantees distinct keys (a client batch after
                                         SparsePushOperator.h:134-141): skips the aggregation */
+#define PSHBM_PUSH_VERIFY_HANDLES 4u /* pshbm_push_dev_handles: trust a handle only if the row it names holds the key */
 /* load flags */
 #define PSHBM_LOAD_UNIQUE 1u         /* a key already present is an error: LoadOperator.h:194,210 */
 
@@ -164,6 +165,29 @@ int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, siz
                    uint32_t flags);
 int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
                        uint32_t flags, void* stream);
+
+/* Row handles: a pull tells the push that follows it where the rows lie. The reference's learner
+ * pulls a batch, computes, and pushes gradients for the same keys, and the server looks every key up
+ * both times (lock_find in SparsePullOperator.h:214 and again in SparsePushOperator.h:248). Here the
+ * second lookup can be spared: pshbm_pull_dev_handles is pshbm_pull_dev that also writes d_handles[i],
+ * an opaque word per key (n words), and *epoch, the table's handle epoch at the time of the call;
+ * pshbm_push_dev_handles is pshbm_push_dev that takes both back, for the SAME key array, and updates
+ * the rows the handles name without probing the hash array; keys whose handle says "not stored" are
+ * looked up (and inserted) as usual. Results are those of pshbm_push_dev. Handles stay good while
+ * the table's epoch is the one the pull reported: pushes, sets, loads and inserting pulls leave it
+ * (rows never move when keys are added), every erase, erase_if and clear begins a new one; handles of
+ * another epoch are ignored (the push then looks every key up). Handles are a hint for batches that
+ * take the partitioned path (16,384 keys and more); smaller ones ignore them.
+ * A handle array that does not belong to the key array is the caller's error, as a gradient array
+ * that does not would be: rows of other keys take the update. PSHBM_PUSH_VERIFY_HANDLES makes the
+ * push trust a handle only where the table's key of that row equals the batch key (one more random
+ * 8-byte read per distinct key, about the cost of the lookup it replaces) and look the others up. */
+int32_t pshbm_pull_dev_handles(pshbm_table* t, const uint64_t* d_keys, size_t n, float* d_out_rows,
+                               uint8_t* d_hit, uint32_t* d_handles, uint64_t* epoch, uint32_t flags,
+                               void* stream);
+int32_t pshbm_push_dev_handles(pshbm_table* t, const uint64_t* d_keys, const float* d_grads,
+                               const uint32_t* d_handles, uint64_t epoch, size_t n, uint32_t flags,
+                               void* stream);
 
 /* pshbm_push_dev for callers that cannot allocate device memory while they run: code under HIP graph
  * capture, tight serving loops, harnesses that forbid it. It has no counterpart in the reference.

@@ -23,6 +23,7 @@ OPT_SUM, OPT_SGD, OPT_ADAGRAD, OPT_FTRL, OPT_USER = 0, 1, 2, 3, 4
 PULL_INSERT_ON_MISS = 1
 PUSH_NO_INSERT = 1
 PUSH_ASSUME_UNIQUE = 2
+PUSH_VERIFY_HANDLES = 4
 LOAD_UNIQUE = 1
 
 # every symbol include/pshbm.h declares
@@ -34,7 +35,7 @@ SYMBOLS = [
     "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve", "pshbm_set_hyperparameters", "pshbm_set_memory_limit", "pshbm_device_memory",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
-    "pshbm_push_dev_noalloc", "pshbm_debug_sort_spin_limit", "pshbm_debug_part_pass_capacity",
+    "pshbm_push_dev_noalloc", "pshbm_pull_dev_handles", "pshbm_push_dev_handles", "pshbm_debug_sort_spin_limit", "pshbm_debug_part_pass_capacity",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
           "fixup_windows", "assign_rows", "push_small", "part_tile", "part_apply", "part_insert"]
@@ -184,6 +185,8 @@ def lib():
         L.pshbm_push.argtypes = [vp, vp, vp, sz, u32]
         L.pshbm_push_dev.argtypes = [vp, vp, vp, sz, u32, vp]
         L.pshbm_push_dev_noalloc.argtypes = [vp, vp, vp, sz, u32, vp]
+        L.pshbm_pull_dev_handles.argtypes = [vp, vp, sz, vp, vp, vp, C.POINTER(C.c_uint64), u32, vp]
+        L.pshbm_push_dev_handles.argtypes = [vp, vp, vp, vp, C.c_uint64, sz, u32, vp]
         L.pshbm_debug_sort_spin_limit.argtypes = [u32]
         L.pshbm_debug_part_pass_capacity.argtypes = [u32]
         L.pshbm_push_pairs.argtypes = [vp, vp, sz, sz, u32]
@@ -499,6 +502,17 @@ class Table:
 
     def push_dev(self, d_keys, d_grads, n, flags=0, stream=0):
         return lib().pshbm_push_dev(self._h, d_keys, d_grads, n, flags, stream)
+
+    def pull_dev_handles(self, d_keys, n, d_out, d_handles, d_hit=None, flags=0, stream=0):
+        """pull_dev that also writes a row handle per key (n uint32 on the device); returns
+        (status, epoch) for push_dev_handles."""
+        epoch = C.c_uint64(0)
+        st = lib().pshbm_pull_dev_handles(self._h, d_keys, n, d_out, d_hit, d_handles, C.byref(epoch), flags, stream)
+        return st, epoch.value
+
+    def push_dev_handles(self, d_keys, d_grads, d_handles, epoch, n, flags=0, stream=0):
+        """push_dev of the key array a pull_dev_handles answered, with that call's handles and epoch."""
+        return lib().pshbm_push_dev_handles(self._h, d_keys, d_grads, d_handles, epoch, n, flags, stream)
 
     def push_dev_noalloc(self, d_keys, d_grads, n, flags=0, stream=0):
         """push_dev with its scratch in the library's fixed device array: allocates nothing."""

@@ -207,6 +207,9 @@ struct pshbm_table {
     // scratch of the partitioned push (batches of PART_MIN_KEYS keys and more)
     DevBuf pt_stage, pt_starts, pt_pstart, pt_psum, pt_new_slot, pt_new_count, pt_ngrad;
     size_t part_keys = 0;       // batch size those arrays serve
+    // Row handles (what a pull reports for the push that follows) stay good while no row moves or
+    // goes: every erase and clear begins a new epoch.
+    uint64_t epoch = 1;
 
     // staging of the host-pointer entry points
     std::mutex st_mu;
@@ -573,7 +576,8 @@ Workspace table_workspace(pshbm_table* t) {
 // One push on stream s with the scratch of `w`. *used_sort_head: the sort took the half of the sort
 // head that w.sort_parity names (and zeroed the other one).
 int32_t push_with(pshbm_table* t, const Workspace& w, const uint64_t* d_keys, const float* d_grads, size_t n,
-                  uint32_t flags, hipStream_t s, bool* used_sort_head, bool* used_won, bool* used_part) {
+                  uint32_t flags, hipStream_t s, bool* used_sort_head, bool* used_won, bool* used_part,
+                  const uint32_t* d_handles = nullptr) {
     *used_sort_head = false;
     *used_won = false;
     *used_part = false;
@@ -593,8 +597,11 @@ int32_t push_with(pshbm_table* t, const Workspace& w, const uint64_t* d_keys, co
     PartPlan pl;
     if (!unique && !checked && n <= w.part_keys && part_plan(t->d, n, &pl)) {
         *used_part = true;
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_TILE, launch_part_tile(t->d, pl, w.part, d_keys, d_grads, s));
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_APPLY, launch_part_apply(t->d, pl, w.part, d_grads, insert, s));
+        // (the other paths look every key up anyway: handles only serve here)
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_TILE, launch_part_tile(t->d, pl, w.part, d_keys, d_grads, d_handles, s));
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_APPLY,
+                     launch_part_apply(t->d, pl, w.part, d_grads, insert, d_handles != nullptr,
+                                       (flags & PSHBM_PUSH_VERIFY_HANDLES) != 0, s));
         if (insert) HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_INSERT, launch_part_insert(t->d, pl, w.part, d_grads, s));
         return PSHBM_OK;
     }
@@ -634,13 +641,13 @@ int32_t push_with(pshbm_table* t, const Workspace& w, const uint64_t* d_keys, co
 }
 
 int32_t push_locked(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
-                    uint32_t flags, hipStream_t s) {
+                    uint32_t flags, hipStream_t s, const uint32_t* d_handles = nullptr) {
     if (n == 0) return PSHBM_OK;
     ST_TRY(begin_op(t, s));
     ST_TRY(ensure_workspace(t, n));
     const Workspace w = table_workspace(t);
     bool used_head = false, used_won = false, used_part = false;
-    const int32_t st = push_with(t, w, d_keys, d_grads, n, flags, s, &used_head, &used_won, &used_part);
+    const int32_t st = push_with(t, w, d_keys, d_grads, n, flags, s, &used_head, &used_won, &used_part, d_handles);
     if (used_head) ++t->sort_parity;
     if (used_won) ++t->won_parity;
     return st;
@@ -776,6 +783,7 @@ int32_t erase_flagged(pshbm_table* t, uint32_t rows, hipStream_t s, uint64_t* er
     if (erased) *erased = gone;
     set_exact_rows(t, rows - gone);
     if (gone == 0) return PSHBM_OK;
+    ++t->epoch;  // rows move into the holes: handles of earlier pulls are void
     ST_TRY(ensure(t, t->ms_lists, 3 * (size_t)gone * 4));
     HIP_TRY(t, launch_erase_apply(t->d, rows, gone, dead, tiles, t->d_info,
                                   static_cast<uint32_t*>(t->ms_lists.p), s));
@@ -929,10 +937,16 @@ int32_t pshbm_destroy(pshbm_table* t) {
 }
 
 // ---- pull ------------------------------------------------------------------------------------
-int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* d_out_rows,
-                       uint8_t* d_hit, uint32_t flags, void* stream) {
+static int32_t pull_dev_impl(pshbm_table* t, const uint64_t* d_keys, size_t n, float* d_out_rows,
+                             uint8_t* d_hit, uint32_t* d_handles, uint64_t* epoch, uint32_t flags, void* stream) {
     if (!t) return PSHBM_INVALID_ID;
-    if (n == 0) return PSHBM_OK;
+    if (n == 0) {
+        if (epoch) {
+            std::shared_lock<std::shared_mutex> rl(t->mu);
+            *epoch = t->epoch;
+        }
+        return PSHBM_OK;
+    }
     if (!d_keys || !d_out_rows) return fail(t, PSHBM_ERROR, "pull: null buffer");
     if (n > 0x7FFFFFFFull) return fail(t, PSHBM_ERROR, "pull: batch larger than 2^31-1 keys");
     DeviceGuard g(t->device);
@@ -941,7 +955,8 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     std::unique_lock<std::shared_mutex> lk(t->mu);
     ST_TRY(begin_op(t, s, !insert));
     if (!insert) {
-        HIP_TRY_PROF(t, s, PSHBM_PHASE_PULL, launch_pull(t->d, d_keys, n, d_out_rows, d_hit, s));
+        if (epoch) *epoch = t->epoch;
+        HIP_TRY_PROF(t, s, PSHBM_PHASE_PULL, launch_pull(t->d, d_keys, n, d_out_rows, d_hit, d_handles, s));
         return PSHBM_OK;
     }
     ST_TRY(ensure_workspace(t, n));
@@ -954,8 +969,21 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
     ST_TRY(locate_and_assign(t, d_keys, n, slot, nullptr, nullptr, true, true, false, w.won_cur, w.won_next,
                              w.won_words, s));
     if (checked) ST_TRY(settle_rows(t, slot, n, s, rows_before));
-    HIP_TRY_PROF(t, s, PSHBM_PHASE_GATHER, launch_gather_slots(t->d, d_keys, slot, n, d_out_rows, d_hit, s));
+    if (epoch) *epoch = t->epoch;
+    HIP_TRY_PROF(t, s, PSHBM_PHASE_GATHER, launch_gather_slots(t->d, d_keys, slot, n, d_out_rows, d_hit, d_handles, s));
     return PSHBM_OK;
+}
+
+int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* d_out_rows,
+                       uint8_t* d_hit, uint32_t flags, void* stream) {
+    return pull_dev_impl(t, d_keys, n, d_out_rows, d_hit, nullptr, nullptr, flags, stream);
+}
+
+int32_t pshbm_pull_dev_handles(pshbm_table* t, const uint64_t* d_keys, size_t n, float* d_out_rows,
+                               uint8_t* d_hit, uint32_t* d_handles, uint64_t* epoch, uint32_t flags,
+                               void* stream) {
+    if (t && (!d_handles || !epoch)) return fail(t, PSHBM_ERROR, "pull_handles: null handle buffer or epoch");
+    return pull_dev_impl(t, d_keys, n, d_out_rows, d_hit, d_handles, epoch, flags, stream);
 }
 
 // A lane that is free, else the next one in turn; held until `lock` goes.
@@ -1035,6 +1063,20 @@ int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_gr
     DeviceGuard g(t->device);
     std::unique_lock<std::shared_mutex> lk(t->mu);
     return push_locked(t, d_keys, d_grads, n, flags, static_cast<hipStream_t>(stream));
+}
+
+int32_t pshbm_push_dev_handles(pshbm_table* t, const uint64_t* d_keys, const float* d_grads,
+                               const uint32_t* d_handles, uint64_t epoch, size_t n, uint32_t flags,
+                               void* stream) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (n == 0) return PSHBM_OK;
+    if (!d_keys || !d_grads) return fail(t, PSHBM_ERROR, "push: null buffer");
+    if (n > MAX_PUSH_BATCH) return fail(t, PSHBM_ERROR, "push: batch larger than 2^30-1 keys");
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    // handles of another epoch say nothing any more: the push looks every key up, as pshbm_push_dev does
+    const uint32_t* h = (d_handles && epoch == t->epoch) ? d_handles : nullptr;
+    return push_locked(t, d_keys, d_grads, n, flags, static_cast<hipStream_t>(stream), h);
 }
 
 // The same push with its scratch in the library's fixed device array: nothing is allocated, by this
@@ -1828,6 +1870,7 @@ int32_t pshbm_clear(pshbm_table* t) {
     HIP_TRY(t, hipStreamSynchronize(s));
     set_exact_rows(t, 0);
     t->tombstones = 0;
+    ++t->epoch;
     return PSHBM_OK;
 }
 

@@ -47,7 +47,8 @@ __device__ __forceinline__ void gather_round(const TableDev& t, u32 row, u64 bas
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void pull_kernel(TableDev t, const u64* __restrict__ keys,
                                                       u32 n, T* __restrict__ out,
-                                                      uint8_t* __restrict__ hit, u32 units,
+                                                      uint8_t* __restrict__ hit,
+                                                      u32* __restrict__ handles, u32 units,
                                                       u32 stride_units, u64 m32) {
     const u32 lane = threadIdx.x & 63u;
     const u32 grp = lane >> 2, sub = lane & 3u;
@@ -60,6 +61,7 @@ __global__ __launch_bounds__(BLOCK) void pull_kernel(TableDev t, const u64* __re
         bool active = inb && key < KEY_DELETED;
         Found f = probe_find(t, key, active, grp, sub);
         if (hit && inb && sub == 0) hit[i] = f.row != ROW_NONE;
+        if (handles && inb && sub == 0) handles[i] = f.row;  // the row, or ROW_NONE
         u32 cnt = (u32)((n - base) < KEYS_PER_ROUND ? (n - base) : KEYS_PER_ROUND);
         gather_round<T>(t, f.row, base, cnt, out, units, stride_units, m32, lane, keys);
     }
@@ -70,7 +72,8 @@ __global__ __launch_bounds__(BLOCK) void gather_slots_kernel(TableDev t,
                                                               const u64* __restrict__ keys,
                                                               const u32* __restrict__ slot_idx,
                                                               u32 n, T* __restrict__ out,
-                                                              uint8_t* __restrict__ hit, u32 units,
+                                                              uint8_t* __restrict__ hit,
+                                                              u32* __restrict__ handles, u32 units,
                                                               u32 stride_units, u64 m32) {
     const u32 lane = threadIdx.x & 63u;
     const u32 grp = lane >> 2, sub = lane & 3u;
@@ -85,6 +88,7 @@ __global__ __launch_bounds__(BLOCK) void gather_slots_kernel(TableDev t,
             if (s != SLOT_NONE) row = reinterpret_cast<const u32*>(&t.slots[s])[2];
             if (row >= t.max_rows) row = ROW_NONE;
             if (hit && sub == 0) hit[i] = row < entry_rows;
+            if (handles && sub == 0) handles[i] = row;
         }
         u32 cnt = (u32)((n - base) < KEYS_PER_ROUND ? (n - base) : KEYS_PER_ROUND);
         gather_round<T>(t, row, base, cnt, out, units, stride_units, m32, lane, keys);
@@ -990,32 +994,32 @@ hipError_t launch_fill_u32(u32* p, size_t n, u32 v, hipStream_t s) {
     return hipGetLastError();
 }
 
-hipError_t launch_pull(const TableDev& t, const u64* keys, size_t n, float* out, uint8_t* hit,
+hipError_t launch_pull(const TableDev& t, const u64* keys, size_t n, float* out, uint8_t* hit, u32* handles,
                        hipStream_t s) {
     if (n == 0) return hipSuccess;
     const u32 grid = grid_for(n, KEYS_PER_ROUND * (BLOCK / 64), 16384);
     if (vec4_ok(t, out)) {
         u32 units = t.dim / 4;
         pull_kernel<float4><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, reinterpret_cast<float4*>(out),
-                                                   hit, units, t.stride_f / 4, magic32(units));
+                                                   hit, handles, units, t.stride_f / 4, magic32(units));
     } else {
-        pull_kernel<float><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, out, hit, t.dim, t.stride_f,
+        pull_kernel<float><<<grid, BLOCK, 0, s>>>(t, keys, (u32)n, out, hit, handles, t.dim, t.stride_f,
                                                   magic32(t.dim));
     }
     return hipGetLastError();
 }
 
 hipError_t launch_gather_slots(const TableDev& t, const u64* keys, const u32* slot_idx, size_t n, float* out,
-                               uint8_t* hit, hipStream_t s) {
+                               uint8_t* hit, u32* handles, hipStream_t s) {
     if (n == 0) return hipSuccess;
     const u32 grid = grid_for(n, KEYS_PER_ROUND * (BLOCK / 64), 16384);
     if (vec4_ok(t, out)) {
         u32 units = t.dim / 4;
         gather_slots_kernel<float4><<<grid, BLOCK, 0, s>>>(t, keys, slot_idx, (u32)n,
-                                                           reinterpret_cast<float4*>(out), hit,
+                                                           reinterpret_cast<float4*>(out), hit, handles,
                                                            units, t.stride_f / 4, magic32(units));
     } else {
-        gather_slots_kernel<float><<<grid, BLOCK, 0, s>>>(t, keys, slot_idx, (u32)n, out, hit, t.dim,
+        gather_slots_kernel<float><<<grid, BLOCK, 0, s>>>(t, keys, slot_idx, (u32)n, out, hit, handles, t.dim,
                                                           t.stride_f, magic32(t.dim));
     }
     return hipGetLastError();

@@ -6,7 +6,7 @@
 // range of home buckets of the hash array. Three launches:
 //   1. part_tile_kernel     a workgroup per tile: finds the keys that repeat inside the tile (a hash
 //                           table in LDS), adds up their gradient rows into one pre-summed row per
-//                           key, and leaves one entry {key, reference} per distinct key of the tile,
+//                           key, and leaves one entry {key, reference, row handle} per distinct key of the tile,
 //                           grouped by partition, in the tile's staging block, with the place where
 //                           each partition's entries start in the block; a reference is the batch
 //                           index of the gradient row or the number of a pre-summed row.
@@ -46,7 +46,9 @@ constexpr u32 NONE32 = 0xFFFFFFFFu;
 constexpr u32 PA_BLOCK = 512, PA_ITEMS = 4, PA_CAP = PA_BLOCK * PA_ITEMS;  // entries a partition pass holds
 constexpr u32 PA_HT = 2 * PA_CAP;
 constexpr u32 PA_ACC_DOUBLES = PA_HT / 2;     // the room of the partition's hash table (16 KiB)
-constexpr u32 AUX_NEW = 0x80000000u;
+constexpr u32 AUX_NEW = 0x80000000u;     // in a distinct key's aux word: the key claimed a slot in this launch
+constexpr u32 AUX_SINGLE = 0x40000000u;  // the key has one entry (low 16 bits: where its reference lies)
+constexpr u32 AUX_MULTI_MASK = 0x3FFFu;  // bits 16..29 of a key with several entries: its list number
 
 // exclusive scan over the NT threads of the block (64-bit packed fields); all threads call it
 template <u32 NT>
@@ -88,6 +90,28 @@ __device__ __forceinline__ void dedupe_insert(u64 key, u32 q, u64 h, const u64* 
         s = (s + 1) & ht_mask;
     }
     arrival = atomicAdd(&cnt[rep], 1u);
+}
+
+// The same with the count kept in the table's word: owner[s] = item | arrivals << 16 (at most 2^15
+// items). `slot` is where the key's word lies, for the count to be read later.
+__device__ __forceinline__ void dedupe_insert_packed(u64 key, u32 q, u64 h, const u64* lkey, u32* owner,
+                                                     u32 ht_mask, u32& rep, u32& arrival, u32& slot) {
+    u32 s = (u32)(h >> 40) & ht_mask;
+    while (true) {
+        const u32 old = atomicCAS(&owner[s], NONE32, q | (1u << 16));
+        if (old == NONE32) {
+            rep = q;
+            arrival = 0;
+            break;
+        }
+        if (lkey[old & 0xFFFFu] == key) {
+            rep = old & 0xFFFFu;
+            arrival = atomicAdd(&owner[s], 1u << 16) >> 16;
+            break;
+        }
+        s = (s + 1) & ht_mask;
+    }
+    slot = s;
 }
 
 template <typename T>
@@ -203,8 +227,8 @@ constexpr u32 PT_LDS_FIXED = PT_OFF_HIST;  // 114688, then one word per partitio
 
 template <typename T>
 __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
-    TableDev t, const u64* __restrict__ keys, const T* __restrict__ grads, u32 n, u32 P, u32 part_shift,
-    uint4* __restrict__ stage, u32* __restrict__ starts, T* __restrict__ psum, u32 units) {
+    TableDev t, const u64* __restrict__ keys, const T* __restrict__ grads, const u32* __restrict__ handles, u32 n,
+    u32 P, u32 part_shift, uint4* __restrict__ stage, u32* __restrict__ starts, T* __restrict__ psum, u32 units) {
     extern __shared__ __align__(16) unsigned char pt_lds[];
     u64* lkey = reinterpret_cast<u64*>(pt_lds);
     u32* owner = reinterpret_cast<u32*>(pt_lds + PT_OFF_OWNER);
@@ -220,12 +244,19 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
     const u64 tb = (u64)tile * PT_TILE;
 
     u64 key[PT_ITEMS], hh[PT_ITEMS];
+    u32 hdl[PT_ITEMS];
     bool valid[PT_ITEMS];
     u32 nbad = 0;
 #pragma unroll
     for (u32 j = 0; j < PT_ITEMS; ++j) {  // no branch around a load: the four stay in flight together
         const u64 i = tb + j * PT_BLOCK + tid;
         key[j] = keys[i < n ? i : (u64)n - 1];
+    }
+#pragma unroll
+    for (u32 j = 0; j < PT_ITEMS; ++j) {
+        const u64 i = tb + j * PT_BLOCK + tid;
+        hdl[j] = ROW_NONE;
+        if (handles) hdl[j] = handles[i < n ? i : (u64)n - 1];  // (block-uniform branch)
     }
 #pragma unroll
     for (u32 j = 0; j < PT_ITEMS; ++j) {
@@ -361,7 +392,7 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
             const u64 pos = tb + hist[part[j]] + prank[j];
             const u32 ref = multi[j] ? (REF_PSUM | (tile * PT_MAX_MULTI + (aux[j * PT_BLOCK + tid] >> 16)))
                                      : (u32)(tb + j * PT_BLOCK + tid);
-            stage[pos] = make_uint4((u32)key[j], (u32)(key[j] >> 32), ref, 0u);
+            stage[pos] = make_uint4((u32)key[j], (u32)(key[j] >> 32), ref, hdl[j]);
         }
     if (n_multi == 0) return;  // block-uniform
 
@@ -395,12 +426,12 @@ __global__ __launch_bounds__(PT_BLOCK) void part_tile_kernel(
 }
 
 // ---- 2. apply -------------------------------------------------------------------------------------
-// LDS (dynamic, 72 KiB): entry keys | hash table (later the accumulators) | counts | aux |
+// LDS (dynamic, 72 KiB): entry keys | hash table (later the accumulators) | entry handles | aux |
 // entry references (later the rows of the distinct keys) | references grouped by key | list numbers |
 // distinct keys | keys with more than one entry.
 constexpr u32 PA_OFF_OWNER = PA_CAP * 8;
-constexpr u32 PA_OFF_CNT = PA_OFF_OWNER + PA_HT * 4;
-constexpr u32 PA_OFF_AUX = PA_OFF_CNT + PA_CAP * 4;
+constexpr u32 PA_OFF_HDL = PA_OFF_OWNER + PA_HT * 4;
+constexpr u32 PA_OFF_AUX = PA_OFF_HDL + PA_CAP * 4;
 constexpr u32 PA_OFF_LREF = PA_OFF_AUX + PA_CAP * 4;
 constexpr u32 PA_OFF_LIST = PA_OFF_LREF + PA_CAP * 4;
 constexpr u32 PA_OFF_LOWN = PA_OFF_LIST + PA_CAP * 4;
@@ -409,7 +440,7 @@ constexpr u32 PA_OFF_MREP = PA_OFF_UREP + PA_CAP * 2;
 constexpr u32 PA_LDS = PA_OFF_MREP + PA_CAP * 2;  // 75776
 
 struct ApplyArgs {
-    const uint4* stage;  // {key low, key high, reference, -}, a block of PT_TILE per tile
+    const uint4* stage;  // {key low, key high, reference, row handle}, a block of PT_TILE per tile
     const u32* starts;   // [tile][P + 1]: where each partition's entries start in the tile's block
     u32* pstart;         // out: entries in lower partitions (where the partition parks its new keys)
     u32 n_tiles, P;
@@ -419,6 +450,8 @@ struct ApplyArgs {
     u32 units;
     int insert;
     u32 cap;  // entries a pass holds: PA_CAP, or less when a test wants to see the passes
+    int handles;  // the entries carry rows that an earlier pull reported
+    int verify;   // ... which count only where row_keys agrees
 };
 
 // The optimizer step of the distinct keys of a pass: a key with one entry takes its gradient row, a
@@ -431,7 +464,6 @@ __device__ __forceinline__ void apply_keys(const TableDev& t, unsigned char* lds
                                            u32 NG, u32 g, u32 c, const double* acc, u32 n_summed) {
     constexpr u32 N = sizeof(T) / 4;
     constexpr int STATES = states_of<KIND>();
-    const u32* cnt = reinterpret_cast<const u32*>(lds + PA_OFF_CNT);
     const u32* aux = reinterpret_cast<const u32*>(lds + PA_OFF_AUX);
     const u32* urow = reinterpret_cast<const u32*>(lds + PA_OFF_LREF);
     const u32* list = reinterpret_cast<const u32*>(lds + PA_OFF_LIST);
@@ -456,11 +488,11 @@ __device__ __forceinline__ void apply_keys(const TableDev& t, unsigned char* lds
             if (u < U) {
                 const u32 i = urep[u];
                 const u32 av_ = aux[i];
-                if (cnt[i] == 1) {
+                if (av_ & AUX_SINGLE) {
                     single[k] = true;
                     ref = list[av_ & 0xFFFFu];
                 } else {
-                    mi = (av_ >> 16) & 0x7FFFu;
+                    mi = (av_ >> 16) & AUX_MULTI_MASK;
                     summed = mi < n_summed;
                     single[k] = summed;
                 }
@@ -513,7 +545,7 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
     constexpr u32 N = sizeof(T) / 4;
     u64* lkey = reinterpret_cast<u64*>(lds);
     u32* owner = reinterpret_cast<u32*>(lds + PA_OFF_OWNER);
-    u32* cnt = reinterpret_cast<u32*>(lds + PA_OFF_CNT);
+    const u32* lhdl = reinterpret_cast<const u32*>(lds + PA_OFF_HDL);
     u32* aux = reinterpret_cast<u32*>(lds + PA_OFF_AUX);
     u32* lref = reinterpret_cast<u32*>(lds + PA_OFF_LREF);
     u32* list = reinterpret_cast<u32*>(lds + PA_OFF_LIST);
@@ -525,20 +557,18 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
 
 #pragma unroll
     for (u32 x = 0; x < PA_HT / PA_BLOCK; ++x) owner[x * PA_BLOCK + tid] = NONE32;
-#pragma unroll
-    for (u32 j = 0; j < PA_ITEMS; ++j) cnt[j * PA_BLOCK + tid] = 0;
     __syncthreads();
 
-    u32 rep[PA_ITEMS], arr[PA_ITEMS];
+    u32 rep[PA_ITEMS], arr[PA_ITEMS], hslot[PA_ITEMS];
     bool valid[PA_ITEMS];
 #pragma unroll
     for (u32 j = 0; j < PA_ITEMS; ++j) {
         const u32 i = j * PA_BLOCK + tid;
         valid[j] = i < count;
-        rep[j] = arr[j] = 0;
+        rep[j] = arr[j] = hslot[j] = 0;
         if (valid[j]) {
             const u64 key = lkey[i];
-            dedupe_insert(key, i, hash64(key), lkey, owner, cnt, PA_HT - 1, rep[j], arr[j]);
+            dedupe_insert_packed(key, i, hash64(key), lkey, owner, PA_HT - 1, rep[j], arr[j], hslot[j]);
         }
     }
     __syncthreads();
@@ -549,7 +579,7 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
     u32 my_u = 0, my_multi = 0, my_len = 0;
 #pragma unroll
     for (u32 j = 0; j < PA_ITEMS; ++j) {
-        m[j] = valid[j] ? cnt[rep[j]] : 0u;
+        m[j] = valid[j] ? owner[hslot[j]] >> 16 : 0u;
         isrep[j] = valid[j] && rep[j] == j * PA_BLOCK + tid;
         my_u += isrep[j] ? 1u : 0u;
         my_multi += (isrep[j] && m[j] >= 2) ? 1u : 0u;
@@ -571,7 +601,7 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
                     ++mr;
                     lo += m[j];
                 } else {
-                    aux[i] = n_elems + (ur - mr);  // single entries follow the lists
+                    aux[i] = (n_elems + (ur - mr)) | AUX_SINGLE;  // single entries follow the lists
                 }
                 ++ur;
             }
@@ -583,7 +613,7 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
             const u32 av = aux[rep[j]];
             const u32 pos = (av & 0xFFFFu) + arr[j];
             list[pos] = lref[j * PA_BLOCK + tid];
-            lown[pos] = (u16)(av >> 16);
+            lown[pos] = (u16)((av >> 16) & AUX_MULTI_MASK);
         }
     // the hash table is done with: its room becomes the accumulators of the keys with several entries,
     // as many lists as it holds (normally all of them)
@@ -604,39 +634,68 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
 
     // One probe per distinct key, four lanes each. A lane group looks at the home buckets of
     // several keys at once (all the loads in flight together); a key that is not in its home
-    // bucket -- or must claim a slot -- then takes the ordinary walk.
+    // bucket -- or must claim a slot -- then takes the ordinary walk. A key whose entries carry the
+    // row an earlier pull found is not looked up at all (with `verify`: once row_keys has
+    // confirmed it, a load that goes out with the bucket loads of the other keys).
     u32* urow = lref;
     const u32 grp = lane >> 2, sub = lane & 3u;
     constexpr u32 KP = 4, QUADS = PA_BLOCK / 4;
+    const u32 rows_now = t.counters[CNT_ROWS];  // (this launch hands out no rows)
     for (u32 u0 = 0; u0 < U; u0 += QUADS * KP) {
-        u32 uu[KP], ii[KP];
-        u64 kk[KP];
-        bool act[KP];
-        uint4 sv[KP];
+        u32 uu[KP], ii[KP], hd[KP];
+        u64 kk[KP], vk[KP] = {};
+        bool act[KP], byh[KP];
+        uint4 sv[KP] = {};
+        bool any_lookup = false;
 #pragma unroll
         for (u32 k = 0; k < KP; ++k) {
             uu[k] = u0 + k * QUADS + (tid >> 2);
             act[k] = uu[k] < U;
             ii[k] = act[k] ? urep[uu[k]] : 0u;
             kk[k] = act[k] ? lkey[ii[k]] : KEY_EMPTY;
-            sv[k] = t.slots[(u64)((u32)hash64(kk[k]) & t.bucket_mask) * 4 + sub];
+            hd[k] = lhdl[ii[k]];
+            byh[k] = act[k] && a.handles && hd[k] < rows_now;
+            any_lookup |= act[k] && !byh[k];
         }
-        if (sums_due) {  // while the buckets are on their way: the sums of the keys with several entries
+        const bool wave_looks = __ballot(any_lookup) != 0;  // wavefront-uniform
+        if (wave_looks) {
+#pragma unroll
+            for (u32 k = 0; k < KP; ++k)  // (a lane group with a handle reads bucket 0 and drops it)
+                sv[k] = t.slots[(u64)(byh[k] ? 0u : ((u32)hash64(kk[k]) & t.bucket_mask)) * 4 + sub];
+        }
+        if (a.verify) {
+#pragma unroll
+            for (u32 k = 0; k < KP; ++k) vk[k] = t.row_keys[byh[k] ? hd[k] : 0u];
+        }
+        if (sums_due) {  // while the loads are on their way: the sums of the keys with several entries
             if (on) flat_sum<T>([&](u32 e) { return src(list[e]); }, lown, 0u, first_hi, 0u, acc, units, NG, g, c);
             sums_due = false;
         }
+        bool late[KP];  // a handle that row_keys does not confirm: looked up after all
 #pragma unroll
         for (u32 k = 0; k < KP; ++k) {
+            late[k] = false;
+            if (a.verify && byh[k] && vk[k] != kk[k]) {
+                byh[k] = false;
+                late[k] = true;
+            }
+            if (byh[k] && sub == 0) urow[uu[k]] = hd[k];
+        }
+        if (!wave_looks && !(a.verify && __ballot(late[0] || late[1] || late[2] || late[3]))) continue;
+#pragma unroll
+        for (u32 k = 0; k < KP; ++k) {
+            const bool look = act[k] && !byh[k];
             const u64 skey = ((u64)sv[k].y << 32) | sv[k].x;
-            const bool match = act[k] && skey == kk[k];
-            const bool empty = act[k] && skey == KEY_EMPTY;
+            const bool home = wave_looks && look && !late[k];  // sv[k] is the key's home bucket
+            const bool match = home && skey == kk[k];
+            const bool empty = home && skey == KEY_EMPTY;
             const u32 m4 = (u32)(__ballot(match) >> (grp * 4)) & 0xFu;
             const u32 e4 = (u32)(__ballot(empty) >> (grp * 4)) & 0xFu;
             const u32 srcl = grp * 4 + (m4 ? (u32)__ffs((int)m4) - 1u : 0u);
-            const u32 hrow = __shfl(sv[k].z, (int)srcl);
+            const u32 hrow = __shfl(wave_looks ? sv[k].z : 0u, (int)srcl);
             // found at home: done. Absent for sure (an empty slot at home) and nothing to insert: done.
-            const bool slow = act[k] && !m4 && (a.insert || !e4);
-            if (act[k] && sub == 0 && !slow) urow[uu[k]] = (m4 && hrow < t.max_rows) ? hrow : ROW_NONE;
+            const bool slow = look && (!home || (!m4 && (a.insert || !e4)));
+            if (look && sub == 0 && !slow) urow[uu[k]] = (m4 && hrow < t.max_rows) ? hrow : ROW_NONE;
             if (__ballot(slow)) {
                 u32 row = ROW_NONE, slot = SLOT_NONE;
                 bool won = false;
@@ -745,6 +804,7 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
     __shared__ u32 stk[24];
     u64* lkey = reinterpret_cast<u64*>(pa_lds);
     u32* lref = reinterpret_cast<u32*>(pa_lds + PA_OFF_LREF);
+    u32* lhdl = reinterpret_cast<u32*>(pa_lds + PA_OFF_HDL);
     u32* toff = reinterpret_cast<u32*>(pa_lds + PA_OFF_LIST);  // (the reference list is written later)
     u32* ta = toff + PA_TILES_MAX;
     const u32 tid = threadIdx.x;
@@ -777,6 +837,7 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
             if (i < np) {
                 lkey[i] = ((u64)e[j].y << 32) | e[j].x;
                 lref[i] = e[j].z;
+                lhdl[i] = e[j].w;
             }
         }
         __syncthreads();
@@ -814,6 +875,7 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
                         if (pos < a.cap) {
                             lkey[pos] = key;
                             lref[pos] = e.z;
+                            lhdl[pos] = e.w;
                         }
                     }
                 }
@@ -970,24 +1032,24 @@ hipError_t part_init() {
 }
 
 hipError_t launch_part_tile(const TableDev& t, const PartPlan& pl, const PartBufs& b, const uint64_t* keys,
-                            const float* grads, hipStream_t s) {
+                            const float* grads, const uint32_t* handles, hipStream_t s) {
     if ((t.dim % 4 == 0) && aligned16(grads))
         part_tile_kernel<float4><<<pl.n_tiles, PT_BLOCK, PT_LDS_FIXED + pl.P * 4, s>>>(
-            t, keys, reinterpret_cast<const float4*>(grads), pl.n, pl.P, pl.part_shift, b.stage, b.starts,
+            t, keys, reinterpret_cast<const float4*>(grads), handles, pl.n, pl.P, pl.part_shift, b.stage, b.starts,
             reinterpret_cast<float4*>(b.psum), t.dim / 4);
     else
         part_tile_kernel<float><<<pl.n_tiles, PT_BLOCK, PT_LDS_FIXED + pl.P * 4, s>>>(
-            t, keys, grads, pl.n, pl.P, pl.part_shift, b.stage, b.starts, b.psum, t.dim);
+            t, keys, grads, handles, pl.n, pl.P, pl.part_shift, b.stage, b.starts, b.psum, t.dim);
     return hipGetLastError();
 }
 
 hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads, bool insert,
-                             hipStream_t s) {
+                             bool handles, bool verify, hipStream_t s) {
     const bool v4 = (t.dim % 4 == 0) && aligned16(grads);
     u32 pow2 = 1;
     while (pow2 < pl.n_tiles) pow2 <<= 1;
     ApplyArgs a{b.stage, b.starts, b.pstart, pl.n_tiles, pl.P, pow2 / 2, b.new_slot, b.new_count,
-                v4 ? t.dim / 4 : t.dim, insert ? 1 : 0, g_part_cap};
+                v4 ? t.dim / 4 : t.dim, insert ? 1 : 0, g_part_cap, handles ? 1 : 0, (handles && verify) ? 1 : 0};
     if (v4)
         part_apply_kernel<float4><<<pl.P, PA_BLOCK, PA_LDS, s>>>(t, reinterpret_cast<const float4*>(grads),
                                                                  reinterpret_cast<const float4*>(b.psum),

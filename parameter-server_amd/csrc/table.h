@@ -107,9 +107,10 @@ inline SegGeom seg_geometry(uint32_t dim, uint32_t vec, uint64_t n) {
 
 hipError_t launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t s);
 
-// Fused probe + gather of pull without insertion. out is n x dim floats; hit may be null.
+// Fused probe + gather of pull without insertion. out is n x dim floats; hit may be null;
+// handles (may be null): handles[i] = row of keys[i], or ROW_NONE.
 hipError_t launch_pull(const TableDev& t, const uint64_t* keys, size_t n, float* out, uint8_t* hit,
-                       hipStream_t s);
+                       uint32_t* handles, hipStream_t s);
 
 // slot_out[i] = slot holding keys[i] or SLOT_NONE; idx_out[i] = i when idx_out is not null.
 // won_count != null: claim a slot for each missing key (insert). The claiming occurrence has the
@@ -132,7 +133,7 @@ hipError_t launch_assign_rows(const TableDev& t, const uint64_t* keys, size_t n,
 
 // Gather through located slots (pull with insertion); hit = row existed when the pull began.
 hipError_t launch_gather_slots(const TableDev& t, const uint64_t* keys, const uint32_t* slot_idx, size_t n, float* out,
-                               uint8_t* hit, hipStream_t s);
+                               uint8_t* hit, uint32_t* handles, hipStream_t s);
 
 // Undo of a batch of claims: every located slot whose row is >= first_new_row (or unset) is
 // emptied, the counters are restored.
@@ -196,17 +197,20 @@ struct PartSizes {
     size_t stage, starts, pstart, psum, new_slot, new_count, ngrad;
 };
 struct PartBufs {
-    uint4* stage;  // entries {key low, key high, reference, -}: a block per tile, grouped by partition
+    uint4* stage;  // entries {key low, key high, reference, row handle}: a block per tile, grouped by partition
     uint32_t *starts, *pstart, *new_slot, *new_count;
     float *psum, *ngrad;
 };
 bool part_plan(const TableDev& t, size_t n, PartPlan* plan);
 PartSizes part_sizes(uint32_t dim, size_t n);
 hipError_t part_init();  // once per device, before the first launch
+// handles (may be null): the row of every key as an earlier pull of the same keys reported it
+// (ROW_NONE where it found none); the apply kernel then looks up only the keys without one.
+// verify: a handle counts only if row_keys[handle] is the key.
 hipError_t launch_part_tile(const TableDev& t, const PartPlan& pl, const PartBufs& b, const uint64_t* keys,
-                            const float* grads, hipStream_t s);
+                            const float* grads, const uint32_t* handles, hipStream_t s);
 hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads, bool insert,
-                             hipStream_t s);
+                             bool handles, bool verify, hipStream_t s);
 hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads,
                               hipStream_t s);
 // Entries a pass of the apply kernel takes (0 = the default, 2048): a test hook that makes small
