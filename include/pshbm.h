@@ -432,6 +432,20 @@ int32_t pshbm_debug_sort_spin_limit(uint32_t polls);
  * kernel takes (0 = the default, 2048). A small value makes ordinary batches go through the
  * several-passes path that otherwise only partitions crowded by hot keys take. Process-wide. */
 int32_t pshbm_debug_part_pass_capacity(uint32_t entries);
+/* Test hook, no counterpart in the reference: the library's stable radix sort of (key, value) pairs
+ * by the low key_bits bits of the key, on its own (a push uses it on (row, batch index) pairs when
+ * it does not take the partitioned path). Both array pairs are device memory of n words each and
+ * scratch for the sort; the sorted pairs end in (d_keys_tmp, d_vals_tmp) when *result_in_tmp is 1,
+ * else in (d_keys, d_vals). Synchronous; allocates and frees its own temporary memory. PSHBM_FATAL
+ * if a tile's bounded wait ran out (the output is then not sorted). */
+int32_t pshbm_debug_sort_pairs(int32_t device, uint32_t* d_keys, uint32_t* d_vals, uint32_t* d_keys_tmp,
+                               uint32_t* d_vals_tmp, size_t n, uint32_t key_bits, int32_t* result_in_tmp,
+                               void* stream);
+/* Test hook, no counterpart in the reference: how many markers of erased keys a hash array of
+ * `slots` slots under a table of at most `max_rows` keys may hold before an erase rebuilds it (an
+ * eighth of the slots, less where a full table plus the markers would pass 95 % of the slots). Pure
+ * arithmetic, no device. */
+uint64_t pshbm_debug_tombstone_limit(uint64_t slots, uint64_t max_rows);
 
 /* Pinned (page-locked) host memory for request/response buffers of the host-pointer entry points.
  * Buffers from here (or from hipHostMalloc) spare the staging copies: pshbm_pull and pshbm_push

@@ -36,6 +36,7 @@ SYMBOLS = [
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
     "pshbm_push_dev_noalloc", "pshbm_pull_dev_handles", "pshbm_push_dev_handles", "pshbm_debug_sort_spin_limit", "pshbm_debug_part_pass_capacity",
+    "pshbm_debug_tombstone_limit", "pshbm_debug_sort_pairs",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
           "fixup_windows", "assign_rows", "push_small", "part_tile", "part_apply", "part_insert"]
@@ -189,6 +190,9 @@ def lib():
         L.pshbm_push_dev_handles.argtypes = [vp, vp, vp, vp, C.c_uint64, sz, u32, vp]
         L.pshbm_debug_sort_spin_limit.argtypes = [u32]
         L.pshbm_debug_part_pass_capacity.argtypes = [u32]
+        L.pshbm_debug_sort_pairs.argtypes = [C.c_int32, vp, vp, vp, vp, sz, u32, C.POINTER(C.c_int32), vp]
+        L.pshbm_debug_tombstone_limit.argtypes = [C.c_uint64, C.c_uint64]
+        L.pshbm_debug_tombstone_limit.restype = C.c_uint64
         L.pshbm_push_pairs.argtypes = [vp, vp, sz, sz, u32]
         L.pshbm_queue.argtypes = [vp, vp, vp, sz]
         L.pshbm_queue_dev.argtypes = [vp, vp, vp, sz, vp]

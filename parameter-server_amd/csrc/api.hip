@@ -771,6 +771,17 @@ int32_t compact_locked(pshbm_table* t, hipStream_t s) {
     return PSHBM_OK;
 }
 
+// Markers of erased keys occupy slots until the hash array is rebuilt, and inserts never reuse
+// them: live keys + markers together must leave the array room to end a probe. The array is
+// rebuilt when the markers pass an eighth of the slots, or earlier when a full table (max_rows
+// keys) plus the markers would pass 95 % of the slots -- with max_load_factor 0.9 that is a
+// twentieth of the slots.
+uint64_t tombstone_limit(uint64_t slots, uint64_t max_rows) {
+    const uint64_t eighth = slots / 8, ceiling = slots - slots / 20;
+    const uint64_t room = ceiling > max_rows ? ceiling - max_rows : 0;
+    return room < eighth ? room : eighth;
+}
+
 // Removes the rows flagged in ms_dead (one byte per row of the `rows` stored). The lock is held.
 int32_t erase_flagged(pshbm_table* t, uint32_t rows, hipStream_t s, uint64_t* erased) {
     uint8_t* dead = static_cast<uint8_t*>(t->ms_dead.p);
@@ -789,7 +800,7 @@ int32_t erase_flagged(pshbm_table* t, uint32_t rows, hipStream_t s, uint64_t* er
                                   static_cast<uint32_t*>(t->ms_lists.p), s));
     HIP_TRY(t, hipStreamSynchronize(s));
     t->tombstones += gone;
-    if (t->tombstones > t->nbuckets * 4 / 8) ST_TRY(compact_locked(t, s));
+    if (t->tombstones > tombstone_limit(t->nbuckets * 4, t->d.max_rows)) ST_TRY(compact_locked(t, s));
     return PSHBM_OK;
 }
 
@@ -1958,6 +1969,41 @@ int32_t pshbm_debug_sort_spin_limit(uint32_t polls) {
     sort_set_spin_limit(polls);
     return PSHBM_OK;
 }
+
+int32_t pshbm_debug_sort_pairs(int32_t device, uint32_t* d_keys, uint32_t* d_vals, uint32_t* d_keys_tmp,
+                               uint32_t* d_vals_tmp, size_t n, uint32_t key_bits, int32_t* result_in_tmp,
+                               void* stream) {
+    if (!d_keys || !d_vals || !d_keys_tmp || !d_vals_tmp || !result_in_tmp || key_bits == 0 || key_bits > 32)
+        return PSHBM_ERROR;
+    if (n == 0) {
+        *result_in_tmp = 0;
+        return PSHBM_OK;
+    }
+    DeviceGuard g(device);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t temp_bytes = sort_pairs_temp_bytes(n);
+    void* temp = nullptr;
+    uint32_t* err = nullptr;
+    if (hipMalloc(&temp, temp_bytes) != hipSuccess) return PSHBM_OUT_OF_MEMORY;
+    if (hipMalloc(reinterpret_cast<void**>(&err), 4) != hipSuccess) {
+        (void)hipFree(temp);
+        return PSHBM_OUT_OF_MEMORY;
+    }
+    bool in_b = false;
+    uint32_t h_err = 0;
+    hipError_t e = hipMemsetAsync(temp, 0, sort_pairs_head_bytes(), s);
+    if (e == hipSuccess) e = hipMemsetAsync(err, 0, 4, s);
+    if (e == hipSuccess) e = sort_pairs(temp, temp_bytes, 0, d_keys, d_keys_tmp, d_vals, d_vals_tmp, n, key_bits, &in_b, err, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(&h_err, err, 4, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    (void)hipFree(temp);
+    (void)hipFree(err);
+    *result_in_tmp = in_b ? 1 : 0;
+    if (e != hipSuccess) return PSHBM_ERROR;
+    return h_err ? PSHBM_FATAL : PSHBM_OK;
+}
+
+uint64_t pshbm_debug_tombstone_limit(uint64_t slots, uint64_t max_rows) { return tombstone_limit(slots, max_rows); }
 
 int32_t pshbm_debug_part_pass_capacity(uint32_t entries) {
     part_set_pass_capacity(entries);

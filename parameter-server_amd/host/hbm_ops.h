@@ -25,6 +25,7 @@
 #include <algorithm>
 #include <functional>
 #include <memory>
+#include <mutex>
 
 #include "../../include/pshbm.h"
 #include "standin.h"
@@ -94,6 +95,7 @@ public:
             return false;
         }
         _shards[shard_id] = t;
+        _locks[shard_id];  // (map nodes stay where they are: the mutex may be held while other shards come and go)
         _capacity[shard_id] = cfg.expected_max_items;
         _vf = pshbm_value_floats(cfg.dim, cfg.optimizer);
         _dim = cfg.dim;
@@ -106,10 +108,19 @@ public:
         _shards.erase(it);
         return true;
     }
+    // The exclusive side of the shard lock that the reference's push and store take
+    // (SparsePushOperator.h:220,343: shard.lock()): held by an operator from the moment it hands its
+    // hyperparameters to the shard's table until its block is applied (and the table grown, if it
+    // had to be), so that server threads pushing to one shard neither race on this object's
+    // bookkeeping nor apply a block with another operator's hyperparameters. The table's own
+    // calls are thread-safe without it.
+    std::unique_lock<std::mutex> lock_shard(int32_t shard_id) { return std::unique_lock<std::mutex>(_locks.at(shard_id)); }
+
     // A hash map of the reference grows inside the insert that needs the room (safe_insert,
     // KVShardStorage.h:791-801) until the memory limit makes it unhealthy; a table grows when an
     // operator finds it full: twice the capacity at a time, up to op_config
-    // `hbm_table.grow_limit` keys (0, the default: never). False = no room to be had.
+    // `hbm_table.grow_limit` keys (0, the default: never). False = no room to be had. The caller
+    // holds lock_shard(shard_id).
     bool grow(int32_t shard_id) {
         const uint64_t limit = (uint64_t)_config.number("hbm_table.grow_limit", 0);
         pshbm_table* t = get(shard_id);
@@ -126,6 +137,7 @@ public:
     // operator's config, pico-ps/operator/Operator.h:53-57): handed to the table when they differ
     // from the ones it has. Operators with different hyperparameters must not push to one table at
     // the same time (the reference advises against changing a registered operator's config at all).
+    // The caller holds lock_shard(shard_id).
     void use_hyperparameters(int32_t shard_id, const pshbm_hyperparameters& hp) {
         auto it = _hp.find(shard_id);
         if (it != _hp.end() && std::memcmp(&it->second, &hp, sizeof hp) == 0) return;
@@ -169,6 +181,7 @@ public:
 private:
     Configure _config;
     std::map<int32_t, pshbm_table*> _shards;
+    std::map<int32_t, std::mutex> _locks;
     std::map<int32_t, uint64_t> _capacity;  // keys each shard's table holds at most
     std::map<int32_t, pshbm_hyperparameters> _hp;  // what each shard's table was last given
     uint32_t _dim = 0, _vf = 0;
@@ -282,6 +295,7 @@ public:
         Status status;
         auto& st = *static_cast<HbmShardStorage*>(storage);
         for_each_block(rt, req, storage, [&](int32_t shard_id, pshbm_table* t, const std::vector<char>& block, int32_t n, size_t stride) {
+            auto lk = st.lock_shard(shard_id);  // shard.lock(), :220
             if (_has_hp) st.use_hyperparameters(shard_id, _hp);
             int32_t rc = pshbm_push_pairs(t, block.data(), n, stride, 0);
             while (rc == PSHBM_OUT_OF_MEMORY && st.grow(shard_id)) rc = pshbm_push_pairs(t, block.data(), n, stride, 0);
@@ -315,6 +329,7 @@ public:
         resp << Status();
         send_response(std::move(resp));
         if (delta_storage == nullptr) return;  // :336-341
+        auto lk = static_cast<HbmShardStorage*>(storage)->lock_shard(shard_id);  // shard.lock(), :343
         if (_has_hp) static_cast<HbmShardStorage*>(storage)->use_hyperparameters(shard_id, _hp);
         pshbm_store(static_cast<HbmShardStorage*>(storage)->get(shard_id), 0);
     }
@@ -926,6 +941,7 @@ public:
             PSHBM_SCHECK(ar.readable() >= (size_t)shard_items * rec, "sync block size mismatch");
             if (status.ok() && shard_items > 0) {
                 pshbm_table* t = st.get(shard_id);
+                auto lk = st.lock_shard(shard_id);
                 int32_t rc = pshbm_load(t, ar.cursor(), (size_t)shard_items, 0);
                 while (rc == PSHBM_OUT_OF_MEMORY && st.grow(shard_id)) rc = pshbm_load(t, ar.cursor(), (size_t)shard_items, 0);
                 if (rc == PSHBM_OUT_OF_MEMORY) status = Status::OOM("PServer OOM during sync op");

@@ -5,10 +5,12 @@
 // synchronously, the store is applied, the table is dumped to files, restored into a new storage,
 // and pulled. The test operator of the reference (TestValue{sum,count}, TestOps.h:53-118) is the
 // dim-2 SUM table: a push of arg = key is the gradient [key, 1].
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <fstream>
 #include <iostream>
+#include <thread>
 
 #include "../../parameter-server_amd/host/hbm_ops.h"
 
@@ -533,6 +535,55 @@ static void test_operator_hyperparameters() {
     for (size_t i = 0; i < keys.size(); ++i) EXPECT(v[i * 2] == -1.25f && v[i * 2 + 1] == -1.25f);
 }
 
+// Several server threads push to the same shards at once (the reference runs apply_async_push_request
+// on its c2s threads and serialises them per shard with shard.lock(), SparsePushOperator.h:220):
+// two operators with different learning rates, a table that has to grow on the way. Each block is
+// applied whole with the rate of the operator that brought it, so with gradients of 1 the weight of
+// every key ends at -(pushes_fast * 0.5 + pushes_slow * 0.25) whatever the interleaving.
+static void test_threaded_pushes() {
+    Configure cfg;
+    cfg.set("dim", 2);
+    cfg.set("optimizer", "sgd");
+    cfg.set("lr", 0.5);
+    cfg.set("hbm_table.expected_max_items", 64);
+    cfg.set("hbm_table.grow_limit", 4096);
+    RuntimeInfo rt(0, {0, 1});
+    HbmStorageOperator storage_op(cfg);
+    std::unique_ptr<Storage> storage = storage_op.create_storage(rt, 0);
+    Configure slow = cfg;
+    slow.set("lr", 0.25);
+    HbmSparsePushOperator push_fast(cfg), push_slow(slow);
+    HbmSparsePullOperator pull_op(cfg);
+    constexpr int THREADS = 6, ROUNDS = 8, KEYS = 600;
+    std::vector<uint64_t> keys;
+    std::vector<float> args;
+    for (int k = 0; k < KEYS; ++k) {
+        keys.push_back(1000 + k);
+        args.push_back(1.0f);  // gradient [arg, 1]
+    }
+    std::atomic<int> failures{0};
+    std::vector<std::thread> pool;
+    for (int th = 0; th < THREADS; ++th)
+        pool.emplace_back([&, th] {
+            HbmSparsePushOperator& op = (th % 2 == 0) ? push_fast : push_slow;
+            for (int r = 0; r < ROUNDS; ++r) {
+                PSRequest req = make_push_request(keys, args);
+                PSResponse resp;
+                Status status;
+                op.apply_async_push_request(rt, req, storage.get(), nullptr, resp);
+                resp >> status;
+                if (!status.ok()) ++failures;
+            }
+        });
+    for (auto& t : pool) t.join();
+    EXPECT(failures.load() == 0);
+    bool ok;
+    auto v = pull(pull_op, rt, storage.get(), keys, &ok);
+    EXPECT(ok);
+    const float want = -(THREADS / 2 * ROUNDS * 0.5f + THREADS / 2 * ROUNDS * 0.25f);
+    for (size_t i = 0; i < keys.size(); ++i) EXPECT(v[i * 2] == want && v[i * 2 + 1] == want);
+}
+
 // hbm_table.init_range: a pull that misses answers the weights an insertion would store; a push
 // of a new key takes its step from them (init_store_value, SparsePullOperator.h:217,307-310).
 static void test_initial_weights() {
@@ -900,6 +951,7 @@ int main(int argc, char** argv) {
     test_dense(dir);
     test_growth();
     test_operator_hyperparameters();
+    test_threaded_pushes();
     test_initial_weights();
     test_memory_limit();
     test_sync();

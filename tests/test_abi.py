@@ -72,3 +72,17 @@ def test_memory_limit_is_kept_per_device_without_a_gpu(ps):
             assert e.status == ps.INVALID_ID
         else:
             raise AssertionError("a device ordinal out of range was accepted")
+
+
+def test_marker_limit_keeps_room_in_the_hash_array(ps):
+    """Markers of erased keys are never reused by inserts: a full table plus its markers must stay
+    below 95 % of the slots whatever max_load_factor (up to 0.9) put the capacity at."""
+    lim = ps.lib().pshbm_debug_tombstone_limit
+    assert lim(1 << 20, 1 << 19) == (1 << 20) // 8                 # load factor 0.5: an eighth of the slots
+    assert lim(1 << 20, 940_000) == (1 << 20) - (1 << 20) // 20 - 940_000   # 0.9: what is left below 95 %
+    assert lim(1 << 20, 1 << 20) == 0
+    for slots in (1 << 10, 1 << 20, 1 << 28):
+        for lf in (0.1, 0.5, 0.75, 0.875, 0.9):
+            rows = int(slots * lf)
+            assert rows + lim(slots, rows) <= slots - slots // 20
+            assert lim(slots, rows) <= slots // 8

@@ -291,3 +291,71 @@ def test_c2_size_for_each_and_erase_if(ps, wl):
     assert bool(hit.all()) and torch.equal(out, vu - 0.5)
     print(f"\nfor_each over {n_table} rows: {dt_all * 1e3:.2f} ms; erase_if of {n_sel} rows: {dt_erase * 1e3:.2f} ms")
     t.close()
+
+
+def test_c1_size_pulls_match_the_closed_form(ps, wl):
+    """C1: 1M keys, dim 8, read-only serving: 100 pulls of 65,536 uniform keys each, a tenth of
+    them absent, every pulled row and every hit flag against the closed form; then the same keys
+    again (a pull changes nothing)."""
+    n_table, dim, batch = 1_000_000, 8, 65_536
+    t = build(ps, wl, n_table, dim, dict(optimizer=1, lr=0.01), batch, 16)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    first = None
+    for step in range(100):
+        idx = torch.randint(0, n_table + n_table // 9, (batch,), device="cuda", generator=gen)   # a tenth absent
+        keys = wl.keys_of_index_torch(idx, 0)
+        out, hit = pull(t, keys, dim)
+        present = idx < n_table
+        assert torch.equal(hit.bool(), present)
+        want = closed_form(idx, dim, dim)
+        want[~present] = 0.0
+        assert torch.equal(out, want)
+        if step == 0:
+            first = (keys, out)
+    out, _ = pull(t, first[0], dim)
+    assert torch.equal(out, first[1]) and t.size() == n_table
+    t.close()
+
+
+def test_c3_size_adagrad_against_float64(ps, wl):
+    """C3: 50M keys, dim 64 + 64 accumulators, Adagrad, 2M-key Zipf(1.2) batches (the hottest key
+    about 200,000 times). The gradients are multiples of 0.25, so their sums are exact in any order
+    and the update is one float64 formula per element; the pull before and after goes with row
+    handles, the second push takes them."""
+    n_table, dim, batch = 50_000_000, 64, 2_000_000
+    lr, acc0 = 0.05, 0.1
+    t = build(ps, wl, n_table, dim, dict(optimizer=2, lr=lr, init_acc=acc0), batch, 2 * batch, state_fill=acc0)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(8)
+    stream = torch.cuda.current_stream().cuda_stream
+    idx = zipf_indices(wl, gen, n_table, 1.2, batch)
+    keys = wl.keys_of_index_torch(idx, 0)
+    out = torch.empty(batch, dim, device="cuda")
+    handles = torch.empty(batch, dtype=torch.int32, device="cuda")
+    st, epoch = t.pull_dev_handles(keys.data_ptr(), batch, out.data_ptr(), handles.data_ptr(), None, 0, stream)
+    assert st == 0, t.last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(out, closed_form(idx, dim, dim))
+
+    g = torch.randint(-3, 4, (batch, dim), device="cuda", generator=gen).to(torch.float32) * 0.25
+    push(t, keys, g)                                   # the plain push
+    uniq, acc = summed_by_index(idx, g)
+    n1 = acc0 + acc * acc
+    w1 = closed_form(uniq, dim, dim).to(torch.float64) - lr * acc / torch.sqrt(n1)
+    got, hit = pull(t, wl.keys_of_index_torch(uniq, 0), dim)
+    assert bool(hit.all())
+    err = (got.to(torch.float64) - w1).abs()
+    assert bool((err <= 1e-7 + 1e-6 * w1.abs()).all()), float(err.max())
+
+    # the same batch again through the handles of the first pull (rows have not moved)
+    st = t.push_dev_handles(keys.data_ptr(), g.data_ptr(), handles.data_ptr(), epoch, batch, 0, stream)
+    assert st == 0, t.last_error()
+    torch.cuda.synchronize()
+    n2 = n1 + acc * acc
+    w2 = w1 - lr * acc / torch.sqrt(n2)
+    got, hit = pull(t, wl.keys_of_index_torch(uniq, 0), dim)
+    err = (got.to(torch.float64) - w2).abs()
+    assert bool((err <= 2e-7 + 2e-6 * w2.abs()).all()), float(err.max())   # two rounded steps
+    assert t.size() == n_table
+    t.close()

@@ -566,6 +566,41 @@ def test_erase_many_rounds_triggers_rebuild(ps, orc, wl):
     t.close()
 
 
+def test_fill_erase_refill_on_a_tight_hash_array(ps, orc, wl):
+    """A capacity that puts the hash array at 90 % load (940,000 keys in 2^20 slots): filled to the
+    brim, an eighth of the slots' worth of keys erased, as many new keys inserted. Markers of
+    erased keys are not reused by inserts, so without an earlier rebuild live keys + markers would
+    fill every slot and a probe could neither end nor insert."""
+    rng = np.random.default_rng(21)
+    cap = 940_000
+    t = ps.Table(2, capacity=cap, max_load_factor=0.9, **OPTS["sum"])
+    r = orc.Oracle(2, capacity=cap, **OPTS["sum"])
+    assert t.stats().slots == 1 << 20
+    keys = wl.table_keys_np(0, cap, seed=12)
+    vals = rng.integers(-5, 6, (cap, 2)).astype(np.float32)
+    for lo in range(0, cap, 235_000):
+        assert t.set(keys[lo:lo + 235_000], vals[lo:lo + 235_000]) == 0
+        assert r.set(keys[lo:lo + 235_000], vals[lo:lo + 235_000]) == 0
+    assert t.size() == cap
+    n = (1 << 20) // 8
+    gone = keys[rng.permutation(cap)[:n]]
+    assert t.erase(gone) == r.erase(gone) == (0, n)
+    fresh = wl.fresh_keys_np(rng, n)
+    g = rng.integers(-3, 4, (n, 2)).astype(np.float32)
+    assert t.push(fresh, g) == 0, t.last_error()       # insert-on-miss through the partitioned push
+    assert r.push(fresh, g) == 0
+    assert t.size() == r.size() == cap
+    q = np.concatenate([fresh[:5000], gone[:5000], keys[:5000]])
+    st, rows, hit = t.pull(q)
+    st2, rows2, hit2 = r.pull(q)
+    assert st == st2 == 0
+    np.testing.assert_array_equal(hit, hit2)
+    np.testing.assert_array_equal(rows, rows2)
+    assert t.push(wl.fresh_keys_np(rng, 20000), np.ones((20000, 2), np.float32)) == ps.OUT_OF_MEMORY
+    assert_same_table(t, r, exact=True)
+    t.close()
+
+
 @pytest.mark.parametrize("opt,dim", [("ftrl", 16384), ("adagrad", 4097), ("sum", 16384)])
 def test_largest_rows(ps, orc, wl, opt, dim):
     """The largest dim the library takes (16384: rows of up to 192 KB with FTRL state) and an odd one
