@@ -226,7 +226,8 @@ int32_t pshbm_store_dev(pshbm_table* t, uint32_t flags, void* stream);
 /* Upsert of whole values: ht[key] = value for every item (safe_set, KVShardStorage.h:804-814).
  * Replaces DirectPushOperator::apply_async_push_request (SparsePushOperator.h:520-574), where
  * Load-with-rehash and the reshard shuffle land. values is n x pshbm_value_floats(); keys of one
- * call must be distinct. OUT_OF_MEMORY (:568-573) leaves the table unchanged. */
+ * call must be distinct (the value stored for a key that repeats is unspecified: each float comes
+ * from one of its items). OUT_OF_MEMORY (:568-573) leaves the table unchanged. */
 int32_t pshbm_set(pshbm_table* t, const uint64_t* keys, const float* values, size_t n);
 int32_t pshbm_set_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_values, size_t n,
                       void* stream);
@@ -238,8 +239,12 @@ int32_t pshbm_set_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_val
  * (pico-ps/operator/LoadOperator.h:164-213) once the file is decoded; with PSHBM_LOAD_UNIQUE a key
  * that is already present (or repeated) fails with PSHBM_ERROR the way restore aborts on it
  * (:194,210), and the records loaded before the failing block stay. Without the flag a key that
- * is present is overwritten, and of several records with one key any one may win. A record with a
- * reserved key is left out and the call returns PSHBM_ERROR after loading the others. */
+ * is present is overwritten. Records of one call should have distinct keys: where a key repeats
+ * within 32 MiB of records the stored value is unspecified (every float of it comes from one of the
+ * key's records, not necessarily all from the same one; the reference's sequential safe_set keeps
+ * the last), so a caller whose blocks may repeat a key keeps the last record of each first, as
+ * HbmDirectPushOperator does. A record with a reserved key is left out and the call returns
+ * PSHBM_ERROR after loading the others. */
 int32_t pshbm_load(pshbm_table* t, const void* records, size_t n, uint32_t flags);
 
 /* Bulk dump of every (key, value) as the same records, in row-slab order, the same way (written by

@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -490,6 +491,30 @@ int32_t reserve_rows(pshbm_table* t, size_t n, hipStream_t s, bool* checked, uin
     if (rows_upper_bound(t) + n <= t->d.max_rows) {
         book_insert(t, n);
         return PSHBM_OK;
+    }
+    // The bound counts every key of the batches still in flight as a new row. A caller that
+    // enqueues faster than the device runs gets many batches ahead, and the bound then passes the
+    // capacity long before the table does: wait for the device to publish the row counts of the
+    // oldest of them (a poll of the pinned word; the device keeps running, nothing is drained)
+    // rather than synchronise the stream. Bounded, because batches recorded into a graph that
+    // is being captured publish nothing until the graph runs.
+    if (!t->pending.empty()) {
+        const auto give_up = std::chrono::steady_clock::now() + std::chrono::milliseconds(20);
+        unsigned spins = 0;
+        while (!t->pending.empty()) {
+            if (rows_upper_bound(t) + n <= t->d.max_rows) {
+                book_insert(t, n);
+                return PSHBM_OK;
+            }
+            if ((++spins & 63u) == 0) {
+                if (std::chrono::steady_clock::now() > give_up) break;
+                std::this_thread::yield();
+            }
+        }
+        if (rows_upper_bound(t) + n <= t->d.max_rows) {
+            book_insert(t, n);
+            return PSHBM_OK;
+        }
     }
     ST_TRY(read_counters(t, s));
     set_exact_rows(t, t->h_counters[CNT_ROWS]);

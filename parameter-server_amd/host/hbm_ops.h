@@ -26,6 +26,7 @@
 #include <functional>
 #include <memory>
 #include <mutex>
+#include <unordered_map>
 
 #include "../../include/pshbm.h"
 #include "standin.h"
@@ -364,6 +365,35 @@ private:
     }
 };
 
+// Of the n records {uint64 key, value} of `rec` bytes each, in place: the last record of every key,
+// in the order of those last occurrences. Returns how many are left. (Blocks without a repeated
+// key -- the normal case -- are left as they are after one pass over the keys.)
+inline size_t keep_last_of_each_key(char* records, size_t n, size_t rec) {
+    std::unordered_map<uint64_t, size_t> last;
+    last.reserve(n * 2);
+    bool repeats = false;
+    for (size_t i = 0; i < n; ++i) {
+        uint64_t k;
+        std::memcpy(&k, records + i * rec, 8);
+        auto it = last.find(k);
+        if (it == last.end()) last.emplace(k, i);
+        else {
+            it->second = i;
+            repeats = true;
+        }
+    }
+    if (!repeats) return n;
+    size_t out = 0;
+    for (size_t i = 0; i < n; ++i) {
+        uint64_t k;
+        std::memcpy(&k, records + i * rec, 8);
+        if (last[k] != i) continue;
+        if (out != i) std::memmove(records + out * rec, records + i * rec, rec);
+        ++out;
+    }
+    return out;
+}
+
 // DirectPushOperator::apply_async_push_request, SparsePushOperator.h:520-574: every item is
 // {key, whole value}; ht[key] = value. OOM -> ELOGICERROR + Status::OOM (:568-573).
 class HbmDirectPushOperator {
@@ -386,7 +416,11 @@ public:
                 std::vector<char> ar;
                 ps_deserialize(req.lazy(), ar);
                 PSHBM_SCHECK(ar.size() == (size_t)shard_items_num * st.record_bytes(), "block size mismatch");
-                if (pshbm_load(st.get(shard_id), ar.data(), shard_items_num, 0) != PSHBM_OK) healthy = false;
+                // The reference sets the items one after the other, so the last item of a key stays
+                // (:548-560). pshbm_load wants distinct keys: keep the last record of each.
+                const size_t rec = st.record_bytes();
+                size_t kept = keep_last_of_each_key(ar.data(), (size_t)shard_items_num, rec);
+                if (pshbm_load(st.get(shard_id), ar.data(), kept, 0) != PSHBM_OK) healthy = false;
             }
         }
         PSHBM_SCHECK(req.archive().is_exhausted(), "request not exhausted");

@@ -907,7 +907,8 @@ int main(int argc, char** argv) {
     // direct push overwrites whole values (SparsePushOperator.h:557-562)
     {
         HbmDirectPushOperator direct(op_config);
-        std::vector<Pair> items = {{0, {7.0f, 8.0f}}, {1, {9.0f, 10.0f}}, {1000, {1.0f, 2.0f}}};
+        // (key 1 twice in one block: the later item stays, as after the reference's sequential safe_set)
+        std::vector<Pair> items = {{0, {7.0f, 8.0f}}, {1, {-1.0f, -2.0f}}, {1000, {1.0f, 2.0f}}, {1, {9.0f, 10.0f}}};
         PSRequest req;
         req << (int32_t)NUM_SHARDS << (int32_t)1;
         for (int32_t s = 0; s < NUM_SHARDS; ++s) {
