@@ -56,6 +56,19 @@ KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist"
 # must be counted again.
 TRAFFIC_FROM_PROFILES = {
     # (config, phase): (bytes, summary)
+    ("c1", "pull"): (19228672, "profiles/c1_pull_trace_and_hbm_counters.md"),
+    ("c2", "pull"): (196070400, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "part_tile"): (78893056, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "part_apply"): (158874624, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "pull"): (703215616, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "part_tile"): (452928512, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "part_apply"): (390892544, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "pull"): (585545728, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_tile"): (251302912, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_apply"): (637811712, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "pull"): (3204963328, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "part_tile"): (1380345856, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "part_apply"): (2715714560, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
 }
 
 
@@ -244,6 +257,8 @@ def cpu_baseline(cfg, wl, budget_keys):
         if cfg["opt"]["optimizer"] == 3:
             vals[:, 2 * dim:] = vals[:, dim:2 * dim] ** 2
         assert o.set(wl.table_keys_np(start, cnt, seed=0), vals) == 0
+        if (start // chunk) % 10 == 9:
+            print(f"cpu_baseline: {start + cnt} of {n} keys stored", file=sys.stderr, flush=True)
     steps, times = 4, []
     for s in range(steps):
         if cfg["s"] is None:
@@ -261,9 +276,12 @@ def cpu_baseline(cfg, wl, budget_keys):
     o.close()
     return {
         "value": keys_per_step / per_step, "unit": "keys/s", "cores": 1, "kind": "port",
-        "sample": f"{n}-key table (of {cfg['n']}: building the full table in a std::unordered_map takes "
-                  f"minutes, this leg is bounded to about 30 s; a smaller table only helps the CPU's caches), "
-                  f"median of {steps - 1} steps of {k}-key batches, oracle/ps_oracle.cpp single thread",
+        "sample": (f"the full {n}-key table" if n == cfg["n"] else
+                   f"{n}-key table (of {cfg['n']}: the two full tables of this leg take 3.5 minutes to build in "
+                   f"std::unordered_map, so the default run is bounded to about 30 s of CPU work; a smaller table "
+                   f"only helps the CPU's caches -- C2 measured once with --cpu-keys 100000000 on the same host: "
+                   f"8.0 M keys/s on one thread, 87.8 M keys/s on 16 shards)") +
+                  f", median of {steps - 1} steps of {k}-key batches, oracle/ps_oracle.cpp single thread",
         "sharded": cpu_baseline_sharded(cfg, wl, n, oracle, np),
     }
 
@@ -292,6 +310,8 @@ def cpu_baseline_sharded(cfg, wl, n, oracle, np):
         for s in range(S):
             m = which == s
             assert shards[s].set(keys[m], vals[m]) == 0
+        if (start // chunk) % 10 == 9:
+            print(f"cpu_baseline, {S} shards: {start + cnt} of {n} keys stored", file=sys.stderr, flush=True)
 
     def apply(job):
         o, keys, grads = job
@@ -399,7 +419,11 @@ def measure(name, args, torch, ps, wl, steps, warmup, headline):
     # the kernel that takes the most time per step (all its launches of a step together)
     dominant = max(phases, key=lambda p: phases[p]["ms_per_step"])
     achieved = phases[dominant]["algorithmic_GBps"]
-    traffic = TRAFFIC_FROM_PROFILES.get((name, dominant)) if n_table == cfg["n"] else None
+    # (the profiled runs were at full table size, with row handles)
+    profiled = n_table == cfg["n"] and (handles is not None or cfg["pull_only"])
+    traffic = TRAFFIC_FROM_PROFILES.get((name, dominant)) if profiled else None
+    step_traffic = [TRAFFIC_FROM_PROFILES.get((name, ph)) for ph in phases if ph != "part_insert"]
+    step_traffic = sum(x[0] for x in step_traffic) if profiled and all(step_traffic) else None
     roofline = {"kernel": KERNEL_OF_PHASE[dominant], "bound": "hbm", "achieved": achieved,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic[0] if traffic else None,
@@ -421,6 +445,8 @@ def measure(name, args, torch, ps, wl, steps, warmup, headline):
         "step_algorithmic_GBps": round(step_bytes / (ms_per_step * 1e6), 1),
         "step_frac_of_hbm_peak": round(step_bytes / (ms_per_step * 1e6) / HBM_PEAK_GBS, 4),
         "kernel_ms_per_step": round(sum(p["ms_per_step"] for p in phases.values()), 5),
+        "step_traffic_bytes_from_profiles": step_traffic,
+        "step_traffic_over_algorithmic": round(step_traffic / step_bytes, 2) if step_traffic else None,
         "roofline": roofline,
         "phases": phases,
         "table_stats": table_stats(t),
