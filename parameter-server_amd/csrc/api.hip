@@ -388,7 +388,7 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
     HIP_TRY(t, hipMemset(t->ws_won.p, 0, t->ws_won.bytes));
     t->won_parity = 0;
     PartPlan probe_plan;
-    if (cap >= PART_MIN_KEYS && part_plan(t->d, std::min(cap, PART_MAX_KEYS), &probe_plan)) {
+    if (cap >= PART_MIN_KEYS && part_plan(t->d, std::min(cap, PART_MAX_KEYS), 1.0, &probe_plan)) {
         const size_t pk = std::min(cap, PART_MAX_KEYS);
         const PartSizes z = part_sizes(t->d.dim, pk);
         ST_TRY(ensure(t, t->pt_stage, z.stage));
@@ -479,6 +479,17 @@ void book_insert(pshbm_table* t, size_t n) {
     t->d.op_seq = t->op_seq;
     t->pending.emplace_back(t->op_seq, (uint32_t)n);
     t->pending_sum += n;
+}
+
+// Entries per key of the last partitioned push whose apply kernel has run (a tile leaves one entry per
+// distinct key it holds: 1 for batches without repeats, about 0.6 for the Zipf batches of the
+// benchmark), as that kernel left it in the pinned word; 1 before the first. A hint for the size of
+// the next push's partitions, nothing more.
+double part_entries_per_key(pshbm_table* t) {
+    const unsigned long long st = static_cast<volatile unsigned long long*>(t->h_pub)[1];
+    const uint32_t keys = (uint32_t)(st >> 32), entries = (uint32_t)st;
+    if (keys == 0 || entries == 0 || entries > keys) return 1.0;
+    return (double)entries / (double)keys;
 }
 
 // Capacity accounting without a device round trip in the common case: the bound above is exact up
@@ -620,7 +631,7 @@ int32_t push_with(pshbm_table* t, const Workspace& w, const uint64_t* d_keys, co
     // A large batch is cut into tiles and partitions (push_part.hip): no global sort, one probe per
     // distinct key. (Not in checked mode: it updates rows in the launch that claims slots.)
     PartPlan pl;
-    if (!unique && !checked && n <= w.part_keys && part_plan(t->d, n, &pl)) {
+    if (!unique && !checked && n <= w.part_keys && part_plan(t->d, n, part_entries_per_key(t), &pl)) {
         *used_part = true;
         // (the other paths look every key up anyway: handles only serve here)
         HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_TILE, launch_part_tile(t->d, pl, w.part, d_keys, d_grads, d_handles, s));
@@ -943,9 +954,11 @@ int32_t pshbm_create(const pshbm_config* cfg, pshbm_table** out) {
     CREATE_TRY(dev_malloc(t->device, reinterpret_cast<void**>(&t->d_hist), 17 * 8));
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_counters), CNT_WORDS * 4, hipHostMallocDefault));
     CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_hist), 17 * 8, hipHostMallocDefault));
-    CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_pub), 8, hipHostMallocDefault));
-    *t->h_pub = 0;
+    CREATE_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->h_pub), 16, hipHostMallocDefault));
+    t->h_pub[0] = 0;
+    t->h_pub[1] = 0;
     d.pub = t->h_pub;
+    d.part_stat = t->h_pub + 1;
     CREATE_TRY(hipStreamCreateWithFlags(&t->stream, hipStreamNonBlocking));
     CREATE_TRY(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));
     for (pshbm_table::PullLane& l : t->lanes) {

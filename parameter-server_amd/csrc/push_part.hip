@@ -45,6 +45,9 @@ constexpr u32 REF_PSUM = 0x80000000u;         // reference to a pre-summed row
 constexpr u32 NONE32 = 0xFFFFFFFFu;
 constexpr u32 PA_BLOCK = 512, PA_ITEMS = 4, PA_CAP = PA_BLOCK * PA_ITEMS;  // entries a partition pass holds
 constexpr u32 PA_HT = 2 * PA_CAP;
+// entries a partition should hold on average: short rows / longer ones (whose list sums take a
+// round of LDS accumulators per 2048 / dim lists, so that fuller partitions cost them rounds)
+constexpr double PART_TARGET = 1250.0, PART_TARGET_LONG_ROWS = 625.0;
 constexpr u32 PA_ACC_DOUBLES = PA_HT / 2;     // the room of the partition's hash table (16 KiB)
 constexpr u32 AUX_NEW = 0x80000000u;     // in a distinct key's aux word: the key claimed a slot in this launch
 constexpr u32 AUX_SINGLE = 0x40000000u;  // the key has one entry (low 16 bits: where its reference lies)
@@ -443,7 +446,7 @@ struct ApplyArgs {
     const uint4* stage;  // {key low, key high, reference, row handle}, a block of PT_TILE per tile
     const u32* starts;   // [tile][P + 1]: where each partition's entries start in the tile's block
     u32* pstart;         // out: entries in lower partitions (where the partition parks its new keys)
-    u32 n_tiles, P;
+    u32 n_tiles, P, n_keys;
     u32 search_step;     // half the power of two that n_tiles rounds up to
     u32* new_slot;
     u32* new_count;
@@ -818,6 +821,11 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
     if (tid == 0) {
         s_nnew = 0;
         a.pstart[p] = s;
+        // the last partition's block knows how many entries the tiles left in all: a hint for the
+        // partition size of the next push (read by the host when it plans that push)
+        if (p + 1 == a.P)
+            __hip_atomic_store(t.part_stat, ((unsigned long long)a.n_keys << 32) | (unsigned long long)(s + np),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     if (np == 0) {
         if (tid == 0) a.new_count[p] = 0;
@@ -988,14 +996,21 @@ u32 g_part_cap = PA_CAP;
 }
 void part_set_pass_capacity(uint32_t entries) { g_part_cap = entries == 0 || entries > PA_CAP ? PA_CAP : entries; }
 
-bool part_plan(const TableDev& t, size_t n, PartPlan* plan) {
+bool part_plan(const TableDev& t, size_t n, double entries_per_key, PartPlan* plan) {
     if (n < PART_MIN_KEYS || n > PART_MAX_KEYS) return false;
     const u32 vec = (t.dim % 4 == 0) ? 4u : 1u;
     if (t.dim / vec > PA_BLOCK) return false;  // a lane per 4 or 16 bytes of a row
     u32 bucket_bits = 0;
     while ((1ull << bucket_bits) <= t.bucket_mask) ++bucket_bits;
-    u32 lp = 6;  // at least 64 partitions, about 1024 keys each
-    while ((1ull << lp) * 1024 < n && lp < 12) ++lp;
+    // A workgroup of the apply kernel is a chain of dependent round trips whatever it holds, so a
+    // partition should fill a pass (PA_CAP entries) as far as it safely can: about PART_TARGET
+    // entries on average (half that for long rows), which leaves room for the spread between partitions and for the entries
+    // of a key that is met in every tile. At least 64 partitions, at most 4096.
+    if (!(entries_per_key > 0.0 && entries_per_key <= 1.0)) entries_per_key = 1.0;
+    const double entries = entries_per_key * (double)n;
+    u32 lp = 6;
+    const double target = t.dim <= 32 ? PART_TARGET : PART_TARGET_LONG_ROWS;
+    while ((double)(1ull << lp) * target < entries && lp < 12) ++lp;
     if (lp > bucket_bits) return false;  // a tiny table under a large batch: the sort path serves it
     plan->n = (u32)n;
     plan->n_tiles = (u32)((n + PT_TILE - 1) / PT_TILE);
@@ -1048,7 +1063,7 @@ hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBu
     const bool v4 = (t.dim % 4 == 0) && aligned16(grads);
     u32 pow2 = 1;
     while (pow2 < pl.n_tiles) pow2 <<= 1;
-    ApplyArgs a{b.stage, b.starts, b.pstart, pl.n_tiles, pl.P, pow2 / 2, b.new_slot, b.new_count,
+    ApplyArgs a{b.stage, b.starts, b.pstart, pl.n_tiles, pl.P, pl.n, pow2 / 2, b.new_slot, b.new_count,
                 v4 ? t.dim / 4 : t.dim, insert ? 1 : 0, g_part_cap, handles ? 1 : 0, (handles && verify) ? 1 : 0};
     if (v4)
         part_apply_kernel<float4><<<pl.P, PA_BLOCK, PA_LDS, s>>>(t, reinterpret_cast<const float4*>(grads),

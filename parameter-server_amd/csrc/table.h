@@ -52,6 +52,7 @@ struct TableDev {
     uint32_t* counters;  // CNT_WORDS
     uint8_t* dirty;      // max_rows bytes, or null: 1 = a push updated the row since the last take
     unsigned long long* pub;  // page-locked host word: {op_seq, rows} as the last inserting operation left them
+    unsigned long long* part_stat;  // page-locked host word: {keys, entries} of the last partitioned push
     uint32_t bucket_mask;
     uint32_t max_rows;
     uint32_t dim;       // weights per key
@@ -201,7 +202,9 @@ struct PartBufs {
     uint32_t *starts, *pstart, *new_slot, *new_count;
     float *psum, *ngrad;
 };
-bool part_plan(const TableDev& t, size_t n, PartPlan* plan);
+// entries_per_key: what the tiles of recent batches left per key (1 = no key repeats inside a tile);
+// partitions are sized so that a pass of the apply kernel is well filled but rarely overflows.
+bool part_plan(const TableDev& t, size_t n, double entries_per_key, PartPlan* plan);
 PartSizes part_sizes(uint32_t dim, size_t n);
 hipError_t part_init();  // once per device, before the first launch
 // handles (may be null): the row of every key as an earlier pull of the same keys reported it
