@@ -437,6 +437,12 @@ int32_t pshbm_debug_sort_spin_limit(uint32_t polls);
  * kernel takes (0 = the default, 2048). A small value makes ordinary batches go through the
  * several-passes path that otherwise only partitions crowded by hot keys take. Process-wide. */
 int32_t pshbm_debug_part_pass_capacity(uint32_t entries);
+/* Test hook, no counterpart in the reference: the smallest batch that takes the partitioned push
+ * (0 = the default, 513 keys: everything the one-launch push does not take). A large value sends
+ * batches of up to 4M keys through the sorted push (locate, radix sort, segmented reduce), which
+ * otherwise only serves batches of more than 4M keys, nearly full tables and
+ * pshbm_push_dev_noalloc. Process-wide. */
+int32_t pshbm_debug_part_min_keys(uint64_t keys);
 /* Test hook, no counterpart in the reference: the library's stable radix sort of (key, value) pairs
  * by the low key_bits bits of the key, on its own (a push uses it on (row, batch index) pairs when
  * it does not take the partitioned path). Both array pairs are device memory of n words each and

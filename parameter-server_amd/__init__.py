@@ -35,7 +35,7 @@ SYMBOLS = [
     "pshbm_increment_size", "pshbm_take_increment", "pshbm_for_each", "pshbm_for_each_write", "pshbm_erase_if", "pshbm_erase", "pshbm_erase_dev", "pshbm_compact", "pshbm_reserve", "pshbm_set_hyperparameters", "pshbm_set_memory_limit", "pshbm_device_memory",
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
-    "pshbm_push_dev_noalloc", "pshbm_pull_dev_handles", "pshbm_push_dev_handles", "pshbm_debug_sort_spin_limit", "pshbm_debug_part_pass_capacity",
+    "pshbm_push_dev_noalloc", "pshbm_pull_dev_handles", "pshbm_push_dev_handles", "pshbm_debug_sort_spin_limit", "pshbm_debug_part_pass_capacity", "pshbm_debug_part_min_keys",
     "pshbm_debug_tombstone_limit", "pshbm_debug_sort_pairs",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
@@ -190,6 +190,7 @@ def lib():
         L.pshbm_push_dev_handles.argtypes = [vp, vp, vp, vp, C.c_uint64, sz, u32, vp]
         L.pshbm_debug_sort_spin_limit.argtypes = [u32]
         L.pshbm_debug_part_pass_capacity.argtypes = [u32]
+        L.pshbm_debug_part_min_keys.argtypes = [C.c_uint64]
         L.pshbm_debug_sort_pairs.argtypes = [C.c_int32, vp, vp, vp, vp, sz, u32, C.POINTER(C.c_int32), vp]
         L.pshbm_debug_tombstone_limit.argtypes = [C.c_uint64, C.c_uint64]
         L.pshbm_debug_tombstone_limit.restype = C.c_uint64
@@ -261,6 +262,12 @@ def debug_sort_spin_limit(polls=0xFFFFFFFF):
 def debug_part_pass_capacity(entries=0):
     """Test hook: entries one pass of the partitioned push's apply kernel takes (0 = default)."""
     return lib().pshbm_debug_part_pass_capacity(entries)
+
+
+def debug_part_min_keys(keys=0):
+    """Test hook: smallest batch that takes the partitioned push (0 = default); a large value sends
+    mid-size batches through the sorted push."""
+    return lib().pshbm_debug_part_min_keys(keys)
 
 
 def init_weight(init_range, key, column):

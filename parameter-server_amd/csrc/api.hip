@@ -2043,6 +2043,11 @@ int32_t pshbm_debug_sort_pairs(int32_t device, uint32_t* d_keys, uint32_t* d_val
 
 uint64_t pshbm_debug_tombstone_limit(uint64_t slots, uint64_t max_rows) { return tombstone_limit(slots, max_rows); }
 
+int32_t pshbm_debug_part_min_keys(uint64_t keys) {
+    part_set_min_keys((size_t)keys);
+    return PSHBM_OK;
+}
+
 int32_t pshbm_debug_part_pass_capacity(uint32_t entries) {
     part_set_pass_capacity(entries);
     return PSHBM_OK;

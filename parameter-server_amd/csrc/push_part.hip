@@ -993,11 +993,13 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // ---- host side --------------------------------------------------------------------------------
 namespace {
 u32 g_part_cap = PA_CAP;
+size_t g_part_min_keys = PART_MIN_KEYS;
 }
 void part_set_pass_capacity(uint32_t entries) { g_part_cap = entries == 0 || entries > PA_CAP ? PA_CAP : entries; }
+void part_set_min_keys(size_t keys) { g_part_min_keys = keys == 0 ? PART_MIN_KEYS : keys; }
 
 bool part_plan(const TableDev& t, size_t n, double entries_per_key, PartPlan* plan) {
-    if (n < PART_MIN_KEYS || n > PART_MAX_KEYS) return false;
+    if (n < g_part_min_keys || n > PART_MAX_KEYS) return false;
     const u32 vec = (t.dim % 4 == 0) ? 4u : 1u;
     if (t.dim / vec > PA_BLOCK) return false;  // a lane per 4 or 16 bytes of a row
     u32 bucket_bits = 0;

@@ -190,7 +190,9 @@ hipError_t launch_probe_hist(const TableDev& t, uint32_t n_rows, unsigned long l
 // Aggregation and update of a batch of PART_MIN_KEYS .. PART_MAX_KEYS keys without a global sort:
 // tiles of 4096 keys, partitions of about 1024 keys (ranges of home buckets). part_plan says whether a batch qualifies (and
 // how it is cut); part_sizes gives the bytes of each scratch array for batches of up to n keys.
-constexpr size_t PART_MIN_KEYS = 16384, PART_MAX_KEYS = 1u << 22;
+// (Below PART_MIN_KEYS one workgroup does the whole push in one launch; above PART_MAX_KEYS, and for
+// a table so full that a batch may have to be undone, the sorted push takes over.)
+constexpr size_t PART_MIN_KEYS = 513, PART_MAX_KEYS = 1u << 22;
 struct PartPlan {
     uint32_t n, n_tiles, P, part_shift;
 };
@@ -219,6 +221,9 @@ hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartB
 // Entries a pass of the apply kernel takes (0 = the default, 2048): a test hook that makes small
 // batches go through the multi-pass path.
 void part_set_pass_capacity(uint32_t entries);
+// Smallest batch that takes the partitioned path (0 = the default, PART_MIN_KEYS): a test hook that
+// sends mid-size batches through the sorted push.
+void part_set_min_keys(size_t keys);
 
 // ---- for-each / erase / rebuild (maint.hip) -------------------------------------------------
 // Count and column sums of the rows that satisfy `pred`. scratch: for_each_scratch_bytes();

@@ -22,6 +22,17 @@ OPTS = {
 }
 
 
+@pytest.fixture(autouse=True, params=["default", "sorted"])
+def push_path(request, ps):
+    """Every test of this file runs twice: with the library's own choice of push path (one launch up
+    to 512 keys, the partitioned push above) and with mid-size and large batches sent through the
+    sorted push (locate, radix sort, segmented reduce, fix-up), which otherwise only serves batches
+    of more than 4M keys, nearly full tables and the entry point that allocates nothing."""
+    ps.debug_part_min_keys((1 << 40) if request.param == "sorted" else 0)
+    yield request.param
+    ps.debug_part_min_keys(0)
+
+
 def pair(ps, orc, dim, opt, capacity=1 << 16, **kw):
     o = OPTS[opt]
     t = ps.Table(dim, capacity=capacity, **o, **kw)
@@ -870,10 +881,12 @@ def test_iterate_keys_follows_the_record_order(ps, orc, wl):
     t.close()
 
 
-def test_sort_that_gives_up_applies_nothing(ps, orc, wl):
+def test_sort_that_gives_up_applies_nothing(ps, orc, wl, push_path):
     """A tile of the aggregation sort that gives up its bounded wait raises a flag; the kernels
     after the sort then leave the rows alone and the table reports FATAL until it is cleared. The
     host makes the wait give up (a limit of zero polls): every kernel still runs to its end."""
+    if push_path != "sorted":
+        pytest.skip("the sorted push only")
     rng = np.random.default_rng(21)
     n_table, dim, n = 30000, 8, 14000          # 4 tiles of 4096 pairs: one-launch passes that wait
     t = ps.Table(dim, capacity=n_table + n, optimizer=1, lr=0.5)
@@ -901,14 +914,16 @@ def test_sort_that_gives_up_applies_nothing(ps, orc, wl):
     t.close()
 
 
-def test_c2_shaped_push_against_reference_order_and_exact_sums(ps, orc, wl, capsys):
+def test_c2_shaped_push_against_reference_order_and_exact_sums(ps, orc, wl, capsys, push_path):
     """The headline workload at a table size the oracle reaches: 1M-key Zipf(1.05) batches (the
     hottest key repeats about 100,000 times) over 10M keys, dim 16, SGD, gradients N(0, 1e-3).
     Every value must be within 1e-6 / 1e-7 of the exactly rounded result; the report says how many
     are further than that from the reference-order result, which drifts from the exact one itself."""
     rng = np.random.default_rng(17)
     n_table, n, dim = 10_000_000, 1_000_000, 16
-    t = ps.Table(dim, capacity=n_table + 16, max_batch=n, **OPTS["sgd"])
+    # (room for a whole batch of new keys: a table that might not hold the batch would take the
+    # sorted push, which can be undone, whatever the path this run asks for)
+    t = ps.Table(dim, capacity=n_table + n + 16, max_batch=n, **OPTS["sgd"])
     r = orc.Oracle(dim, capacity=n_table + 16, **OPTS["sgd"])
     x = orc.Oracle(dim, capacity=n_table + 16, **OPTS["sgd"])
     chunk = 1_000_000
@@ -934,5 +949,5 @@ def test_c2_shaped_push_against_reference_order_and_exact_sums(ps, orc, wl, caps
         # both oracles restart from the reference-order state, as the table does
         assert t.set(uk, b) == 0 and x.set(uk, b) == 0
     with capsys.disabled():
-        print("\nC2-shaped push parity report:", report)
+        print(f"\nC2-shaped push parity report ({push_path} push):", report)
     t.close()
