@@ -56,19 +56,19 @@ KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist"
 # must be counted again.
 TRAFFIC_FROM_PROFILES = {
     # (config, phase): (bytes, summary)
-    ("c1", "pull"): (19228672, "profiles/c1_pull_trace_and_hbm_counters.md"),
-    ("c2", "pull"): (196070400, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
-    ("c2", "part_tile"): (78893056, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
-    ("c2", "part_apply"): (158874624, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
-    ("c3", "pull"): (703215616, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c3", "part_tile"): (452928512, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c3", "part_apply"): (390892544, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "pull"): (585545728, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "part_tile"): (251302912, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "part_apply"): (637811712, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c5", "pull"): (3204963328, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
-    ("c5", "part_tile"): (1380345856, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
-    ("c5", "part_apply"): (2715714560, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c1", "pull"): (19226624, "profiles/c1_pull_trace_and_hbm_counters.md"),
+    ("c2", "pull"): (196069376, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "part_tile"): (78283776, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "part_apply"): (152215552, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "pull"): (703240192, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "part_tile"): (450812928, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "part_apply"): (378161152, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "pull"): (585565184, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_tile"): (241188864, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_apply"): (642350080, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "pull"): (3204072448, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "part_tile"): (1380431872, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "part_apply"): (2715749376, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
 }
 
 
