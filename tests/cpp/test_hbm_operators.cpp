@@ -961,5 +961,6 @@ int main(int argc, char** argv) {
         return 1;
     }
     std::printf("PASS test_hbm_operators\n");
+    std::fflush(stdout);
     return 0;
 }
