@@ -136,6 +136,11 @@ const char* pshbm_last_error(const pshbm_table* t);
  * state starts as without init_range. pshbm_init_weight gives the same number on the host. */
 float pshbm_init_weight(float init_range, uint64_t key, uint32_t column);
 
+/* Partition of a key among n_partitions (1 .. 2^31-1): jump_consistent_hash(fmix64(key), n_partitions),
+ * the host side of PSHBM_CMP_PART_EQ / PSHBM_CMP_PART_NE (see there for what it mirrors); -1 if
+ * n_partitions is out of range. */
+int32_t pshbm_partition(uint64_t key, int32_t n_partitions);
+
 /* Floats per stored value (weights + optimizer state) for a dim and optimizer; 0 if invalid. */
 uint32_t pshbm_value_floats(uint32_t dim, int32_t optimizer);
 
@@ -279,7 +284,18 @@ enum {
     PSHBM_CMP_GE = 3,
     PSHBM_CMP_EQ = 4,
     PSHBM_CMP_NE = 5,
-    PSHBM_CMP_MOD_EQ = 6 /* key % u == u2 (keys only; u > 0) */
+    PSHBM_CMP_MOD_EQ = 6, /* key % u == u2 (keys only; u > 0) */
+    /* The key's partition among u partitions is (PART_EQ) / is not (PART_NE) u2 (keys only; 0 < u < 2^31):
+     * partition = jump_consistent_hash(murmur_hash(key), u), the shape of the reference's
+     * DefaultPartitioner<uint64_t> (pico-ps/common/Partitioner.h:43-61). Both functions live in
+     * pico-core, which the reference tree does not hold; here they are the published ones: the 64-bit
+     * finalizer of MurmurHash3 (the fmix64 of pshbm_init_weight) and the jump consistent hash of
+     * Lamping and Veach (arXiv:1406.2294). pshbm_partition gives the same number on the host. With
+     * PART_NE a shard's purge after a reshard (apply_purge_request,
+     * pico-ps/operator/UpdateContextOperator.h:143-196: every key whose partition is no longer this
+     * shard goes) is one pshbm_erase_if on the device. */
+    PSHBM_CMP_PART_EQ = 7,
+    PSHBM_CMP_PART_NE = 8
 };
 typedef struct pshbm_term {
     int32_t column; /* 0 .. value_floats-1, or PSHBM_COL_KEY */

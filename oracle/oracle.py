@@ -38,7 +38,7 @@ class _Config(C.Structure):
 
 
 COL_KEY = -1
-CMP_LT, CMP_LE, CMP_GT, CMP_GE, CMP_EQ, CMP_NE, CMP_MOD_EQ = range(7)
+CMP_LT, CMP_LE, CMP_GT, CMP_GE, CMP_EQ, CMP_NE, CMP_MOD_EQ, CMP_PART_EQ, CMP_PART_NE = range(9)
 
 
 class _Term(C.Structure):
@@ -58,7 +58,7 @@ def predicate(*terms):
     for i, (col, cmp_, operand) in enumerate(terms):
         p.term[i].column, p.term[i].cmp = col, cmp_
         if col == COL_KEY:
-            if cmp_ == CMP_MOD_EQ:
+            if cmp_ in (CMP_MOD_EQ, CMP_PART_EQ, CMP_PART_NE):
                 p.term[i].u, p.term[i].u2 = operand
             else:
                 p.term[i].u = operand
@@ -97,6 +97,8 @@ def lib():
         L.pso_value_floats.restype = C.c_uint32
         L.pso_value_floats.argtypes = [C.c_uint32, C.c_int32]
         L.pso_create.argtypes = [C.POINTER(_Config), C.POINTER(vp)]
+        L.pso_partition.restype = C.c_int32
+        L.pso_partition.argtypes = [C.c_uint64, C.c_int32]
         L.pso_init_weight.restype = C.c_float
         L.pso_init_weight.argtypes = [C.c_float, C.c_uint64, C.c_uint32]
         L.pso_destroy.argtypes = [vp]
@@ -143,6 +145,11 @@ def record_dtype(value_floats):
 def init_weight(init_range, key, column):
     """Weight `column` of a new key of a table that draws initial weights in [-init_range, init_range)."""
     return lib().pso_init_weight(init_range, key, column)
+
+
+def partition(key, n):
+    """Partition of `key` among n (DefaultPartitioner<uint64_t>'s shape with the published functions)."""
+    return lib().pso_partition(key, n)
 
 
 class Oracle:

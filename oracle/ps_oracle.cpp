@@ -48,6 +48,15 @@
 //       pico-ps ships only zeros. The formula is this repository's; it is pinned by MurmurHash3's
 //       published finalizer vectors, an integer-only Python restatement, the exact bounds and the
 //       first two moments of the uniform distribution (tests/test_initial_weights.py).
+//   Key partition (pso_partition, the PART_EQ / PART_NE terms of a predicate)
+//       the shape is the reference's DefaultPartitioner<uint64_t> (pico-ps/common/Partitioner.h:43-61:
+//       jump_consistent_hash(murmur_hash(key), n)); both functions live in pico-core, which the
+//       reference tree does not hold: PARITY UNPINNED BY THE REFERENCE. Restated from their
+//       publications and pinned by those: MurmurHash3's fmix64 (published finalizer vectors) and
+//       the jump consistent hash of Lamping and Veach (arXiv:1406.2294; the test vectors of its widely
+//       used Go port github.com/dgryski/go-jump, the paper's properties -- one bucket for n = 1,
+//       keys only ever move to the new bucket when n grows, even spread -- and an integer-only
+//       Python restatement) in tests/test_partitioner.py.
 //   Capacity handling (PSO_OUT_OF_MEMORY, all-or-nothing per batch)
 //       this repository's decision for a fixed-capacity table; the reference instead parks the
 //       items in an overflow vector (SparsePushOperator.h:257-259). Documented, not pinned.
@@ -125,6 +134,19 @@ uint64_t fmix64(uint64_t k) {
 
 // Weight j of a new key when the table draws initial weights: the top 24 bits of a hash of
 // (key, column) as a number in [-1, 1) (exact in fp32), times the range (one rounding).
+// DefaultPartitioner<uint64_t>::partition (pico-ps/common/Partitioner.h:36-38,47-54) with the
+// published functions: fmix64, then the loop of Lamping and Veach's paper.
+int32_t jump_partition(uint64_t key, int32_t n) {
+    uint64_t k = fmix64(key);
+    int64_t b = -1, j = 0;
+    while (j < n) {
+        b = j;
+        k = k * 2862933555777941757ull + 1;
+        j = (int64_t)((double)(b + 1) * ((double)(1ll << 31) / (double)((k >> 33) + 1)));
+    }
+    return (int32_t)b;
+}
+
 float init_weight(float range, uint64_t key, uint32_t j) {
     const uint64_t h = fmix64(key ^ ((uint64_t)(j + 1u) * 0x9E3779B97F4A7C15ull));
     const float unit = (float)(uint32_t)(h >> 40) * (1.0f / 8388608.0f) - 1.0f;
@@ -282,6 +304,7 @@ struct pso_config {
 };
 
 float pso_init_weight(float range, uint64_t key, uint32_t column) { return init_weight(range, key, column); }
+int32_t pso_partition(uint64_t key, int32_t n) { return n > 0 ? jump_partition(key, n) : -1; }
 
 uint32_t pso_value_floats(uint32_t dim, int32_t opt) { return value_floats(dim, opt); }
 
@@ -464,7 +487,8 @@ int32_t pso_dump(void* h, void* records, size_t capacity_records, size_t* n_out)
 // which must hold. Layout identical to pshbm_term / pshbm_predicate.
 struct pso_term {
     int32_t column;  // -1 = the key
-    int32_t cmp;     // 0 LT, 1 LE, 2 GT, 3 GE, 4 EQ, 5 NE, 6 MOD_EQ (key % u == u2)
+    int32_t cmp;     // 0 LT, 1 LE, 2 GT, 3 GE, 4 EQ, 5 NE, 6 MOD_EQ (key % u == u2),
+                     // 7 PART_EQ / 8 PART_NE (the key's partition among u is / is not u2)
     float f;
     uint32_t reserved;
     uint64_t u, u2;
@@ -489,6 +513,8 @@ static bool holds(const pso_predicate* p, uint64_t key, const float* v) {
                 case 4: r = key == t.u; break;
                 case 5: r = key != t.u; break;
                 case 6: r = t.u != 0 && key % t.u == t.u2; break;
+                case 7: r = t.u != 0 && (uint64_t)jump_partition(key, (int32_t)t.u) == t.u2; break;
+                case 8: r = t.u != 0 && (uint64_t)jump_partition(key, (int32_t)t.u) != t.u2; break;
             }
         } else {
             const float x = v[t.column];

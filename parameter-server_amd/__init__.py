@@ -36,7 +36,7 @@ SYMBOLS = [
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
     "pshbm_push_dev_noalloc", "pshbm_pull_dev_handles", "pshbm_push_dev_handles", "pshbm_debug_sort_spin_limit", "pshbm_debug_part_pass_capacity", "pshbm_debug_part_min_keys",
-    "pshbm_debug_tombstone_limit", "pshbm_debug_sort_pairs",
+    "pshbm_debug_tombstone_limit", "pshbm_debug_sort_pairs", "pshbm_partition",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
           "fixup_windows", "assign_rows", "push_small", "part_tile", "part_apply", "part_insert"]
@@ -88,7 +88,7 @@ class Stats(C.Structure):
 
 
 COL_KEY = -1
-CMP_LT, CMP_LE, CMP_GT, CMP_GE, CMP_EQ, CMP_NE, CMP_MOD_EQ = range(7)
+CMP_LT, CMP_LE, CMP_GT, CMP_GE, CMP_EQ, CMP_NE, CMP_MOD_EQ, CMP_PART_EQ, CMP_PART_NE = range(9)
 
 
 class Term(C.Structure):
@@ -103,7 +103,8 @@ class Predicate(C.Structure):
 
 def predicate(*terms):
     """predicate((column, cmp, operand), ...): column COL_KEY compares the key with an integer
-    operand -- (COL_KEY, CMP_MOD_EQ, (modulus, remainder)) for key % modulus == remainder --,
+    operand -- (COL_KEY, CMP_MOD_EQ, (modulus, remainder)) for key % modulus == remainder,
+    (COL_KEY, CMP_PART_EQ / CMP_PART_NE, (partitions, partition)) for the key's partition --,
     any other column compares that value column with a float."""
     p = Predicate()
     p.struct_size = C.sizeof(Predicate)
@@ -111,7 +112,7 @@ def predicate(*terms):
     for i, (col, cmp_, operand) in enumerate(terms):
         p.term[i].column, p.term[i].cmp = col, cmp_
         if col == COL_KEY:
-            if cmp_ == CMP_MOD_EQ:
+            if cmp_ in (CMP_MOD_EQ, CMP_PART_EQ, CMP_PART_NE):
                 p.term[i].u, p.term[i].u2 = operand
             else:
                 p.term[i].u = operand
@@ -191,6 +192,8 @@ def lib():
         L.pshbm_debug_sort_spin_limit.argtypes = [u32]
         L.pshbm_debug_part_pass_capacity.argtypes = [u32]
         L.pshbm_debug_part_min_keys.argtypes = [C.c_uint64]
+        L.pshbm_partition.argtypes = [C.c_uint64, C.c_int32]
+        L.pshbm_partition.restype = C.c_int32
         L.pshbm_debug_sort_pairs.argtypes = [C.c_int32, vp, vp, vp, vp, sz, u32, C.POINTER(C.c_int32), vp]
         L.pshbm_debug_tombstone_limit.argtypes = [C.c_uint64, C.c_uint64]
         L.pshbm_debug_tombstone_limit.restype = C.c_uint64
@@ -268,6 +271,11 @@ def debug_part_min_keys(keys=0):
     """Test hook: smallest batch that takes the partitioned push (0 = default); a large value sends
     mid-size batches through the sorted push."""
     return lib().pshbm_debug_part_min_keys(keys)
+
+
+def partition(key, n_partitions):
+    """Partition of a key among n_partitions: jump_consistent_hash(fmix64(key), n) (pshbm_partition)."""
+    return lib().pshbm_partition(key, n_partitions)
 
 
 def init_weight(init_range, key, column):

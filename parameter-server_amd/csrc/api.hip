@@ -778,8 +778,11 @@ int32_t check_predicate(pshbm_table* t, const pshbm_predicate* w, pshbm_predicat
         const pshbm_term& m = w->term[i];
         if (m.column != PSHBM_COL_KEY && (m.column < 0 || (uint32_t)m.column >= t->d.vf))
             return fail(t, PSHBM_INVALID_CONFIG, "predicate: term %u names column %d of %u", i, m.column, t->d.vf);
-        if (m.cmp < PSHBM_CMP_LT || m.cmp > PSHBM_CMP_MOD_EQ)
+        if (m.cmp < PSHBM_CMP_LT || m.cmp > PSHBM_CMP_PART_NE)
             return fail(t, PSHBM_INVALID_CONFIG, "predicate: term %u has no such comparison", i);
+        if ((m.cmp == PSHBM_CMP_PART_EQ || m.cmp == PSHBM_CMP_PART_NE) &&
+            (m.column != PSHBM_COL_KEY || m.u == 0 || m.u > 0x7FFFFFFFull))
+            return fail(t, PSHBM_INVALID_CONFIG, "predicate: term %u: a partition test needs the key and 1 .. 2^31-1 partitions", i);
         if (m.cmp == PSHBM_CMP_MOD_EQ && (m.column != PSHBM_COL_KEY || m.u == 0))
             return fail(t, PSHBM_INVALID_CONFIG, "predicate: term %u: MOD_EQ needs the key and a modulus", i);
     }
@@ -844,6 +847,10 @@ int32_t erase_flagged(pshbm_table* t, uint32_t rows, hipStream_t s, uint64_t* er
 }  // namespace
 
 extern "C" {
+
+int32_t pshbm_partition(uint64_t key, int32_t n_partitions) {
+    return n_partitions > 0 ? jump_partition(key, n_partitions) : -1;
+}
 
 uint32_t pshbm_value_floats(uint32_t dim, int32_t optimizer) {
     switch (optimizer) {

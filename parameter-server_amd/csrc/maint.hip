@@ -36,6 +36,8 @@ __device__ __forceinline__ bool cmp_u(u64 k, const pshbm_term& t) {
         case PSHBM_CMP_EQ: return k == t.u;
         case PSHBM_CMP_NE: return k != t.u;
         case PSHBM_CMP_MOD_EQ: return t.u != 0 && k % t.u == t.u2;
+        case PSHBM_CMP_PART_EQ: return (u64)jump_partition(k, (int32_t)t.u) == t.u2;
+        case PSHBM_CMP_PART_NE: return (u64)jump_partition(k, (int32_t)t.u) != t.u2;
     }
     return false;
 }

@@ -71,6 +71,23 @@ __host__ __device__ inline uint64_t hash64(uint64_t h) {
     return h;
 }
 
+// The partition of a key among n (1 .. 2^31-1): the shape of the reference's DefaultPartitioner<uint64_t>
+// (pico-ps/common/Partitioner.h:43-61: jump_consistent_hash(murmur_hash(key), n)), with the published
+// functions in the place of pico-core's: MurmurHash3's 64-bit finalizer and the jump consistent hash of
+// Lamping and Veach (arXiv:1406.2294, the loop below is the paper's). The two floating-point operations
+// are IEEE double division and multiplication on the host and on the device alike.
+__host__ __device__ inline int32_t jump_partition(uint64_t key, int32_t n) {
+    uint64_t k = hash64(key);
+    int64_t b = -1, j = 0;
+    while (j < n) {
+        b = j;
+        k = k * 2862933555777941757ull + 1;
+        const double q = 2147483648.0 / (double)((k >> 33) + 1);
+        j = (int64_t)((double)(b + 1) * q);
+    }
+    return (int32_t)b;
+}
+
 // Weight `col` of a key that is inserted, when the table draws initial weights: a pure function
 // of key and column (24 bits of a hash, mapped to [-1, 1) exactly, times the range with one
 // rounding), so that every path -- and the CPU restatement -- gives the key the same weights.

@@ -26,6 +26,7 @@
 #include <functional>
 #include <memory>
 #include <mutex>
+#include <type_traits>
 #include <unordered_map>
 
 #include "../../include/pshbm.h"
@@ -788,11 +789,27 @@ private:
     size_t _block_size;
 };
 
+// The key partitioner of sparse tables: DefaultPartitioner<uint64_t> (common/Partitioner.h:43-61),
+// partition = jump_consistent_hash(murmur_hash(key), n). pico-core's two functions are not in the
+// reference tree; these are the published ones (MurmurHash3's 64-bit finalizer, Lamping and Veach's
+// jump consistent hash), which the library also evaluates on the device: a partitioner that
+// declares `device_terms` lets HbmShuffleOperator purge a shard with one erase_if on the device
+// instead of walking its keys over the link.
+struct HbmDefaultPartitioner {
+    static constexpr bool device_terms = true;
+    int32_t partition(uint64_t key, int32_t num_buckets) const { return pshbm_partition(key, num_buckets); }
+};
+template <class P, class = void>
+struct hbm_partitioner_on_device : std::false_type {};
+template <class P>
+struct hbm_partitioner_on_device<P, std::enable_if_t<P::device_terms>> : std::true_type {};
+
 // Re-sharding after the set of servers changed (UpdateContextOperator.h:100-305). The host logic
 // that drives it stays as it is; what it needs from the storage is (1) the items of a shard that
 // now belong elsewhere, a bounded block at a time, and (2) the purge of those items.
 // PARTITIONER::partition(key, global_shard_num) is the reference's key partitioner
-// (common/Partitioner.h:43-61), evaluated on the host.
+// (common/Partitioner.h:43-61), evaluated on the host -- except in the purge, which runs on the
+// device when the partitioner is the library's (HbmDefaultPartitioner).
 template <class PARTITIONER>
 class HbmShuffleOperator {
 public:
@@ -856,16 +873,27 @@ public:
         req >> shard_id;
         if (new_rt.local_shards().count(shard_id)) {
             pshbm_table* t = st.get(shard_id);
-            std::vector<uint64_t> keys(_block_items), gone;
-            for (size_t offset = 0;;) {  // the keys first: erasing moves rows, which would disturb the walk
-                size_t got = 0;
-                PSHBM_SCHECK(pshbm_iterate_keys(t, offset, _block_items, keys.data(), &got) == PSHBM_OK, "iterate failed");
-                for (size_t i = 0; i < got; ++i)
-                    if (_key_partitioner.partition(keys[i], new_rt.global_shard_num()) != shard_id) gone.push_back(keys[i]);
-                offset += got;
-                if (got < _block_items) break;
+            if constexpr (hbm_partitioner_on_device<PARTITIONER>::value) {
+                pshbm_predicate not_mine{};
+                not_mine.struct_size = sizeof not_mine;
+                not_mine.n_terms = 1;
+                not_mine.term[0].column = PSHBM_COL_KEY;
+                not_mine.term[0].cmp = PSHBM_CMP_PART_NE;
+                not_mine.term[0].u = (uint64_t)new_rt.global_shard_num();
+                not_mine.term[0].u2 = (uint64_t)shard_id;
+                PSHBM_SCHECK(pshbm_erase_if(t, &not_mine, nullptr) == PSHBM_OK, "erase_if failed");
+            } else {
+                std::vector<uint64_t> keys(_block_items), gone;
+                for (size_t offset = 0;;) {  // the keys first: erasing moves rows, which would disturb the walk
+                    size_t got = 0;
+                    PSHBM_SCHECK(pshbm_iterate_keys(t, offset, _block_items, keys.data(), &got) == PSHBM_OK, "iterate failed");
+                    for (size_t i = 0; i < got; ++i)
+                        if (_key_partitioner.partition(keys[i], new_rt.global_shard_num()) != shard_id) gone.push_back(keys[i]);
+                    offset += got;
+                    if (got < _block_items) break;
+                }
+                PSHBM_SCHECK(pshbm_erase(t, gone.data(), gone.size(), nullptr) == PSHBM_OK, "erase failed");
             }
-            PSHBM_SCHECK(pshbm_erase(t, gone.data(), gone.size(), nullptr) == PSHBM_OK, "erase failed");
             PSHBM_SCHECK(pshbm_compact(t) == PSHBM_OK, "compact failed");
         } else {
             st.erase_shard(shard_id);

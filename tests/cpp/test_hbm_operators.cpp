@@ -584,6 +584,79 @@ static void test_threaded_pushes() {
     for (size_t i = 0; i < keys.size(); ++i) EXPECT(v[i * 2] == want && v[i * 2 + 1] == want);
 }
 
+// Re-sharding with the library's key partitioner (HbmDefaultPartitioner: the shape of
+// DefaultPartitioner<uint64_t>, common/Partitioner.h:43-61): two shards placed by partition(key, 2)
+// become three; the generator hands out exactly the items whose partition changed, and the purge --
+// one erase_if on the device per shard -- leaves exactly the others.
+static void test_default_partitioner_purge() {
+    Configure cfg;
+    cfg.set("dim", 2);
+    cfg.set("optimizer", "sum");
+    cfg.set("hbm_table.expected_max_items", 4000);
+    cfg.set("shuffle_block_items", 128);
+    RuntimeInfo rt(0, {0, 1});
+    HbmStorageOperator storage_op(cfg);
+    std::unique_ptr<Storage> storage = storage_op.create_storage(rt, 0);
+    HbmDefaultPartitioner part;
+    HbmDirectPushOperator direct(cfg);
+    std::vector<std::vector<Pair>> mine(2);
+    constexpr uint64_t KEYS = 3000;
+    for (uint64_t k = 1; k <= KEYS; ++k) {
+        const uint64_t key = k * 0x9E3779B97F4A7C15ull;
+        const int32_t sh = part.partition(key, 2);
+        EXPECT(sh == 0 || sh == 1);
+        mine[sh].push_back(Pair{key, {(float)k, 1.0f}});
+    }
+    EXPECT(mine[0].size() > KEYS / 3 && mine[1].size() > KEYS / 3);
+    {
+        PSRequest req;
+        req << (int32_t)2 << (int32_t)1;
+        for (int32_t sh = 0; sh < 2; ++sh) {
+            req << sh << (int32_t)mine[sh].size();
+            const char* p = reinterpret_cast<const char*>(mine[sh].data());
+            req.lazy().emplace_back(p, p + mine[sh].size() * sizeof(Pair));
+        }
+        PSResponse resp;
+        direct.apply_async_push_request(rt, req, storage.get(), nullptr, resp);
+        Status s;
+        resp >> s;
+        EXPECT(s.ok());
+    }
+    HbmShuffleOperator<HbmDefaultPartitioner> shuffle_op(cfg);
+    RuntimeInfo new_rt(0, {0, 1, 2});
+    auto& st = *static_cast<HbmShardStorage*>(storage.get());
+    size_t leaving = 0, expect_leaving = 0, expect_left[2] = {0, 0};
+    for (int32_t sh = 0; sh < 2; ++sh)
+        for (const Pair& it : mine[sh]) {
+            if (part.partition(it.key, 3) != sh) ++expect_leaving;
+            else ++expect_left[sh];
+        }
+    EXPECT(expect_leaving > KEYS / 6 && expect_leaving < KEYS / 2);  // about a third moves, all of it to shard 2
+    for (int32_t sh = 0; sh < 2; ++sh) {
+        auto gen = shuffle_op.lock_push_items_generator(new_rt, storage.get(), sh, false);
+        std::vector<uint64_t> keys;
+        std::vector<float> vals;
+        while (gen->generate_push_items(keys, vals)) {}
+        for (uint64_t key : keys) EXPECT(part.partition(key, 2) == sh && part.partition(key, 3) == 2);
+        leaving += keys.size();
+    }
+    EXPECT(leaving == expect_leaving);
+    for (int32_t sh = 0; sh < 2; ++sh) {
+        PSRequest req;
+        req << sh;
+        PSResponse resp;
+        shuffle_op.apply_purge_request(new_rt, req, storage.get(), resp);
+        Status s;
+        resp >> s;
+        EXPECT(s.ok());
+        EXPECT(st.shard_size(sh) == expect_left[sh]);
+        std::vector<uint64_t> left(expect_left[sh] + 1);
+        size_t got = 0;
+        EXPECT(pshbm_iterate_keys(st.get(sh), 0, left.size(), left.data(), &got) == PSHBM_OK && got == expect_left[sh]);
+        for (size_t i = 0; i < got; ++i) EXPECT(part.partition(left[i], 3) == sh);
+    }
+}
+
 // hbm_table.init_range: a pull that misses answers the weights an insertion would store; a push
 // of a new key takes its step from them (init_store_value, SparsePullOperator.h:217,307-310).
 static void test_initial_weights() {
@@ -953,6 +1026,7 @@ int main(int argc, char** argv) {
     test_growth();
     test_operator_hyperparameters();
     test_threaded_pushes();
+    test_default_partitioner_purge();
     test_initial_weights();
     test_memory_limit();
     test_sync();
