@@ -210,3 +210,54 @@ def test_handles_are_ignored_by_small_batches(ps, orc, wl):
         assert r.push(q, g) == 0
         same(t, r, exact=True)
     t.close()
+
+
+@pytest.mark.parametrize("verify", [False, True])
+def test_handles_in_partitions_that_need_several_passes(ps, orc, wl, verify):
+    """With the pass capacity turned down every partition takes the several-passes path (entries
+    chosen by hash class, a class at a time): the handles travel with the chosen entries."""
+    dim, opt = 16, "sgd"
+    rng = np.random.default_rng(14)
+    n_table, n = 40000, 60000
+    t = ps.Table(dim, capacity=n_table + n, max_batch=n, **OPTS[opt])
+    r = orc.Oracle(dim, capacity=n_table + n, **OPTS[opt])
+    fill(t, r, wl, rng, n_table, opt, dim, seed=15)
+    q, g = batch(wl, rng, n_table, n, 1.05, dim, 15, 0.05, integer=True)
+    d = Dev(q, g, dim)
+    epoch = d.pull(t)
+    try:
+        ps.debug_part_pass_capacity(256)
+        d.push(t, epoch, ps.PUSH_VERIFY_HANDLES if verify else 0)
+    finally:
+        ps.debug_part_pass_capacity(0)
+    assert r.push(q, g) == 0
+    same(t, r, exact=True)
+    assert t.size() == r.size()
+    t.close()
+
+
+def test_handles_with_track_increment_and_a_second_table(ps, orc, wl):
+    """Two tables on the device, each with its own handles and epoch; pushes mark what they touch."""
+    dim, opt = 8, "adagrad"
+    rng = np.random.default_rng(16)
+    n_table, n = 30000, 20000
+    tabs = [ps.Table(dim, capacity=n_table + n, max_batch=n, track_increment=True, **OPTS[opt]) for _ in range(2)]
+    refs = [orc.Oracle(dim, capacity=n_table + n, track_increment=True, **OPTS[opt]) for _ in range(2)]
+    for t, r, seed in zip(tabs, refs, (17, 18)):
+        fill(t, r, wl, rng, n_table, opt, dim, seed=seed)
+        t.take_increment(), r.take_increment()
+    work = []
+    for t, seed in zip(tabs, (17, 18)):
+        q, g = batch(wl, rng, n_table, n, 1.1, dim, seed, 0.02)
+        d = Dev(q, g, dim)
+        work.append((d, d.pull(t), q, g))
+    for (d, epoch, q, g), t, r in zip(work, tabs, refs):      # the pushes after both pulls
+        d.push(t, epoch)
+        assert r.push(q, g, orc.PUSH_EXACT_AGGREGATION) == 0
+        same(t, r, exact=False)
+        st, rec = t.take_increment()
+        st2, rec2 = r.take_increment()
+        assert st == st2 == 0
+        np.testing.assert_array_equal(np.sort(rec["key"]), np.sort(rec2["key"]))
+    for t in tabs:
+        t.close()
