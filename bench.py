@@ -63,9 +63,9 @@ TRAFFIC_FROM_PROFILES = {
     ("c3", "pull"): (703240192, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
     ("c3", "part_tile"): (450812928, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
     ("c3", "part_apply"): (378161152, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "pull"): (585565184, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "part_tile"): (241188864, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "part_apply"): (642350080, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "pull"): (558432256, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_tile"): (233840640, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_apply"): (663741440, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
     ("c5", "pull"): (3204072448, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
     ("c5", "part_tile"): (1380431872, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
     ("c5", "part_apply"): (2715749376, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
@@ -387,7 +387,11 @@ def measure(name, args, torch, ps, wl, steps, warmup, headline):
     cfg = dict(CONFIGS[name])
     n_table = (args.table_keys if headline else 0) or cfg["n"]
     t = build_table(ps, wl, torch, cfg, n_table)
-    batches = make_batches(wl, torch, cfg, n_table, n_batches=8)
+    # Eight batches in turn -- except where batches bring fresh keys (c4): there every step of the
+    # warm-up, of the timed run and of the run under events gets a batch of its own, so that each
+    # step really inserts its fresh keys (a batch that comes round again would find them stored).
+    n_batches = (warmup + 2 * steps) if cfg["fresh"] > 0 else 8
+    batches = make_batches(wl, torch, cfg, n_table, n_batches=n_batches)
     out = torch.empty(cfg["batch"], cfg["dim"], device="cuda")
     k = cfg["batch"]
     keys_per_step = k * (1 if cfg["pull_only"] else 2)
@@ -402,7 +406,7 @@ def measure(name, args, torch, ps, wl, steps, warmup, headline):
     ms_per_step = elapsed * 1e3 / steps
 
     t.profile_enable(True)
-    run_steps(t, torch, cfg, batches, out, steps, first=warmup, handles=handles)
+    run_steps(t, torch, cfg, batches, out, steps, first=warmup + (steps if cfg["fresh"] > 0 else 0), handles=handles)
     torch.cuda.synchronize()
     prof = t.profile_read()
     t.profile_enable(False)
@@ -440,7 +444,8 @@ def measure(name, args, torch, ps, wl, steps, warmup, headline):
         "value": keys_per_step * steps / elapsed, "ms_per_step": ms_per_step, "steps": steps, "warmup": warmup,
         "config": {"workload": cfg["desc"], "table_keys": n_table, "batch": k, "dim": cfg["dim"],
                    "unique_keys_per_batch": round(u_mean), "keys_alone_in_their_tile": round(alone_mean),
-                   "row_handles": handles is not None and not cfg["pull_only"]},
+                   "row_handles": handles is not None and not cfg["pull_only"],
+                   "batches": n_batches},
         "step_algorithmic_bytes": int(step_bytes),
         "step_algorithmic_GBps": round(step_bytes / (ms_per_step * 1e6), 1),
         "step_frac_of_hbm_peak": round(step_bytes / (ms_per_step * 1e6) / HBM_PEAK_GBS, 4),
