@@ -1,6 +1,7 @@
 """Random operation sequences on the HIP path and the oracle side by side (needs an MI355X).
 
-Each case draws a table shape (dim, optimizer) and a sequence of pulls, pushes, queued pushes and
+Each case draws a table shape (dim, optimizer) and a sequence of pulls, pushes (plain, from the wire
+layout, from page-locked buffers, or as a pull + push pair through row handles), queued pushes and
 stores, sets, erases, erase-ifs, for-eachs, dump / load round trips, growth and increment takes, with
 gradients that are small integers (times a power of two for the optimizers with a learning rate)
 so that duplicate sums are exact and every value can be compared bit for bit after every step --
@@ -8,6 +9,8 @@ except under FTRL and Adagrad, whose steps are not exact; those cases push disti
 """
 import numpy as np
 import pytest
+
+torch = pytest.importorskip("torch")
 
 pytestmark = pytest.mark.gpu
 
@@ -66,8 +69,20 @@ def test_random_operation_sequences(ps, orc, wl, seed):
             q = batch(n)
             g = grads(q.size)
             flags = ps.PUSH_NO_INSERT if op == "push_no_insert" else 0
-            how = int(rng.integers(0, 3))
-            if how == 0:                                 # the wire layout of a push block
+            how = int(rng.integers(0, 4))
+            if how == 3:                                 # a pull, then the push through its row handles
+                dk = torch.from_numpy(q.view(np.int64)).cuda()
+                dg = torch.from_numpy(g).cuda()
+                rows = torch.empty(q.size, dim, device="cuda")
+                hd = torch.empty(q.size, dtype=torch.int32, device="cuda")
+                stream = torch.cuda.current_stream().cuda_stream
+                st, epoch = t.pull_dev_handles(dk.data_ptr(), q.size, rows.data_ptr(), hd.data_ptr(), None, 0, stream)
+                assert st == 0
+                np.testing.assert_array_equal(rows.cpu().numpy().view(np.uint32), r.pull(q)[1].view(np.uint32))
+                vflag = ps.PUSH_VERIFY_HANDLES if rng.random() < 0.5 else 0
+                a = t.push_dev_handles(dk.data_ptr(), dg.data_ptr(), hd.data_ptr(), epoch, q.size, flags | vflag, stream)
+                torch.cuda.synchronize()
+            elif how == 0:                               # the wire layout of a push block
                 pairs = np.empty(q.size, np.dtype([("key", np.uint64), ("value", np.float32, (dim,))]))
                 pairs["key"], pairs["value"] = q, g
                 a = t.push_pairs(pairs, flags)
@@ -113,7 +128,8 @@ def test_random_operation_sequences(ps, orc, wl, seed):
             assert t.erase(q) == r.erase(q)
         elif op == "erase_if":
             m = int(rng.integers(2, 6))
-            terms = [(-1, 6, (m, int(rng.integers(0, m))))]
+            # key % m == x, or the key's partition among m is / is not x
+            terms = [(-1, int(rng.choice([6, 6, 7, 8])), (m, int(rng.integers(0, m))))]
             if rng.random() < 0.5:
                 terms.append((int(rng.integers(0, vf)), int(rng.integers(0, 6)), float(rng.integers(-3, 4))))
             assert t.erase_if(ps.predicate(*terms)) == r.erase_if(orc.predicate(*terms))
