@@ -164,8 +164,12 @@ int32_t pshbm_pull_dev(pshbm_table* t, const uint64_t* d_keys, size_t n, float* 
  * store_push_value = one optimizer step with the summed gradient). grads is n x dim.
  * OUT_OF_MEMORY when the new keys do not fit: then the table is unchanged (the reference parks
  * such items in the shard's overflow vector, :257-259; a fixed-capacity table refuses the batch).
- * The *_dev form synchronizes only when the table is within n keys of its capacity. A batch (and
- * what is queued for one store) holds at most 2^30-1 keys; pulls, sets and erases 2^31-1. */
+ * The *_dev form only enqueues. The one exception is a table whose keys stored plus the keys of every
+ * batch still in flight come within n of its capacity: the call then waits (without synchronizing
+ * the stream) for the device to report the row counts of the oldest batches in flight, and only if
+ * the table really is within n keys of its capacity does it synchronize the stream to count exactly.
+ * A batch (and what is queued for one store) holds at most 2^30-1 keys; pulls, sets and erases
+ * 2^31-1. */
 int32_t pshbm_push(pshbm_table* t, const uint64_t* keys, const float* grads, size_t n,
                    uint32_t flags);
 int32_t pshbm_push_dev(pshbm_table* t, const uint64_t* d_keys, const float* d_grads, size_t n,
@@ -198,8 +202,8 @@ int32_t pshbm_push_dev_handles(pshbm_table* t, const uint64_t* d_keys, const flo
  * capture, tight serving loops, harnesses that forbid it. It has no counterpart in the reference.
  * The scratch of the push (probe results, sort buffers, partial sums) lies in a fixed array of
  * about 2.8 MB inside the library, one copy per device, instead of the table's workspace, and the
- * call allocates nothing on the device or through any library; it synchronizes only where
- * pshbm_push_dev does (a table within n keys of its capacity). Limits: n <= 16384 keys and
+ * call allocates nothing on the device or through any library; it waits or synchronizes only where
+ * pshbm_push_dev does (a table nearly at its capacity). Limits: n <= 16384 keys and
  * n * dim <= 2^20 gradient floats per call, PSHBM_ERROR beyond. Results are those of pshbm_push_dev.
  * All tables of a device share the one array: calls that overlap on the device (different streams,
  * no ordering between them) race on it, also across tables; calls on one stream, or ordered by
