@@ -440,7 +440,9 @@ constexpr u32 PA_OFF_LIST = PA_OFF_LREF + PA_CAP * 4;
 constexpr u32 PA_OFF_LOWN = PA_OFF_LIST + PA_CAP * 4;
 constexpr u32 PA_OFF_UREP = PA_OFF_LOWN + PA_CAP * 2;
 constexpr u32 PA_OFF_MREP = PA_OFF_UREP + PA_CAP * 2;
-constexpr u32 PA_LDS = PA_OFF_MREP + PA_CAP * 2;  // 75776
+constexpr u32 PA_OFF_SUMS = PA_OFF_MREP + PA_CAP * 2;          // partial sums of the block scans
+constexpr u32 PA_OFF_MISC = PA_OFF_SUMS + (PA_BLOCK / 64) * 8;  // three counters
+constexpr u32 PA_LDS = PA_OFF_MISC + 64;  // 75904
 
 struct ApplyArgs {
     const uint4* stage;  // {key low, key high, reference, row handle}, a block of PT_TILE per tile
@@ -455,6 +457,8 @@ struct ApplyArgs {
     u32 cap;  // entries a pass holds: PA_CAP, or less when a test wants to see the passes
     int handles;  // the entries carry rows that an earlier pull reported
     int verify;   // ... which count only where row_keys agrees
+    const u32* order;  // the partition each workgroup takes, or null
+    u32* psize;        // out: entries of each partition
 };
 
 // The optimizer step of the distinct keys of a pass: a key with one entry takes its gradient row, a
@@ -768,6 +772,12 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
 // loads are issued before anything waits. Returns {entries of the partition, entries in lower
 // partitions}. All threads call it.
 constexpr u32 PA_TILES_MAX = 2 * PA_BLOCK;
+constexpr u32 PA_STACK = 72;  // classes that can wait at once: one per bit of the second hash, and a few
+static_assert(PA_CAP + PA_STACK * 12 <= PA_CAP * 2, "the stack fits the upper half of mrep");
+
+// The second hash, by which a crowded partition is taken in passes: one-to-one like hash64, and
+// unrelated to the bits of hash64 that choose partition and bucket.
+__device__ __forceinline__ u64 class_hash(u64 key) { return hash64(hash64(key) ^ 0x9E3779B97F4A7C15ull); }
 static_assert(PART_MAX_KEYS / PT_TILE <= PA_TILES_MAX, "two tiles per thread cover the largest batch");
 static_assert(2 * PA_TILES_MAX <= PA_CAP, "the offsets fit the room of the reference list");
 
@@ -797,14 +807,87 @@ __device__ __forceinline__ uint4 partition_entry(const ApplyArgs& a, const u32* 
     return a.stage[(size_t)x * PT_TILE + ta[x] + (i - toff[x])];
 }
 
+// A partition with more entries than a pass holds (several keys that are met in most tiles share
+// it) is taken in passes by hash class, a class being the keys that agree in the low bits of a
+// second hash: first two classes; one that still holds too many is split in two by the next bit,
+// as often as it takes -- the second hash is one-to-one, so two keys part company at some bit, and
+// one key alone has at most an entry per tile, which a pass holds. (Only a pass capacity below the
+// number of tiles, which a test may set, can leave a class of one key too large; that is
+// reported.) The classes still to do wait on a stack in the upper half of the room of `mrep`,
+// which no pass touches (it numbers keys with several entries: at most half a pass).
+template <typename T>
+__device__ __forceinline__ void apply_crowded(const TableDev& t, unsigned char* pa_lds, const T* __restrict__ grads,
+                                              const T* __restrict__ psum, T* __restrict__ ngrad, const ApplyArgs& a,
+                                              u32 p, u32 s, u32 np) {
+    u64* sums = reinterpret_cast<u64*>(pa_lds + PA_OFF_SUMS);
+    u32* misc = reinterpret_cast<u32*>(pa_lds + PA_OFF_MISC);
+    u32& s_sel = misc[1];
+    u32& s_sp = misc[2];
+    u64* lkey = reinterpret_cast<u64*>(pa_lds);
+    u32* lref = reinterpret_cast<u32*>(pa_lds + PA_OFF_LREF);
+    u32* lhdl = reinterpret_cast<u32*>(pa_lds + PA_OFF_HDL);
+    u32* toff = reinterpret_cast<u32*>(pa_lds + PA_OFF_LIST);
+    u32* ta = toff + PA_TILES_MAX;
+    u64* stk_cls = reinterpret_cast<u64*>(pa_lds + PA_OFF_MREP + PA_CAP);
+    u32* stk_lg = reinterpret_cast<u32*>(stk_cls + PA_STACK);
+    const u32 tid = threadIdx.x;
+    if (tid == 0) {
+        stk_cls[0] = 0;
+        stk_cls[1] = 1;
+        stk_lg[0] = stk_lg[1] = 1;
+        s_sp = 2;
+    }
+    __syncthreads();
+    while (s_sp) {  // block-uniform: read between barriers
+        const u32 lg = stk_lg[s_sp - 1];
+        const u64 cls = stk_cls[s_sp - 1];
+        __syncthreads();
+        if (tid == 0) {
+            s_sp -= 1;
+            s_sel = 0;
+        }
+        __syncthreads();
+        const u64 mask = lg >= 64u ? ~0ull : (1ull << lg) - 1ull;
+        tile_segments(a, p, tid, sums, toff, ta);  // (a pass overwrites them)
+        __syncthreads();
+        for (u32 i = tid; i < np; i += PA_BLOCK) {
+            const uint4 e = partition_entry(a, toff, ta, i);
+            const u64 key = ((u64)e.y << 32) | e.x;
+            if ((class_hash(key) & mask) == cls) {
+                const u32 pos = atomicAdd(&s_sel, 1u);
+                if (pos < a.cap) {
+                    lkey[pos] = key;
+                    lref[pos] = e.z;
+                    lhdl[pos] = e.w;
+                }
+            }
+        }
+        __syncthreads();
+        const u32 sel = s_sel;
+        if (sel > a.cap) {
+            if (lg >= 64u) {  // one key with more entries than a pass holds: reported, never silent
+                if (tid == 0) t.counters[CNT_PART_ERR] = 1u;
+            } else if (tid == 0) {  // (a pop and two pushes per level: never more than 65 waiting)
+                stk_cls[s_sp] = cls;
+                stk_lg[s_sp] = lg + 1u;
+                stk_cls[s_sp + 1] = cls | (1ull << lg);
+                stk_lg[s_sp + 1] = lg + 1u;
+                s_sp += 2;
+            }
+        } else if (sel) {
+            apply_pass<T>(t, pa_lds, sums, misc, grads, psum, ngrad, a, s, sel);
+        }
+        __syncthreads();
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, const T* __restrict__ grads,
                                                                const T* __restrict__ psum, T* __restrict__ ngrad,
                                                                ApplyArgs a) {
     extern __shared__ __align__(16) unsigned char pa_lds[];
-    __shared__ u64 sums[PA_BLOCK / 64];
-    __shared__ u32 s_nnew, s_sel, s_sp;
-    __shared__ u32 stk[24];
+    u64* sums = reinterpret_cast<u64*>(pa_lds + PA_OFF_SUMS);
+    u32& s_nnew = *reinterpret_cast<u32*>(pa_lds + PA_OFF_MISC);
     u64* lkey = reinterpret_cast<u64*>(pa_lds);
     u32* lref = reinterpret_cast<u32*>(pa_lds + PA_OFF_LREF);
     u32* lhdl = reinterpret_cast<u32*>(pa_lds + PA_OFF_HDL);
@@ -812,8 +895,11 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
     u32* ta = toff + PA_TILES_MAX;
     const u32 tid = threadIdx.x;
     // Workgroups are dealt to the eight XCDs in turn: each XCD takes a run of consecutive partitions,
-    // whose start words and staging segments share cache lines, into its own L2.
-    const u32 p = (blockIdx.x & 7u) * (a.P >> 3) + (blockIdx.x >> 3);
+    // whose start words and staging segments share cache lines, into its own L2. With an order (the
+    // partitions of each run ranked by the entries the last push found in them) the fullest go
+    // first: a kernel of several rounds of workgroups ends when its last workgroup does, and a
+    // crowded partition that starts in the last round would be that one.
+    const u32 p = a.order ? a.order[blockIdx.x] : (blockIdx.x & 7u) * (a.P >> 3) + (blockIdx.x >> 3);
     const u64 seg = tile_segments(a, p, tid, sums, toff, ta);
     const u32 np = (u32)seg, s = (u32)(seg >> 32);
     // the row count as it is when this operation begins (this launch hands out no rows)
@@ -821,6 +907,7 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
     if (tid == 0) {
         s_nnew = 0;
         a.pstart[p] = s;
+        a.psize[p] = np;
         // the last partition's block knows how many entries the tiles left in all: a hint for the
         // partition size of the next push (read by the host when it plans that push)
         if (p + 1 == a.P)
@@ -832,7 +919,7 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
         return;
     }
     __syncthreads();
-    if (np <= a.cap) {
+    if (__builtin_expect(np <= a.cap, 1)) {
         uint4 e[PA_ITEMS];
 #pragma unroll
         for (u32 j = 0; j < PA_ITEMS; ++j) {
@@ -851,58 +938,7 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
         __syncthreads();
         apply_pass<T>(t, pa_lds, sums, &s_nnew, grads, psum, ngrad, a, s, np);
     } else {
-        // More entries than a pass holds (several keys that are met in most tiles share the
-        // partition): passes over the entries by hash class. A class that still holds too many is
-        // split in two by the next hash bit, down to 1024 classes; a key has at most one entry per
-        // tile, so only keys that agree in all ten bits could make the last split fail.
-        u32 lgR = 1;
-        while ((np >> lgR) > a.cap / 2 && lgR < 10u) ++lgR;
-        for (u32 r0 = 0; r0 < (1u << lgR); ++r0) {
-            __syncthreads();
-            if (tid == 0) {
-                stk[0] = (lgR << 16) | r0;
-                s_sp = 1;
-            }
-            __syncthreads();
-            while (s_sp) {  // block-uniform: read between barriers
-                const u32 top = stk[s_sp - 1];
-                __syncthreads();
-                if (tid == 0) {
-                    s_sp -= 1;
-                    s_sel = 0;
-                }
-                __syncthreads();
-                const u32 lg = top >> 16, cls = top & 0xFFFFu, mask = (1u << lg) - 1u;
-                tile_segments(a, p, tid, sums, toff, ta);  // (a pass overwrites them)
-                __syncthreads();
-                for (u32 i = tid; i < np; i += PA_BLOCK) {
-                    const uint4 e = partition_entry(a, toff, ta, i);
-                    const u64 key = ((u64)e.y << 32) | e.x;
-                    if (((u32)(hash64(key) >> 53) & mask) == cls) {
-                        const u32 pos = atomicAdd(&s_sel, 1u);
-                        if (pos < a.cap) {
-                            lkey[pos] = key;
-                            lref[pos] = e.z;
-                            lhdl[pos] = e.w;
-                        }
-                    }
-                }
-                __syncthreads();
-                const u32 sel = s_sel;
-                if (sel > a.cap) {
-                    if (lg >= 10u) {  // reported, never silent
-                        if (tid == 0) t.counters[CNT_PART_ERR] = 1u;
-                    } else if (tid == 0) {
-                        stk[s_sp] = ((lg + 1u) << 16) | cls;
-                        stk[s_sp + 1] = ((lg + 1u) << 16) | (cls + (1u << lg));
-                        s_sp += 2;
-                    }
-                } else if (sel) {
-                    apply_pass<T>(t, pa_lds, sums, &s_nnew, grads, psum, ngrad, a, s, sel);
-                }
-                __syncthreads();
-            }
-        }
+        apply_crowded<T>(t, pa_lds, grads, psum, ngrad, a, p, s, np);
     }
     __syncthreads();
     if (tid == 0) {
@@ -914,14 +950,40 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
 // ---- 3. insert ------------------------------------------------------------------------------------
 constexpr u32 PI_BLOCK = 256;
 
+// The order for the apply kernel of the next push with this plan: the partitions of run g (P / 8
+// consecutive ones, at most 512) ranked by their entries, fullest first, ties by number; workgroup
+// x of that kernel is on XCD x & 7 and takes the (x >> 3)-th of run x & 7. A permutation of the
+// partitions whatever the sizes are.
+__device__ __forceinline__ void rank_partitions(const u32* __restrict__ psize, u32* __restrict__ order, u32 P, u32 g,
+                                                u32 tid) {
+    __shared__ u32 sz[PT_MAX_PARTS / 8];
+    const u32 m = P >> 3;
+    for (u32 i = tid; i < m; i += PI_BLOCK) sz[i] = psize[g * m + i];
+    __syncthreads();
+    for (u32 i = tid; i < m; i += PI_BLOCK) {
+        const u32 mine = sz[i];
+        u32 rank = 0;
+        for (u32 j = 0; j < m; ++j) {
+            const u32 o = sz[j];
+            rank += (o > mine || (o == mine && j < i)) ? 1u : 0u;
+        }
+        order[(rank << 3) | g] = g * m + i;
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(PI_BLOCK) void part_insert_kernel(TableDev t, const u32* __restrict__ new_slot,
                                                                 const T* __restrict__ ngrad,
                                                                 const u32* __restrict__ new_count,
-                                                                const u32* __restrict__ pstart, u32 P, u32 units) {
+                                                                const u32* __restrict__ pstart, u32 P, u32 units,
+                                                                const u32* __restrict__ psize, u32* __restrict__ order) {
     constexpr u32 N = sizeof(T) / 4;
     __shared__ u32 red[PI_BLOCK / 64];
     const u32 p = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    if (p >= P) {  // eight more workgroups, when an order is wanted: one per run of P / 8 partitions
+        rank_partitions(psize, order, P, p - P, tid);
+        return;
+    }
     if (!t.counters[CNT_ANY_NEW]) {  // block-uniform: the batch inserted nothing
         if (p == 0 && tid == 0) publish_rows(t, t.counters[CNT_ENTRY]);
         return;
@@ -1032,6 +1094,8 @@ PartSizes part_sizes(uint32_t dim, size_t n) {
     z.new_slot = np * 4;
     z.new_count = PT_MAX_PARTS * 4;
     z.ngrad = np * (size_t)dim * 4;
+    z.psize = PT_MAX_PARTS * 4;
+    z.order = PT_MAX_PARTS * 4;
     return z;
 }
 
@@ -1061,12 +1125,13 @@ hipError_t launch_part_tile(const TableDev& t, const PartPlan& pl, const PartBuf
 }
 
 hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads, bool insert,
-                             bool handles, bool verify, hipStream_t s) {
+                             bool handles, bool verify, bool use_order, hipStream_t s) {
     const bool v4 = (t.dim % 4 == 0) && aligned16(grads);
     u32 pow2 = 1;
     while (pow2 < pl.n_tiles) pow2 <<= 1;
     ApplyArgs a{b.stage, b.starts, b.pstart, pl.n_tiles, pl.P, pl.n, pow2 / 2, b.new_slot, b.new_count,
-                v4 ? t.dim / 4 : t.dim, insert ? 1 : 0, g_part_cap, handles ? 1 : 0, (handles && verify) ? 1 : 0};
+                v4 ? t.dim / 4 : t.dim, insert ? 1 : 0, g_part_cap, handles ? 1 : 0, (handles && verify) ? 1 : 0,
+                use_order ? b.order : nullptr, b.psize};
     if (v4)
         part_apply_kernel<float4><<<pl.P, PA_BLOCK, PA_LDS, s>>>(t, reinterpret_cast<const float4*>(grads),
                                                                  reinterpret_cast<const float4*>(b.psum),
@@ -1077,13 +1142,14 @@ hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBu
 }
 
 hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads,
-                              hipStream_t s) {
+                              bool make_order, hipStream_t s) {
+    const u32 grid = pl.P + (make_order ? 8u : 0u);
     if ((t.dim % 4 == 0) && aligned16(grads))
-        part_insert_kernel<float4><<<pl.P, PI_BLOCK, 0, s>>>(t, b.new_slot, reinterpret_cast<const float4*>(b.ngrad),
-                                                             b.new_count, b.pstart, pl.P, t.dim / 4);
+        part_insert_kernel<float4><<<grid, PI_BLOCK, 0, s>>>(t, b.new_slot, reinterpret_cast<const float4*>(b.ngrad),
+                                                             b.new_count, b.pstart, pl.P, t.dim / 4, b.psize, b.order);
     else
-        part_insert_kernel<float><<<pl.P, PI_BLOCK, 0, s>>>(t, b.new_slot, b.ngrad, b.new_count, b.pstart, pl.P,
-                                                            t.dim);
+        part_insert_kernel<float><<<grid, PI_BLOCK, 0, s>>>(t, b.new_slot, b.ngrad, b.new_count, b.pstart, pl.P,
+                                                            t.dim, b.psize, b.order);
     return hipGetLastError();
 }
 

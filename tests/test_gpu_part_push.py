@@ -129,6 +129,53 @@ def test_partitions_that_need_several_passes(ps, orc, wl):
     t.close()
 
 
+M64 = (1 << 64) - 1
+C1, C2, GOLD = 0xff51afd7ed558ccd, 0xc4ceb9fe1a85ec53, 0x9E3779B97F4A7C15
+
+
+def unmix64(h):
+    """Inverse of MurmurHash3's 64-bit finaliser (the table's hash), on numpy uint64 arrays."""
+    i1, i2 = np.uint64(pow(C1, -1, 1 << 64)), np.uint64(pow(C2, -1, 1 << 64))
+    h = h ^ (h >> np.uint64(33))
+    h = h * i2
+    h = h ^ (h >> np.uint64(33))
+    h = h * i1
+    return h ^ (h >> np.uint64(33))
+
+
+def test_hot_keys_that_agree_in_partition_and_class_bits(ps, orc, wl):
+    """Five keys met in every one of 700 tiles, made to share one bucket of the hash array (hence
+    the partition) and the low 30 bits of the hash by which a crowded partition is taken in passes:
+    their 3,500 entries do not fit a pass, and the classes split thirty times before they part."""
+    rng = np.random.default_rng(21)
+    n_table, dim, tiles, tile = 40000, 4, 700, 4096
+    n = tiles * tile
+    # (room for a row per key of the batch: a table that might fill takes the sorted push)
+    t = ps.Table(dim, capacity=n_table + n, max_batch=n, **OPTS["sgd"])
+    r = orc.Oracle(dim, capacity=n_table + n, **OPTS["sgd"])
+    table_keys = fill(t, r, wl, rng, n_table, "sgd", dim, seed=8)
+    bucket_mask = np.uint64(t.stats().slots // 4 - 1)
+    hot = np.zeros(0, dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        for chunk in range(64):
+            if len(hot) >= 5:
+                break
+            i = np.arange(chunk << 22, (chunk + 1) << 22, dtype=np.uint64) + np.uint64(1)
+            c = (i << np.uint64(30)) | np.uint64(0x2AAAAAAA)
+            h = unmix64(c) ^ np.uint64(GOLD)       # hash of the key whose class hash is c
+            hot = np.concatenate([hot, unmix64(h[(h & bucket_mask) == np.uint64(77)])])
+    hot = hot[:5]
+    assert len(hot) == 5 and len(set(hot.tolist()) | set(table_keys.tolist())) == n_table + 5
+    q = table_keys[rng.integers(0, n_table, (tiles, tile))]
+    q[:, :5] = hot
+    q = np.ascontiguousarray(q.reshape(-1))
+    g = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+    assert t.push(q, g) == 0 and r.push(q, g) == 0
+    assert t.size() == r.size() == n_table + 5
+    same(t, r, exact=True)
+    t.close()
+
+
 def test_track_increment_through_the_partitioned_push(ps, orc, wl):
     rng = np.random.default_rng(13)
     n_table, n, dim = 30000, 20000, 4
