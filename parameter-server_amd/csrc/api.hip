@@ -206,7 +206,7 @@ struct pshbm_table {
     DevBuf ws_slot, ws_row, ws_idx, ws_srow, ws_sidx, ws_sort, ws_hdr, ws_pval, ws_wrow, ws_wval, ws_won;
     unsigned won_parity = 0;  // which half of ws_won the next inserting operation counts into
     // scratch of the partitioned push (batches of PART_MIN_KEYS keys and more)
-    DevBuf pt_stage, pt_starts, pt_pstart, pt_psum, pt_new_slot, pt_new_count, pt_ngrad, pt_psize, pt_order;
+    DevBuf pt_stage, pt_starts, pt_pstart, pt_psum, pt_new_slot, pt_new_count, pt_ngrad, pt_psize, pt_order, pt_resv;
     size_t part_keys = 0;       // batch size those arrays serve
     // pt_order ranks the partitions of the plan {order_P partitions, order_mask buckets} (0: of none yet)
     uint32_t order_P = 0, order_mask = 0;
@@ -402,6 +402,8 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
         ST_TRY(ensure(t, t->pt_ngrad, z.ngrad));
         ST_TRY(ensure(t, t->pt_psize, z.psize));
         ST_TRY(ensure(t, t->pt_order, z.order));
+        ST_TRY(ensure(t, t->pt_resv, z.resv));
+        HIP_TRY(t, hipMemset(t->pt_resv.p, 0, t->pt_resv.bytes));
         t->order_P = 0;
         t->part_keys = pk;
     }
@@ -612,6 +614,7 @@ Workspace table_workspace(pshbm_table* t) {
         w.part.ngrad = static_cast<float*>(t->pt_ngrad.p);
         w.part.psize = static_cast<uint32_t*>(t->pt_psize.p);
         w.part.order = static_cast<uint32_t*>(t->pt_order.p);
+        w.part.resv = static_cast<uint32_t*>(t->pt_resv.p);
     }
     return w;
 }
@@ -650,7 +653,7 @@ int32_t push_with(pshbm_table* t, const Workspace& w, const uint64_t* d_keys, co
                                        (flags & PSHBM_PUSH_VERIFY_HANDLES) != 0, use_order, s));
         if (insert) {
             const bool make_order = pl.P >= PART_ORDER_MIN;
-            HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_INSERT, launch_part_insert(t->d, pl, w.part, d_grads, make_order, s));
+            HIP_TRY_PROF(t, s, PSHBM_PHASE_PART_INSERT, launch_part_insert(t->d, pl, w.part, d_grads, use_order, make_order, s));
             if (make_order) {
                 t->order_P = pl.P;
                 t->order_mask = t->d.bucket_mask;
@@ -747,7 +750,7 @@ void destroy_impl(pshbm_table* t) {
                       &t->ws_pval, &t->ws_wrow, &t->ws_wval, &t->ws_won, &t->st_keys, &t->st_vals,  &t->st_raw,
                       &t->ms_dead, &t->ms_tiles, &t->ms_lists, &t->ms_fe,
                       &t->pt_stage, &t->pt_starts, &t->pt_pstart, &t->pt_psum, &t->pt_new_slot, &t->pt_new_count,
-                      &t->pt_ngrad, &t->pt_psize, &t->pt_order,
+                      &t->pt_ngrad, &t->pt_psize, &t->pt_order, &t->pt_resv,
                       &t->q_keys,  &t->q_grads};
     for (DevBuf* b : bufs)
         if (b->p) (void)dev_free(t->device, b->p);

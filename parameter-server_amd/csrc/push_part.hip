@@ -457,8 +457,9 @@ struct ApplyArgs {
     u32 cap;  // entries a pass holds: PA_CAP, or less when a test wants to see the passes
     int handles;  // the entries carry rows that an earlier pull reported
     int verify;   // ... which count only where row_keys agrees
-    const u32* order;  // the partition each workgroup takes, or null
+    const u32* order;  // the work item of each workgroup (see rank_partitions), or null
     u32* psize;        // out: entries of each partition
+    u32* resv;         // per partition, zero: where the workgroups that share a partition reserve room for new keys
 };
 
 // The optimizer step of the distinct keys of a pass: a key with one entry takes its gradient row, a
@@ -818,7 +819,7 @@ __device__ __forceinline__ uint4 partition_entry(const ApplyArgs& a, const u32* 
 template <typename T>
 __device__ __forceinline__ void apply_crowded(const TableDev& t, unsigned char* pa_lds, const T* __restrict__ grads,
                                               const T* __restrict__ psum, T* __restrict__ ngrad, const ApplyArgs& a,
-                                              u32 p, u32 s, u32 np) {
+                                              u32 p, u32 s, u32 np, u32 lg0, u32 cls0, u32 unit) {
     u64* sums = reinterpret_cast<u64*>(pa_lds + PA_OFF_SUMS);
     u32* misc = reinterpret_cast<u32*>(pa_lds + PA_OFF_MISC);
     u32& s_sel = misc[1];
@@ -832,11 +833,20 @@ __device__ __forceinline__ void apply_crowded(const TableDev& t, unsigned char* 
     u32* stk_lg = reinterpret_cast<u32*>(stk_cls + PA_STACK);
     const u32 tid = threadIdx.x;
     if (tid == 0) {
-        stk_cls[0] = 0;
-        stk_cls[1] = 1;
-        stk_lg[0] = stk_lg[1] = 1;
-        s_sp = 2;
+        if (lg0) {  // this workgroup's share of a partition that several take: one class
+            stk_cls[0] = cls0;
+            stk_lg[0] = lg0;
+            s_sp = 1;
+        } else {
+            stk_cls[0] = 0;
+            stk_cls[1] = 1;
+            stk_lg[0] = stk_lg[1] = 1;
+            s_sp = 2;
+        }
     }
+    // Workgroups that share a partition share its room for new keys: each reserves as much as its
+    // class has entries (known after its first sweep) and parks its new keys there.
+    bool reserve = lg0 != 0 && a.insert;  // block-uniform
     __syncthreads();
     while (s_sp) {  // block-uniform: read between barriers
         const u32 lg = stk_lg[s_sp - 1];
@@ -864,6 +874,15 @@ __device__ __forceinline__ void apply_crowded(const TableDev& t, unsigned char* 
         }
         __syncthreads();
         const u32 sel = s_sel;
+        if (reserve) {
+            if (tid == 0) {
+                misc[4] = atomicAdd(&a.resv[p], sel);
+                a.pstart[unit] = s + misc[4];
+            }
+            __syncthreads();
+            s += misc[4];
+            reserve = false;
+        }
         if (sel > a.cap) {
             if (lg >= 64u) {  // one key with more entries than a pass holds: reported, never silent
                 if (tid == 0) t.counters[CNT_PART_ERR] = 1u;
@@ -899,14 +918,23 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
     // partitions of each run ranked by the entries the last push found in them) the fullest go
     // first: a kernel of several rounds of workgroups ends when its last workgroup does, and a
     // crowded partition that starts in the last round would be that one.
-    const u32 p = a.order ? a.order[blockIdx.x] : (blockIdx.x & 7u) * (a.P >> 3) + (blockIdx.x >> 3);
+    // A work item names a partition and, for one that the last push found crowded, one of the
+    // 2, 4 or 8 classes of its keys (by the low bits of the second hash): that many workgroups
+    // share it from the start instead of one taking its passes one after the other.
+    const u32 unit = blockIdx.x;
+    const u32 item = a.order ? a.order[unit] : (unit & 7u) * (a.P >> 3) + (unit >> 3);
+    if (item == NONE32) {  // (block-uniform) a spare slot of the order
+        if (tid == 0) a.new_count[unit] = 0;
+        return;
+    }
+    const u32 p = item & 0xFFFFu, lg0 = (item >> 16) & 3u, cls0 = item >> 20;
     const u64 seg = tile_segments(a, p, tid, sums, toff, ta);
     const u32 np = (u32)seg, s = (u32)(seg >> 32);
     // the row count as it is when this operation begins (this launch hands out no rows)
     if (p == 0 && tid == 0) t.counters[CNT_ENTRY] = t.counters[CNT_ROWS];
     if (tid == 0) {
         s_nnew = 0;
-        a.pstart[p] = s;
+        a.pstart[unit] = s;
         a.psize[p] = np;
         // the last partition's block knows how many entries the tiles left in all: a hint for the
         // partition size of the next push (read by the host when it plans that push)
@@ -915,11 +943,11 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     if (np == 0) {
-        if (tid == 0) a.new_count[p] = 0;
+        if (tid == 0) a.new_count[unit] = 0;
         return;
     }
     __syncthreads();
-    if (__builtin_expect(np <= a.cap, 1)) {
+    if (__builtin_expect(np <= a.cap && lg0 == 0, 1)) {
         uint4 e[PA_ITEMS];
 #pragma unroll
         for (u32 j = 0; j < PA_ITEMS; ++j) {
@@ -938,11 +966,11 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
         __syncthreads();
         apply_pass<T>(t, pa_lds, sums, &s_nnew, grads, psum, ngrad, a, s, np);
     } else {
-        apply_crowded<T>(t, pa_lds, grads, psum, ngrad, a, p, s, np);
+        apply_crowded<T>(t, pa_lds, grads, psum, ngrad, a, p, s, np, lg0, cls0, unit);
     }
     __syncthreads();
     if (tid == 0) {
-        a.new_count[p] = s_nnew;
+        a.new_count[unit] = s_nnew;
         if (s_nnew) t.counters[CNT_ANY_NEW] = 1u;  // (every writer writes the same value)
     }
 }
@@ -950,15 +978,29 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
 // ---- 3. insert ------------------------------------------------------------------------------------
 constexpr u32 PI_BLOCK = 256;
 
-// The order for the apply kernel of the next push with this plan: the partitions of run g (P / 8
-// consecutive ones, at most 512) ranked by their entries, fullest first, ties by number; workgroup
-// x of that kernel is on XCD x & 7 and takes the (x >> 3)-th of run x & 7. A permutation of the
-// partitions whatever the sizes are.
-__device__ __forceinline__ void rank_partitions(const u32* __restrict__ psize, u32* __restrict__ order, u32 P, u32 g,
-                                                u32 tid) {
+// The work items for the apply kernel of the next push with this plan. Run g (P / 8 consecutive
+// partitions, at most 512) gets P / 8 + P / 64 slots; workgroup x of that kernel is on XCD x & 7
+// and takes slot x >> 3 of run x & 7. The partitions of the run are ranked by the entries this
+// push found in them, fullest first (ties by number). One that was crowded, or nearly (a pass holds
+// PA_CAP entries), gets 2, 4 or 8 slots while spare slots last: item = partition | log2(slots) <<
+// 16 | class << 20, each workgroup taking the keys of one class. The rest get one slot each, and
+// what is left of the spare slots says so (NONE32). Every partition is covered whatever the sizes
+// are. The reservation words of the run are cleared for the next push.
+constexpr u32 PART_SPLIT_ABOVE = PA_CAP - PA_CAP / 7;  // 1756 entries: crowded next time, for all we know
+constexpr u32 PART_SHARE = 1300;                        // entries a workgroup of a shared partition should get
+
+__host__ __device__ inline u32 part_units(u32 P, bool ordered) { return ordered ? P + P / 8 : P; }
+
+__device__ __forceinline__ void rank_partitions(const u32* __restrict__ psize, u32* __restrict__ order,
+                                                u32* __restrict__ resv, u32 P, u32 g, u32 tid) {
     __shared__ u32 sz[PT_MAX_PARTS / 8];
-    const u32 m = P >> 3;
-    for (u32 i = tid; i < m; i += PI_BLOCK) sz[i] = psize[g * m + i];
+    __shared__ u16 sorted[PT_MAX_PARTS / 8];
+    __shared__ u32 s_head, s_items;
+    const u32 m = P >> 3, slots = m + (m >> 3);
+    for (u32 i = tid; i < m; i += PI_BLOCK) {
+        sz[i] = psize[g * m + i];
+        resv[g * m + i] = 0;
+    }
     __syncthreads();
     for (u32 i = tid; i < m; i += PI_BLOCK) {
         const u32 mine = sz[i];
@@ -967,8 +1009,28 @@ __device__ __forceinline__ void rank_partitions(const u32* __restrict__ psize, u
             const u32 o = sz[j];
             rank += (o > mine || (o == mine && j < i)) ? 1u : 0u;
         }
-        order[(rank << 3) | g] = g * m + i;
+        sorted[rank] = (u16)i;
     }
+    __syncthreads();
+    if (tid == 0) {  // the partitions that get more than one slot are the first of the ranking
+        u32 spare = m >> 3, pos = 0, r = 0;
+        for (; r < m && spare; ++r) {
+            const u32 i = sorted[r], size = sz[i];
+            if (size <= PART_SPLIT_ABOVE) break;
+            u32 lg = 1;
+            while ((size >> lg) > PART_SHARE && lg < 3u) ++lg;
+            while (lg && (1u << lg) - 1u > spare) --lg;
+            if (lg == 0) break;
+            spare -= (1u << lg) - 1u;
+            for (u32 c = 0; c < (1u << lg); ++c) order[(pos++ << 3) | g] = (g * m + i) | (lg << 16) | (c << 20);
+        }
+        s_head = r;
+        s_items = pos;
+    }
+    __syncthreads();
+    const u32 head = s_head, items = s_items;
+    for (u32 r = head + tid; r < m; r += PI_BLOCK) order[((items + r - head) << 3) | g] = g * m + sorted[r];
+    for (u32 x = items + (m - head) + tid; x < slots; x += PI_BLOCK) order[(x << 3) | g] = NONE32;
 }
 
 template <typename T>
@@ -976,12 +1038,15 @@ __global__ __launch_bounds__(PI_BLOCK) void part_insert_kernel(TableDev t, const
                                                                 const T* __restrict__ ngrad,
                                                                 const u32* __restrict__ new_count,
                                                                 const u32* __restrict__ pstart, u32 P, u32 units,
-                                                                const u32* __restrict__ psize, u32* __restrict__ order) {
+                                                                const u32* __restrict__ psize, u32* __restrict__ order,
+                                                                u32* __restrict__ resv, u32 n_parts) {
+    // P: workgroups the apply kernel had (one per partition, or the slots of its order); each left
+    // its new keys parked at pstart[its number], new_count of them. n_parts: partitions.
     constexpr u32 N = sizeof(T) / 4;
     __shared__ u32 red[PI_BLOCK / 64];
     const u32 p = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
-    if (p >= P) {  // eight more workgroups, when an order is wanted: one per run of P / 8 partitions
-        rank_partitions(psize, order, P, p - P, tid);
+    if (p >= P) {  // eight more workgroups, when an order is wanted: one per run of n_parts / 8 partitions
+        rank_partitions(psize, order, resv, n_parts, p - P, tid);
         return;
     }
     if (!t.counters[CNT_ANY_NEW]) {  // block-uniform: the batch inserted nothing
@@ -1089,13 +1154,14 @@ PartSizes part_sizes(uint32_t dim, size_t n) {
     const size_t np = n_tiles * PT_TILE;
     z.stage = np * 16;
     z.starts = n_tiles * (PT_MAX_PARTS + 1) * 4;
-    z.pstart = (PT_MAX_PARTS + 1) * 4;
+    z.pstart = (part_units(PT_MAX_PARTS, true) + 1) * 4;
     z.psum = n_tiles * PT_MAX_MULTI * (size_t)dim * 4;
     z.new_slot = np * 4;
-    z.new_count = PT_MAX_PARTS * 4;
+    z.new_count = part_units(PT_MAX_PARTS, true) * 4;
     z.ngrad = np * (size_t)dim * 4;
     z.psize = PT_MAX_PARTS * 4;
-    z.order = PT_MAX_PARTS * 4;
+    z.order = part_units(PT_MAX_PARTS, true) * 4;
+    z.resv = PT_MAX_PARTS * 4;
     return z;
 }
 
@@ -1131,25 +1197,28 @@ hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBu
     while (pow2 < pl.n_tiles) pow2 <<= 1;
     ApplyArgs a{b.stage, b.starts, b.pstart, pl.n_tiles, pl.P, pl.n, pow2 / 2, b.new_slot, b.new_count,
                 v4 ? t.dim / 4 : t.dim, insert ? 1 : 0, g_part_cap, handles ? 1 : 0, (handles && verify) ? 1 : 0,
-                use_order ? b.order : nullptr, b.psize};
+                use_order ? b.order : nullptr, b.psize, b.resv};
+    const u32 grid = part_units(pl.P, use_order);
     if (v4)
-        part_apply_kernel<float4><<<pl.P, PA_BLOCK, PA_LDS, s>>>(t, reinterpret_cast<const float4*>(grads),
+        part_apply_kernel<float4><<<grid, PA_BLOCK, PA_LDS, s>>>(t, reinterpret_cast<const float4*>(grads),
                                                                  reinterpret_cast<const float4*>(b.psum),
                                                                  reinterpret_cast<float4*>(b.ngrad), a);
     else
-        part_apply_kernel<float><<<pl.P, PA_BLOCK, PA_LDS, s>>>(t, grads, b.psum, b.ngrad, a);
+        part_apply_kernel<float><<<grid, PA_BLOCK, PA_LDS, s>>>(t, grads, b.psum, b.ngrad, a);
     return hipGetLastError();
 }
 
 hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads,
-                              bool make_order, hipStream_t s) {
-    const u32 grid = pl.P + (make_order ? 8u : 0u);
+                              bool used_order, bool make_order, hipStream_t s) {
+    const u32 units = part_units(pl.P, used_order);  // workgroups the apply kernel had
+    const u32 grid = units + (make_order ? 8u : 0u);
     if ((t.dim % 4 == 0) && aligned16(grads))
         part_insert_kernel<float4><<<grid, PI_BLOCK, 0, s>>>(t, b.new_slot, reinterpret_cast<const float4*>(b.ngrad),
-                                                             b.new_count, b.pstart, pl.P, t.dim / 4, b.psize, b.order);
+                                                             b.new_count, b.pstart, units, t.dim / 4, b.psize, b.order,
+                                                             b.resv, pl.P);
     else
-        part_insert_kernel<float><<<grid, PI_BLOCK, 0, s>>>(t, b.new_slot, b.ngrad, b.new_count, b.pstart, pl.P,
-                                                            t.dim, b.psize, b.order);
+        part_insert_kernel<float><<<grid, PI_BLOCK, 0, s>>>(t, b.new_slot, b.ngrad, b.new_count, b.pstart, units,
+                                                            t.dim, b.psize, b.order, b.resv, pl.P);
     return hipGetLastError();
 }
 

@@ -214,14 +214,15 @@ struct PartPlan {
     uint32_t n, n_tiles, P, part_shift;
 };
 struct PartSizes {
-    size_t stage, starts, pstart, psum, new_slot, new_count, ngrad, psize, order;
+    size_t stage, starts, pstart, psum, new_slot, new_count, ngrad, psize, order, resv;
 };
 struct PartBufs {
     uint4* stage;  // entries {key low, key high, reference, row handle}: a block per tile, grouped by partition
     uint32_t *starts, *pstart, *new_slot, *new_count;
     float *psum, *ngrad;
     uint32_t* psize;  // entries each partition held in the last push
-    uint32_t* order;  // partitions in the order the apply kernel's workgroups should take them
+    uint32_t* order;  // what each workgroup of the apply kernel should take: partitions, fullest first
+    uint32_t* resv;   // per partition, zero between pushes: room reserved by the workgroups that share it
 };
 // entries_per_key: what the tiles of recent batches left per key (1 = no key repeats inside a tile);
 // partitions are sized so that a pass of the apply kernel is well filled but rarely overflows.
@@ -233,13 +234,15 @@ hipError_t part_init();  // once per device, before the first launch
 // verify: a handle counts only if row_keys[handle] is the key.
 hipError_t launch_part_tile(const TableDev& t, const PartPlan& pl, const PartBufs& b, const uint64_t* keys,
                             const float* grads, const uint32_t* handles, hipStream_t s);
-// use_order: workgroup x takes partition b.order[x] (a permutation of the partitions that an earlier
-// push with the same plan left: fullest first); otherwise the partitions go round the XCDs in turn.
+// use_order: workgroup x takes work item b.order[x] (left by an earlier push with the same plan: the
+// partitions fullest first, the crowded ones shared by several workgroups); otherwise the partitions go
+// round the XCDs in turn.
 hipError_t launch_part_apply(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads, bool insert,
                              bool handles, bool verify, bool use_order, hipStream_t s);
-// make_order: also rank the partitions by the entries the apply kernel found in them (b.psize) into b.order.
+// used_order: what the apply kernel was launched with. make_order: also rank the partitions by the
+// entries the apply kernel found in them (b.psize) into b.order, and clear b.resv.
 hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartBufs& b, const float* grads,
-                              bool make_order, hipStream_t s);
+                              bool used_order, bool make_order, hipStream_t s);
 // Partitions from which an order pays: the apply kernel's workgroups then run in several rounds.
 constexpr uint32_t PART_ORDER_MIN = 1024;
 // Entries a pass of the apply kernel takes (0 = the default, 2048): a test hook that makes small

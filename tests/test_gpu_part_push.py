@@ -151,8 +151,8 @@ def test_hot_keys_that_agree_in_partition_and_class_bits(ps, orc, wl):
     n_table, dim, tiles, tile = 40000, 4, 700, 4096
     n = tiles * tile
     # (room for a row per key of the batch: a table that might fill takes the sorted push)
-    t = ps.Table(dim, capacity=n_table + n, max_batch=n, **OPTS["sgd"])
-    r = orc.Oracle(dim, capacity=n_table + n, **OPTS["sgd"])
+    t = ps.Table(dim, capacity=n_table + n + 1000, max_batch=n, **OPTS["sgd"])
+    r = orc.Oracle(dim, capacity=n_table + n + 1000, **OPTS["sgd"])
     table_keys = fill(t, r, wl, rng, n_table, "sgd", dim, seed=8)
     bucket_mask = np.uint64(t.stats().slots // 4 - 1)
     hot = np.zeros(0, dtype=np.uint64)
@@ -173,6 +173,21 @@ def test_hot_keys_that_agree_in_partition_and_class_bits(ps, orc, wl):
     assert t.push(q, g) == 0 and r.push(q, g) == 0
     assert t.size() == r.size() == n_table + 5
     same(t, r, exact=True)
+    # The next pushes find that partition in the order the first one left: shared by several
+    # workgroups from the start, a class of keys each. New keys of that partition (their buckets are
+    # near the hot keys') then park where the workgroup that meets them has reserved room.
+    bucket_bits = int(bucket_mask + 1).bit_length() - 1
+    assert bucket_bits >= 19            # buckets 0 .. 127 share a partition however the push is cut (at most 4096 ways)
+    for step in range(2):
+        with np.errstate(over="ignore"):
+            k = np.arange(300, dtype=np.uint64)
+            near = unmix64(((k + np.uint64(1000 * (step + 1))) << np.uint64(40)) | (k % np.uint64(50) + np.uint64(70)))
+        q2 = q.copy()
+        q2[rng.choice(n, 300, replace=False)] = near
+        g2 = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+        assert t.push(q2, g2) == 0 and r.push(q2, g2) == 0
+        assert t.size() == r.size()
+        same(t, r, exact=True)
     t.close()
 
 
