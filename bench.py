@@ -57,18 +57,18 @@ KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist"
 TRAFFIC_FROM_PROFILES = {
     # (config, phase): (bytes, summary)
     ("c1", "pull"): (19226624, "profiles/c1_pull_trace_and_hbm_counters.md"),
-    ("c2", "pull"): (196069376, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
-    ("c2", "part_tile"): (78283776, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
-    ("c2", "part_apply"): (152215552, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
-    ("c3", "pull"): (703240192, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c3", "part_tile"): (450812928, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c3", "part_apply"): (378161152, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "pull"): (558432256, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "part_tile"): (233840640, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "part_apply"): (663741440, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c5", "pull"): (3204072448, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
-    ("c5", "part_tile"): (1380431872, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
-    ("c5", "part_apply"): (2715749376, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "pull"): (196080640, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "part_tile"): (78080000, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "part_apply"): (146957312, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "pull"): (703201280, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "part_tile"): (450787328, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "part_apply"): (379213824, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "pull"): (558399488, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_tile"): (232773632, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_apply"): (777693184, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "pull"): (3204252672, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "part_tile"): (1380334592, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "part_apply"): (2990774272, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
 }
 
 

@@ -452,8 +452,9 @@ int32_t read_counters(pshbm_table* t, hipStream_t s) {
                                     "belonged to, and every push since, was not applied (keys they inserted "
                                     "keep their initial values); pshbm_clear resets the table");
     if (t->h_counters[CNT_PART_ERR])
-        return fail(t, PSHBM_FATAL, "a partition of a push held more entries of one hash class than a pass takes: "
-                                    "that push was applied in part; pshbm_clear resets the table");
+        return fail(t, PSHBM_FATAL, "a push held more entries of one key than a pass of its apply kernel takes (only a "
+                                    "pass capacity lowered by pshbm_debug_part_pass_capacity allows that): that push "
+                                    "was applied in part; pshbm_clear resets the table");
     return PSHBM_OK;
 }
 
