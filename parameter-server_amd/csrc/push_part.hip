@@ -981,11 +981,13 @@ constexpr u32 PI_BLOCK = 256;
 // The work items for the apply kernel of the next push with this plan. Run g (P / 8 consecutive
 // partitions, at most 512) gets P / 8 + P / 64 slots; workgroup x of that kernel is on XCD x & 7
 // and takes slot x >> 3 of run x & 7. The partitions of the run are ranked by the entries this
-// push found in them, fullest first (ties by number). One that was crowded, or nearly (a pass holds
-// PA_CAP entries), gets 2, 4 or 8 slots while spare slots last: item = partition | log2(slots) <<
-// 16 | class << 20, each workgroup taking the keys of one class. The rest get one slot each, and
-// what is left of the spare slots says so (NONE32). Every partition is covered whatever the sizes
-// are. The reservation words of the run are cleared for the next push.
+// push found in them, fullest first (ties by number). Those that were crowded, or nearly (a pass
+// holds PA_CAP entries), come first and get 2, 4 or 8 slots each while spare slots last: item =
+// partition | log2(slots) << 16 | class << 20, each workgroup taking the keys of one class. The
+// others follow with one slot each in their natural order -- neighbours share cache lines of start
+// words and staging blocks, and run at about the same time that way -- and what is left of the
+// spare slots says so (NONE32). Every partition is covered whatever the sizes are. The
+// reservation words of the run are cleared for the next push.
 constexpr u32 PART_SPLIT_ABOVE = PA_CAP - PA_CAP / 7;  // 1756 entries: crowded next time, for all we know
 constexpr u32 PART_SHARE = 1300;                        // entries a workgroup of a shared partition should get
 
@@ -994,7 +996,7 @@ __host__ __device__ inline u32 part_units(u32 P, bool ordered) { return ordered 
 __device__ __forceinline__ void rank_partitions(const u32* __restrict__ psize, u32* __restrict__ order,
                                                 u32* __restrict__ resv, u32 P, u32 g, u32 tid) {
     __shared__ u32 sz[PT_MAX_PARTS / 8];
-    __shared__ u16 sorted[PT_MAX_PARTS / 8];
+    __shared__ u16 sorted[PT_MAX_PARTS / 8], rank_of[PT_MAX_PARTS / 8];
     __shared__ u32 s_head, s_items;
     const u32 m = P >> 3, slots = m + (m >> 3);
     for (u32 i = tid; i < m; i += PI_BLOCK) {
@@ -1010,6 +1012,7 @@ __device__ __forceinline__ void rank_partitions(const u32* __restrict__ psize, u
             rank += (o > mine || (o == mine && j < i)) ? 1u : 0u;
         }
         sorted[rank] = (u16)i;
+        rank_of[i] = (u16)rank;
     }
     __syncthreads();
     if (tid == 0) {  // the partitions that get more than one slot are the first of the ranking
@@ -1029,7 +1032,12 @@ __device__ __forceinline__ void rank_partitions(const u32* __restrict__ psize, u
     }
     __syncthreads();
     const u32 head = s_head, items = s_items;
-    for (u32 r = head + tid; r < m; r += PI_BLOCK) order[((items + r - head) << 3) | g] = g * m + sorted[r];
+    for (u32 i = tid; i < m; i += PI_BLOCK) {
+        if (rank_of[i] < head) continue;  // placed above
+        u32 before = 0;                   // partitions below i that were
+        for (u32 k = 0; k < head; ++k) before += sorted[k] < i ? 1u : 0u;
+        order[((items + i - before) << 3) | g] = g * m + i;
+    }
     for (u32 x = items + (m - head) + tid; x < slots; x += PI_BLOCK) order[(x << 3) | g] = NONE32;
 }
 
