@@ -51,6 +51,7 @@ constexpr double PART_TARGET = 1250.0, PART_TARGET_LONG_ROWS = 625.0;
 constexpr u32 PA_ACC_DOUBLES = PA_HT / 2;     // the room of the partition's hash table (16 KiB)
 constexpr u32 AUX_NEW = 0x80000000u;     // in a distinct key's aux word: the key claimed a slot in this launch
 constexpr u32 AUX_SINGLE = 0x40000000u;  // the key has one entry (low 16 bits: where its reference lies)
+constexpr u32 ROW_WALK = 0xFFFFFFFDu;    // in a distinct key's row word: still to be looked up by the walk
 constexpr u32 AUX_MULTI_MASK = 0x3FFFu;  // bits 16..29 of a key with several entries: its list number
 
 // exclusive scan over the NT threads of the block (64-bit packed fields); all threads call it
@@ -563,6 +564,8 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
     const u32 tid = threadIdx.x, lane = tid & 63u;
     const u32 units = a.units;
 
+    u32& s_nwalk = reinterpret_cast<u32*>(lds + PA_OFF_MISC)[5];  // keys that take the walk
+    if (tid == 0) s_nwalk = 0;
 #pragma unroll
     for (u32 x = 0; x < PA_HT / PA_BLOCK; ++x) owner[x * PA_BLOCK + tid] = NONE32;
     __syncthreads();
@@ -702,34 +705,53 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
             const u32 srcl = grp * 4 + (m4 ? (u32)__ffs((int)m4) - 1u : 0u);
             const u32 hrow = __shfl(wave_looks ? sv[k].z : 0u, (int)srcl);
             // found at home: done. Absent for sure (an empty slot at home) and nothing to insert: done.
+            // Everything else -- a key that is not in its home bucket, a key to insert -- takes the
+            // ordinary walk, and not here: such keys are few per wavefront, and a walk (or a claim,
+            // a round trip of an atomic) at this point would hold up sixteen keys for one. They are
+            // marked, and collected below.
             const bool slow = look && (!home || (!m4 && (a.insert || !e4)));
-            if (look && sub == 0 && !slow) urow[uu[k]] = (m4 && hrow < t.max_rows) ? hrow : ROW_NONE;
-            if (__ballot(slow)) {
-                u32 row = ROW_NONE, slot = SLOT_NONE;
-                bool won = false;
-                if (a.insert) {
-                    const Located l = find_or_claim(t, kk[k], slow, grp, sub, true);
-                    row = l.row;
-                    slot = l.slot;
-                    won = l.won;
-                } else {
-                    const Found f = probe_find(t, kk[k], slow, grp, sub);
-                    row = f.row;
-                }
-                if (slow && sub == 0) {
-                    if (won) {
-                        const u32 kn = atomicAdd(s_nnew, 1u);
-                        a.new_slot[s + kn] = slot;
-                        urow[uu[k]] = kn;
-                        aux[ii[k]] |= AUX_NEW;
-                    } else {
-                        urow[uu[k]] = row < t.max_rows ? row : ROW_NONE;
-                    }
-                }
-            }
+            if (look && sub == 0) urow[uu[k]] = slow ? ROW_WALK : (m4 && hrow < t.max_rows) ? hrow : ROW_NONE;
         }
     }
     __syncthreads();
+    // The marked keys, packed (the handles have been read: the queue takes their room), one per
+    // lane group and all lane groups at once.
+    {
+        u16* queue = reinterpret_cast<u16*>(lds + PA_OFF_HDL);
+        for (u32 u = tid; u < U; u += PA_BLOCK)
+            if (urow[u] == ROW_WALK) queue[atomicAdd(&s_nwalk, 1u)] = (u16)u;
+        __syncthreads();
+        const u32 n_walk = s_nwalk;  // block-uniform
+        for (u32 q0 = 0; q0 < n_walk; q0 += QUADS) {
+            const u32 q = q0 + (tid >> 2);
+            const bool on_q = q < n_walk;
+            const u32 u = on_q ? (u32)queue[q] : 0u;
+            const u32 i = urep[u];
+            const u64 key = on_q ? lkey[i] : KEY_EMPTY;
+            u32 row = ROW_NONE, slot = SLOT_NONE;
+            bool won = false;
+            if (a.insert) {
+                const Located l = find_or_claim(t, key, on_q, grp, sub, true);
+                row = l.row;
+                slot = l.slot;
+                won = l.won;
+            } else {
+                const Found f = probe_find(t, key, on_q, grp, sub);
+                row = f.row;
+            }
+            if (on_q && sub == 0) {
+                if (won) {
+                    const u32 kn = atomicAdd(s_nnew, 1u);
+                    a.new_slot[s + kn] = slot;
+                    urow[u] = kn;
+                    aux[i] |= AUX_NEW;
+                } else {
+                    urow[u] = row < t.max_rows ? row : ROW_NONE;
+                }
+            }
+        }
+        if (n_walk) __syncthreads();
+    }
 
     auto apply = [&](u32 u, u32 i, T gv) {
         if (aux[i] & AUX_NEW) {
@@ -1047,16 +1069,19 @@ __global__ __launch_bounds__(PI_BLOCK) void part_insert_kernel(TableDev t, const
                                                                 const u32* __restrict__ new_count,
                                                                 const u32* __restrict__ pstart, u32 P, u32 units,
                                                                 const u32* __restrict__ psize, u32* __restrict__ order,
-                                                                u32* __restrict__ resv, u32 n_parts) {
+                                                                u32* __restrict__ resv, u32 n_parts, u32 n_rankers) {
     // P: workgroups the apply kernel had (one per partition, or the slots of its order); each left
     // its new keys parked at pstart[its number], new_count of them. n_parts: partitions.
     constexpr u32 N = sizeof(T) / 4;
     __shared__ u32 red[PI_BLOCK / 64];
-    const u32 p = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
-    if (p >= P) {  // eight more workgroups, when an order is wanted: one per run of n_parts / 8 partitions
-        rank_partitions(psize, order, resv, n_parts, p - P, tid);
+    const u32 tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    // eight more workgroups when an order is wanted, one per run of n_parts / 8 partitions: the first
+    // of the grid, because theirs is the longest job of the launch
+    if (blockIdx.x < n_rankers) {
+        rank_partitions(psize, order, resv, n_parts, blockIdx.x, tid);
         return;
     }
+    const u32 p = blockIdx.x - n_rankers;
     if (!t.counters[CNT_ANY_NEW]) {  // block-uniform: the batch inserted nothing
         if (p == 0 && tid == 0) publish_rows(t, t.counters[CNT_ENTRY]);
         return;
@@ -1223,10 +1248,10 @@ hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartB
     if ((t.dim % 4 == 0) && aligned16(grads))
         part_insert_kernel<float4><<<grid, PI_BLOCK, 0, s>>>(t, b.new_slot, reinterpret_cast<const float4*>(b.ngrad),
                                                              b.new_count, b.pstart, units, t.dim / 4, b.psize, b.order,
-                                                             b.resv, pl.P);
+                                                             b.resv, pl.P, make_order ? 8u : 0u);
     else
         part_insert_kernel<float><<<grid, PI_BLOCK, 0, s>>>(t, b.new_slot, b.ngrad, b.new_count, b.pstart, units,
-                                                            t.dim, b.psize, b.order, b.resv, pl.P);
+                                                            t.dim, b.psize, b.order, b.resv, pl.P, make_order ? 8u : 0u);
     return hipGetLastError();
 }
 
