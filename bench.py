@@ -57,18 +57,18 @@ KERNEL_OF_PHASE = {"pull": "pull_kernel", "locate": "locate_kernel", "sort_hist"
 TRAFFIC_FROM_PROFILES = {
     # (config, phase): (bytes, summary)
     ("c1", "pull"): (19226624, "profiles/c1_pull_trace_and_hbm_counters.md"),
-    ("c2", "pull"): (196080640, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
-    ("c2", "part_tile"): (78080000, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
-    ("c2", "part_apply"): (146957312, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
-    ("c3", "pull"): (703201280, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c3", "part_tile"): (450787328, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c3", "part_apply"): (379213824, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "pull"): (558399488, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "part_tile"): (232773632, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c4", "part_apply"): (777693184, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
-    ("c5", "pull"): (3204252672, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
-    ("c5", "part_tile"): (1380334592, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
-    ("c5", "part_apply"): (2990774272, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "pull"): (196078592, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "part_tile"): (78201856, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c2", "part_apply"): (146975744, "profiles/c2_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "pull"): (703205376, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "part_tile"): (450809856, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c3", "part_apply"): (367959040, "profiles/c3_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "pull"): (558414848, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_tile"): (234421248, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c4", "part_apply"): (640694272, "profiles/c4_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "pull"): (3204195328, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "part_tile"): (1380374528, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
+    ("c5", "part_apply"): (2679222272, "profiles/c5_pull_push_trace_and_hbm_counters.md"),
 }
 
 
