@@ -404,6 +404,7 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
         ST_TRY(ensure(t, t->pt_order, z.order));
         ST_TRY(ensure(t, t->pt_resv, z.resv));
         HIP_TRY(t, hipMemset(t->pt_resv.p, 0, t->pt_resv.bytes));
+        HIP_TRY(t, hipMemset(t->pt_order.p, 0, t->pt_order.bytes));  // (an order of no plan)
         t->order_P = 0;
         t->part_keys = pk;
     }

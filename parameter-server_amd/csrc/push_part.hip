@@ -795,6 +795,7 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
 // loads are issued before anything waits. Returns {entries of the partition, entries in lower
 // partitions}. All threads call it.
 constexpr u32 PA_TILES_MAX = 2 * PA_BLOCK;
+constexpr u32 ORDER_TAG = PT_MAX_PARTS + PT_MAX_PARTS / 8;  // where the order names its plan: {partitions, bucket mask}
 constexpr u32 PA_STACK = 72;  // classes that can wait at once: one per bit of the second hash, and a few
 static_assert(PA_CAP + PA_STACK * 12 <= PA_CAP * 2, "the stack fits the upper half of mrep");
 
@@ -943,8 +944,11 @@ __global__ __launch_bounds__(PA_BLOCK, 4) void part_apply_kernel(TableDev t, con
     // A work item names a partition and, for one that the last push found crowded, one of the
     // 2, 4 or 8 classes of its keys (by the low bits of the second hash): that many workgroups
     // share it from the start instead of one taking its passes one after the other.
+    // The order names the plan it was made for in the two words behind its slots: one left by a
+    // push with another plan (a launch recorded earlier and replayed, say) is not followed.
     const u32 unit = blockIdx.x;
-    const u32 item = a.order ? a.order[unit] : (unit & 7u) * (a.P >> 3) + (unit >> 3);
+    const bool ordered = a.order && a.order[ORDER_TAG] == a.P && a.order[ORDER_TAG + 1] == t.bucket_mask;
+    const u32 item = ordered ? a.order[unit] : unit < a.P ? (unit & 7u) * (a.P >> 3) + (unit >> 3) : NONE32;
     if (item == NONE32) {  // (block-uniform) a spare slot of the order
         if (tid == 0) a.new_count[unit] = 0;
         return;
@@ -1016,7 +1020,7 @@ constexpr u32 PART_SHARE = 1300;                        // entries a workgroup o
 __host__ __device__ inline u32 part_units(u32 P, bool ordered) { return ordered ? P + P / 8 : P; }
 
 __device__ __forceinline__ void rank_partitions(const u32* __restrict__ psize, u32* __restrict__ order,
-                                                u32* __restrict__ resv, u32 P, u32 g, u32 tid) {
+                                                u32* __restrict__ resv, u32 P, u32 bucket_mask, u32 g, u32 tid) {
     __shared__ u32 sz[PT_MAX_PARTS / 8];
     __shared__ u16 sorted[PT_MAX_PARTS / 8], rank_of[PT_MAX_PARTS / 8];
     __shared__ u32 s_head, s_items;
@@ -1024,6 +1028,10 @@ __device__ __forceinline__ void rank_partitions(const u32* __restrict__ psize, u
     for (u32 i = tid; i < m; i += PI_BLOCK) {
         sz[i] = psize[g * m + i];
         resv[g * m + i] = 0;
+    }
+    if (g == 0 && tid == 0) {
+        order[ORDER_TAG] = P;
+        order[ORDER_TAG + 1] = bucket_mask;
     }
     __syncthreads();
     for (u32 i = tid; i < m; i += PI_BLOCK) {
@@ -1078,7 +1086,7 @@ __global__ __launch_bounds__(PI_BLOCK) void part_insert_kernel(TableDev t, const
     // eight more workgroups when an order is wanted, one per run of n_parts / 8 partitions: the first
     // of the grid, because theirs is the longest job of the launch
     if (blockIdx.x < n_rankers) {
-        rank_partitions(psize, order, resv, n_parts, blockIdx.x, tid);
+        rank_partitions(psize, order, resv, n_parts, t.bucket_mask, blockIdx.x, tid);
         return;
     }
     const u32 p = blockIdx.x - n_rankers;
@@ -1193,7 +1201,7 @@ PartSizes part_sizes(uint32_t dim, size_t n) {
     z.new_count = part_units(PT_MAX_PARTS, true) * 4;
     z.ngrad = np * (size_t)dim * 4;
     z.psize = PT_MAX_PARTS * 4;
-    z.order = part_units(PT_MAX_PARTS, true) * 4;
+    z.order = (part_units(PT_MAX_PARTS, true) + 2) * 4;  // slots, then {partitions, bucket mask} of its plan
     z.resv = PT_MAX_PARTS * 4;
     return z;
 }
