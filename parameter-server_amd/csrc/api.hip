@@ -401,11 +401,16 @@ int32_t ensure_workspace(pshbm_table* t, size_t n) {
         ST_TRY(ensure(t, t->pt_new_count, z.new_count));
         ST_TRY(ensure(t, t->pt_ngrad, z.ngrad));
         ST_TRY(ensure(t, t->pt_psize, z.psize));
+        // (of fixed size: allocated by the first batch that qualifies, and cleared then only -- later
+        // calls leave them to the kernels that may still be using them)
+        const void *order_was = t->pt_order.p, *resv_was = t->pt_resv.p;
         ST_TRY(ensure(t, t->pt_order, z.order));
         ST_TRY(ensure(t, t->pt_resv, z.resv));
-        HIP_TRY(t, hipMemset(t->pt_resv.p, 0, t->pt_resv.bytes));
-        HIP_TRY(t, hipMemset(t->pt_order.p, 0, t->pt_order.bytes));  // (an order of no plan)
-        t->order_P = 0;
+        if (t->pt_order.p != order_was) {
+            HIP_TRY(t, hipMemset(t->pt_order.p, 0, t->pt_order.bytes));  // (an order of no plan)
+            t->order_P = 0;
+        }
+        if (t->pt_resv.p != resv_was) HIP_TRY(t, hipMemset(t->pt_resv.p, 0, t->pt_resv.bytes));
         t->part_keys = pk;
     }
     t->ws_cap = cap;
