@@ -191,6 +191,32 @@ def test_hot_keys_that_agree_in_partition_and_class_bits(ps, orc, wl):
     t.close()
 
 
+def test_batches_of_changing_size_follow_and_drop_the_order(ps, orc, wl):
+    """Pushes of 0.3M to 2.9M keys in turn, so that the number of partitions changes from push to
+    push: the order a push leaves (fullest partitions first, crowded ones shared) is followed by the
+    next push with the same cut and by no other. Integer gradients: bit for bit against the oracle,
+    new keys in every batch, the last push without inserts."""
+    rng = np.random.default_rng(77)
+    n_table, dim = 120_000, 4
+    sizes = [1_400_000, 1_400_000, 300_000, 2_900_000, 1_400_000, 700_000, 2_900_000, 2_900_000]
+    cap = n_table + sum(sizes) // 50 + max(sizes) + 1000
+    t = ps.Table(dim, capacity=cap, max_batch=max(sizes), **OPTS["sgd"])
+    r = orc.Oracle(dim, capacity=cap, **OPTS["sgd"])
+    fill(t, r, wl, rng, n_table, "sgd", dim, seed=12)
+    for step, n in enumerate(sizes):
+        q = wl.zipf_batch_np(rng, n_table, 1.15, n, seed=12)
+        nf = n // 100
+        q[rng.choice(n, nf, replace=False)] = wl.fresh_keys_np(rng, nf)
+        g = rng.integers(-3, 4, (n, dim)).astype(np.float32)
+        flags = ps.PUSH_NO_INSERT if step == len(sizes) - 1 else 0
+        assert t.push(q, g, flags) == 0, t.last_error()
+        assert r.push(q, g, flags) == 0
+        assert t.size() == r.size()
+        if step % 2 == 1 or step == len(sizes) - 1:
+            same(t, r, exact=True)
+    t.close()
+
+
 def test_track_increment_through_the_partitioned_push(ps, orc, wl):
     rng = np.random.default_rng(13)
     n_table, n, dim = 30000, 20000, 4
