@@ -680,13 +680,14 @@ def test_reserve_grows_a_full_table(ps, orc, wl, opt, dim):
 
 
 @pytest.mark.parametrize("dim", [1, 4, 16, 100, 260])
-@pytest.mark.parametrize("n", [1, 33, 257, 500, 512, 1000])
+@pytest.mark.parametrize("n", [1, 33, 257, 500, 512, 513, 1000, 4096, 4097, 8193])
 def test_one_launch_push_heavy_repeats(ps, orc, dim, n):
-    """Batches of up to 512 keys take the one-launch push: a few keys repeated hundreds of times
-    (runs added by the whole workgroup), keys that are new and repeated inside the batch, keys not
-    stored under PUSH_NO_INSERT; integer gradients, so the sums are exact in any order."""
+    """Batches of up to 512 keys take the one-launch push, larger ones the partitioned push (one
+    tile up to 4096 keys, then two, then three): a few keys repeated hundreds of times (runs added by
+    the whole workgroup), keys that are new and repeated inside the batch, keys not stored under
+    PUSH_NO_INSERT; integer gradients, so the sums are exact in any order."""
     rng = np.random.default_rng(dim * 1000 + n)
-    t, r = pair(ps, orc, dim, "sum", capacity=5000)
+    t, r = pair(ps, orc, dim, "sum", capacity=5000 + 4 * n)
     base = np.arange(1, 41, dtype=np.uint64) * 7919
     assert t.set(base[:20], np.ones((20, dim), np.float32)) == 0
     assert r.set(base[:20], np.ones((20, dim), np.float32)) == 0
