@@ -472,6 +472,14 @@ int32_t pshbm_debug_part_min_keys(uint64_t keys);
 int32_t pshbm_debug_sort_pairs(int32_t device, uint32_t* d_keys, uint32_t* d_vals, uint32_t* d_keys_tmp,
                                uint32_t* d_vals_tmp, size_t n, uint32_t key_bits, int32_t* result_in_tmp,
                                void* stream);
+/* Test hook, no counterpart in the reference: the work items that the table's last inserting push of
+ * 1024 partitions or more left for the apply kernel of the next push with the same cut (fullest
+ * partitions first, crowded ones shared by several workgroups). items[0 .. *n_items) receive them
+ * in workgroup order, 0xFFFFFFFF for a spare slot, else partition | log2(workgroups that share it)
+ * << 16 | class of keys << 20; *partitions is the cut they are for (0: no such push yet, *n_items =
+ * 0). `capacity` words must hold them (4608 always do). Synchronises with the table's work. */
+int32_t pshbm_debug_part_order(pshbm_table* t, uint32_t* items, size_t capacity, size_t* n_items,
+                               uint32_t* partitions);
 /* Test hook, no counterpart in the reference: how many markers of erased keys a hash array of
  * `slots` slots under a table of at most `max_rows` keys may hold before an erase rebuilds it (an
  * eighth of the slots, less where a full table plus the markers would pass 95 % of the slots). Pure

@@ -36,7 +36,7 @@ SYMBOLS = [
     "pshbm_clear", "pshbm_size", "pshbm_memory_usage", "pshbm_get_stats",
     "pshbm_host_alloc", "pshbm_host_free", "pshbm_profile_enable", "pshbm_profile_read",
     "pshbm_push_dev_noalloc", "pshbm_pull_dev_handles", "pshbm_push_dev_handles", "pshbm_debug_sort_spin_limit", "pshbm_debug_part_pass_capacity", "pshbm_debug_part_min_keys",
-    "pshbm_debug_tombstone_limit", "pshbm_debug_sort_pairs", "pshbm_partition",
+    "pshbm_debug_tombstone_limit", "pshbm_debug_sort_pairs", "pshbm_debug_part_order", "pshbm_partition",
 ]
 PHASES = ["pull", "locate", "sort_hist", "segreduce", "fixup", "update_unique", "gather", "sort_pass",
           "fixup_windows", "assign_rows", "push_small", "part_tile", "part_apply", "part_insert"]
@@ -195,6 +195,7 @@ def lib():
         L.pshbm_partition.argtypes = [C.c_uint64, C.c_int32]
         L.pshbm_partition.restype = C.c_int32
         L.pshbm_debug_sort_pairs.argtypes = [C.c_int32, vp, vp, vp, vp, sz, u32, C.POINTER(C.c_int32), vp]
+        L.pshbm_debug_part_order.argtypes = [vp, vp, sz, C.POINTER(sz), C.POINTER(u32)]
         L.pshbm_debug_tombstone_limit.argtypes = [C.c_uint64, C.c_uint64]
         L.pshbm_debug_tombstone_limit.restype = C.c_uint64
         L.pshbm_push_pairs.argtypes = [vp, vp, sz, sz, u32]
@@ -496,6 +497,16 @@ class Table:
         n = C.c_uint64()
         lib().pshbm_memory_usage(self._h, C.byref(n))
         return n.value
+
+    def debug_part_order(self):
+        """(work items the last inserting push of 1024 partitions or more left for the next one, the
+        number of partitions they are for): pshbm_debug_part_order; (empty array, 0) before any."""
+        items = np.empty(4608, dtype=np.uint32)
+        n, parts = C.c_size_t(0), C.c_uint32(0)
+        st = lib().pshbm_debug_part_order(self._h, items.ctypes.data, items.size, C.byref(n), C.byref(parts))
+        if st != OK:
+            raise PshbmError(st, self.last_error())
+        return items[: n.value].copy(), parts.value
 
     def stats(self):
         s = Stats()

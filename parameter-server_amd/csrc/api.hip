@@ -2082,6 +2082,28 @@ int32_t pshbm_debug_part_min_keys(uint64_t keys) {
     return PSHBM_OK;
 }
 
+int32_t pshbm_debug_part_order(pshbm_table* t, uint32_t* items, size_t capacity, size_t* n_items,
+                               uint32_t* partitions) {
+    if (!t) return PSHBM_INVALID_ID;
+    if (!items || !n_items || !partitions) return fail(t, PSHBM_ERROR, "part_order: null argument");
+    DeviceGuard g(t->device);
+    std::unique_lock<std::shared_mutex> lk(t->mu);
+    *n_items = 0;
+    *partitions = 0;
+    if (!t->pt_order.p) return PSHBM_OK;
+    HIP_TRY(t, hipDeviceSynchronize());
+    uint32_t tag[2] = {0, 0};
+    const uint32_t* d_order = static_cast<const uint32_t*>(t->pt_order.p);
+    HIP_TRY(t, hipMemcpy(tag, d_order + PART_ORDER_TAG, sizeof tag, hipMemcpyDeviceToHost));
+    if (tag[0] == 0) return PSHBM_OK;
+    const size_t n = part_order_slots(tag[0]);
+    if (n > capacity) return fail(t, PSHBM_ERROR, "part_order: %zu items, room for %zu", n, capacity);
+    HIP_TRY(t, hipMemcpy(items, d_order, n * 4, hipMemcpyDeviceToHost));
+    *n_items = n;
+    *partitions = tag[0];
+    return PSHBM_OK;
+}
+
 int32_t pshbm_debug_part_pass_capacity(uint32_t entries) {
     part_set_pass_capacity(entries);
     return PSHBM_OK;

@@ -795,7 +795,8 @@ __device__ __forceinline__ void apply_pass(const TableDev& t, unsigned char* lds
 // loads are issued before anything waits. Returns {entries of the partition, entries in lower
 // partitions}. All threads call it.
 constexpr u32 PA_TILES_MAX = 2 * PA_BLOCK;
-constexpr u32 ORDER_TAG = PT_MAX_PARTS + PT_MAX_PARTS / 8;  // where the order names its plan: {partitions, bucket mask}
+constexpr u32 ORDER_TAG = PART_ORDER_TAG;  // where the order names its plan: {partitions, bucket mask}
+static_assert(PT_MAX_PARTS == PART_MAX_PARTS, "the order's layout follows the largest cut");
 constexpr u32 PA_STACK = 72;  // classes that can wait at once: one per bit of the second hash, and a few
 static_assert(PA_CAP + PA_STACK * 12 <= PA_CAP * 2, "the stack fits the upper half of mrep");
 

@@ -245,6 +245,11 @@ hipError_t launch_part_insert(const TableDev& t, const PartPlan& pl, const PartB
                               bool used_order, bool make_order, hipStream_t s);
 // Partitions from which an order pays: the apply kernel's workgroups then run in several rounds.
 constexpr uint32_t PART_ORDER_MIN = 1024;
+// Layout of PartBufs::order: the slots of a plan of P partitions (P + P / 8 of them), and at
+// PART_ORDER_TAG the two words {P, bucket mask} of the plan it was made for.
+constexpr uint32_t PART_MAX_PARTS = 4096;
+constexpr uint32_t PART_ORDER_TAG = PART_MAX_PARTS + PART_MAX_PARTS / 8;
+inline uint32_t part_order_slots(uint32_t P) { return P + P / 8; }
 // Entries a pass of the apply kernel takes (0 = the default, 2048): a test hook that makes small
 // batches go through the multi-pass path.
 void part_set_pass_capacity(uint32_t entries);

@@ -217,6 +217,48 @@ def test_batches_of_changing_size_follow_and_drop_the_order(ps, orc, wl):
     t.close()
 
 
+def test_work_items_left_for_the_next_push_cover_every_partition(ps, wl):
+    """What a push of 1024 partitions or more leaves for the next one (pshbm_debug_part_order): every
+    partition once, or 2, 4 or 8 times with one class of keys each; spare slots marked; the crowded
+    partition built here is among the shared ones. No oracle needed: an invariant of the order."""
+    rng = np.random.default_rng(31)
+    n_table, dim, tiles, tile = 60000, 4, 400, 4096
+    n = tiles * tile
+    t = ps.Table(dim, capacity=n_table + n + 1000, max_batch=n, **OPTS["sum"])
+    keys = wl.table_keys_np(0, n_table, seed=4)
+    assert t.set(keys, np.zeros((n_table, dim), np.float32)) == 0
+    items, parts = t.debug_part_order()
+    assert parts == 0 and items.size == 0
+    q = keys[rng.integers(0, n_table, (tiles, tile))]
+    with np.errstate(over="ignore"):                # six keys met in every tile, made to lie in buckets 0 .. 5:
+        hot = unmix64(((np.arange(6, dtype=np.uint64) + np.uint64(1)) << np.uint64(40)) | np.arange(6, dtype=np.uint64))
+    q[:, :6] = hot                                  # one partition holds their 2,400 entries
+    q = np.ascontiguousarray(q.reshape(-1))
+    g = np.ones((n, dim), np.float32)
+    for step in range(2):
+        assert t.push(q, g) == 0
+        items, parts = t.debug_part_order()
+        assert parts >= 1024 and items.size == parts + parts // 8
+        live = items[items != 0xFFFFFFFF]
+        p, lg, cls = live & 0xFFFF, (live >> 16) & 3, live >> 20
+        assert (p < parts).all() and (cls < (1 << lg)).all()
+        seen = {}
+        for pi, li, ci in zip(p.tolist(), lg.tolist(), cls.tolist()):
+            seen.setdefault(pi, []).append((li, ci))
+        assert sorted(seen) == list(range(parts))                       # every partition
+        assert len(seen[0]) > 1                                          # the crowded one shared
+        for pi, lst in seen.items():
+            l0 = lst[0][0]
+            assert sorted(lst) == [(l0, c) for c in range(1 << l0)]     # once, or every class once
+        # slot x belongs to run x & 7 of parts / 8 consecutive partitions
+        x = np.flatnonzero(items != 0xFFFFFFFF)
+        assert ((items[x] & 0xFFFF) // (parts // 8) == (x & 7)).all()
+    st, rows, hit = t.pull(hot)
+    times = np.array([(q == k).sum() for k in hot], dtype=np.float32)
+    assert st == 0 and hit.all() and (rows == 2 * times[:, None]).all()    # both pushes, every occurrence once
+    t.close()
+
+
 def test_track_increment_through_the_partitioned_push(ps, orc, wl):
     rng = np.random.default_rng(13)
     n_table, n, dim = 30000, 20000, 4
